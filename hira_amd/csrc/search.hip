@@ -1,0 +1,644 @@
+// Halfspace range search over the fixed-fan-out ball tree, fused with sparse attention.
+//
+// One launch covers every tree and every query head.  A wavefront owns a run of
+// consecutive level-1 nodes ("leaf parents").  For each of them it re-derives the gates of
+// the node's ancestors (levels L-1 .. 2: one row each, shared by whole subtrees and served
+// by the caches), then the node's own gate, and then scans the node's child block of keys.
+// No global frontier is exchanged between workgroups, so the walk needs no grid-wide
+// synchronisation and a pruned subtree costs its waves one or two row reads.
+//
+// Lane layout: a row of D elements is 16-byte chunks; LPR lanes hold one row (lane % LPR =
+// chunk), so a wave reads 64/LPR rows per 128-bit load instruction, fully coalesced.  The
+// G query heads that share the tree (GQA group) are scored against every chunk that is
+// loaded: one HBM read of a centroid or key row serves the whole group.
+//
+// Semantics (reference: kernels/cpp/torch_ext_v3.cpp:172-242, with the conservative
+// non-unit-query bound of searcher/cpu.py:61-63): keep a node when q.c + ||q||*r >= tau,
+// select a key when q.k >= tau.
+#include "common.hip.h"
+
+namespace hira {
+
+constexpr int kUnroll = 8;        // row loads in flight per lane while scanning a block
+constexpr int kPseudoBlock = 32;  // rows per block when there is no level-1 node (flat scan, queue)
+
+struct SearchParams {
+    // tree
+    const void* keys;
+    const void* values;
+    const int32_t* perm;
+    const void* centers[HIRA_MAX_LEVELS];
+    const float* radii[HIRA_MAX_LEVELS];
+    const int32_t* counts[HIRA_MAX_LEVELS];
+    int32_t size[HIRA_MAX_LEVELS];
+    int32_t cap[HIRA_MAX_LEVELS];
+    int32_t num_levels, bf, dim, vdim;
+    // queries
+    const void* q;
+    const float* tau;
+    const float* scaling;
+    const int32_t* tree_q_off;
+    const int32_t* tree_q_heads;
+    // queue
+    const void* queue_keys;
+    const void* queue_values;
+    int32_t queue_len, queue_cap;
+    // work split
+    int32_t nodes_per_wave;  // level-1 nodes (or pseudo blocks) per wave
+    int32_t tree_blocks;     // workgroups that walk the tree; the rest scan the queue
+    int32_t num_nodes;       // level-1 nodes (or pseudo blocks over the keys when L == 1)
+    int32_t num_queue_blocks;
+    // outputs
+    float* dense;
+    int64_t dense_stride;
+    int32_t dense_by_position;
+    int32_t* sel_index;
+    float* sel_score;
+    int32_t* sel_count;
+    int32_t sel_cap;
+    float* part_m;    // (H_q, P)
+    float* part_l;    // (H_q, P)
+    float* part_acc;  // (H_q, P, Dv)
+    int32_t num_parts;  // P = gridDim.x
+    unsigned long long* stats;
+};
+
+template <typename T, int LPR, int GMAX>
+__global__ __launch_bounds__(256) void search_kernel(const SearchParams p) {
+    constexpr int EPL = Elem<T>::kPerChunk;
+    constexpr int RPW = kWave / LPR;  // rows per wave-wide load
+    constexpr int DVP = LPR * EPL;    // widest row a lane group can hold
+
+    extern __shared__ float smem[];
+
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int nwaves = blockDim.x >> 6;
+    const int rg = lane / LPR;
+    const int ch = lane % LPR;
+    const int tree = blockIdx.y;
+    const int D = p.dim;
+    const int Dv = p.vdim;
+    const int L = p.num_levels;
+    const bool chunk_ok = ch * EPL < D;
+    const bool vchunk_ok = ch * EPL < Dv;
+    const bool want_attn = p.part_acc != nullptr;
+
+    const int hoff = p.tree_q_off[tree] + blockIdx.z * GMAX;
+    const int G = min(GMAX, p.tree_q_off[tree + 1] - hoff);
+    if (G <= 0) return;  // uniform for the workgroup
+    const unsigned gmask = (1u << G) - 1u;
+
+    // ---- queries of the group: this lane's chunk of each, plus tau, scaling, ||q|| ----
+    int qh[GMAX];
+    float qf[GMAX][EPL];
+    float tau[GMAX], sc[GMAX], qn[GMAX];
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g) {
+        qh[g] = (g < G) ? p.tree_q_heads[hoff + g] : 0;
+        uint4 raw = make_uint4(0, 0, 0, 0);
+        if (g < G && chunk_ok) raw = load_chunk<T>(p.q, (size_t)qh[g] * D, ch);
+        unpack<T>(raw, qf[g]);
+        tau[g] = (g < G) ? p.tau[qh[g]] : INFINITY;
+        sc[g] = (g < G) ? p.scaling[qh[g]] : 0.0f;
+        float ss = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) ss += qf[g][e] * qf[g][e];
+        qn[g] = sqrtf(group_sum<LPR>(ss));
+    }
+
+    // ---- attention state of this lane group -------------------------------------------
+    float acc[GMAX][EPL];
+    float mrun[GMAX], lrun[GMAX];
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g) {
+        mrun[g] = -INFINITY;
+        lrun[g] = 0.0f;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) acc[g][e] = 0.0f;
+    }
+
+    unsigned long long st_nodes[HIRA_MAX_LEVELS];
+    unsigned long long st_sel_any = 0, st_sel_pairs = 0;
+#pragma unroll
+    for (int l = 0; l < HIRA_MAX_LEVELS; ++l) st_nodes[l] = 0;
+
+    const bool is_queue = (int)blockIdx.x >= p.tree_blocks;
+    const int blk = is_queue ? (int)blockIdx.x - p.tree_blocks : (int)blockIdx.x;
+    const int n_nodes = is_queue ? p.num_queue_blocks : p.num_nodes;
+    const bool real_nodes = !is_queue && L >= 2;
+    const int node_first = (blk * nwaves + wave) * p.nodes_per_wave;
+    const int node_last = min(node_first + p.nodes_per_wave, n_nodes);
+
+    const void* kbase = is_queue ? p.queue_keys : p.keys;
+    const void* vbase = is_queue ? p.queue_values : p.values;
+    const size_t krow0 = (size_t)tree * (is_queue ? p.queue_cap : p.cap[0]);
+    const int n_rows = is_queue ? p.queue_len : p.size[0];
+    const int block_rows = real_nodes ? p.bf : kPseudoBlock;
+
+    for (int n0 = node_first; n0 < node_last; n0 += RPW) {
+        // -------- gates: lane group rg owns node n0 + rg -----------------------------
+        const int node = n0 + rg;
+        const bool node_ok = node < node_last;
+        unsigned alive = node_ok ? gmask : 0u;
+        int cnt = 0;
+        if (real_nodes) {
+            // ancestors at levels L-1 .. 2 (independent loads, issued together)
+            uint4 araw[HIRA_MAX_LEVELS - 2];
+            float arad[HIRA_MAX_LEVELS - 2];
+            int aid[HIRA_MAX_LEVELS - 2];
+            {
+                int id = node;
+#pragma unroll
+                for (int l = 2; l < HIRA_MAX_LEVELS; ++l) {
+                    id /= p.bf;
+                    aid[l - 2] = id;
+                    araw[l - 2] = make_uint4(0, 0, 0, 0);
+                    arad[l - 2] = 0.0f;
+                    if (l < L && node_ok) {
+                        const size_t r = (size_t)tree * p.cap[l] + id;
+                        if (chunk_ok) araw[l - 2] = load_chunk<T>(p.centers[l], r * D, ch);
+                        arad[l - 2] = p.radii[l][r];
+                    }
+                }
+            }
+            // top-down so that `alive` before level l says whether level l is evaluated
+#pragma unroll
+            for (int l = HIRA_MAX_LEVELS - 1; l >= 2; --l) {
+                if (l < L) {
+                    if (p.stats && alive && ch == 0) {
+                        // count the node once: by its first level-1 descendant
+                        int span = 1;
+                        for (int t = 1; t < l; ++t) span *= p.bf;
+                        if (node % span == 0) st_nodes[l]++;
+                    }
+                    float kf[EPL];
+                    unpack<T>(araw[l - 2], kf);
+                    unsigned pass = 0;
+#pragma unroll
+                    for (int g = 0; g < GMAX; ++g) {
+                        float d = 0.0f;
+#pragma unroll
+                        for (int e = 0; e < EPL; ++e) d += kf[e] * qf[g][e];
+                        d = group_sum<LPR>(d);
+                        if (d + qn[g] * arad[l - 2] >= tau[g]) pass |= 1u << g;
+                    }
+                    alive &= pass;
+                }
+            }
+            // the level-1 node itself, only if some head is still alive above it
+            if (alive) {
+                const size_t r = (size_t)tree * p.cap[1] + node;
+                uint4 raw = make_uint4(0, 0, 0, 0);
+                if (chunk_ok) raw = load_chunk<T>(p.centers[1], r * D, ch);
+                const float rad = p.radii[1][r];
+                cnt = p.counts[1][r];
+                if (p.stats && ch == 0) st_nodes[1]++;
+                float kf[EPL];
+                unpack<T>(raw, kf);
+                unsigned pass = 0;
+#pragma unroll
+                for (int g = 0; g < GMAX; ++g) {
+                    float d = 0.0f;
+#pragma unroll
+                    for (int e = 0; e < EPL; ++e) d += kf[e] * qf[g][e];
+                    d = group_sum<LPR>(d);
+                    if (d + qn[g] * rad >= tau[g]) pass |= 1u << g;
+                }
+                alive &= pass;
+            }
+        } else if (node_ok) {
+            cnt = min(kPseudoBlock, n_rows - node * kPseudoBlock);
+        }
+        if (cnt <= 0) alive = 0u;
+
+        // -------- scan the child blocks of the nodes that survived, one at a time -----
+#pragma unroll 1
+        for (int b = 0; b < RPW; ++b) {
+            const unsigned am = __shfl(alive, b * LPR, 64);  // wave-uniform
+            if (am == 0u) continue;
+            const int bcnt = __shfl(cnt, b * LPR, 64);
+            const int first = (n0 + b) * block_rows;  // first key slot of the block
+            if (p.stats && lane == 0) st_nodes[0] += (unsigned long long)bcnt;
+
+#pragma unroll 1
+            for (int i0 = 0; i0 < bcnt; i0 += RPW * kUnroll) {
+                uint4 raw[kUnroll];
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u) {
+                    const int row = i0 + u * RPW + rg;
+                    raw[u] = make_uint4(0, 0, 0, 0);
+                    if (row < bcnt && chunk_ok)
+                        raw[u] = load_chunk<T>(kbase, (krow0 + first + row) * D, ch);
+                }
+#pragma unroll
+                for (int u = 0; u < kUnroll; ++u) {
+                    const int row = i0 + u * RPW + rg;
+                    float kf[EPL];
+                    unpack<T>(raw[u], kf);
+                    float s[GMAX];
+                    unsigned sel = 0;
+#pragma unroll
+                    for (int g = 0; g < GMAX; ++g) {
+                        float d = 0.0f;
+#pragma unroll
+                        for (int e = 0; e < EPL; ++e) d += kf[e] * qf[g][e];
+                        s[g] = group_sum<LPR>(d);
+                        if (((am >> g) & 1u) && row < bcnt && (is_queue || s[g] >= tau[g]))
+                            sel |= 1u << g;
+                    }
+                    if (__ballot(sel != 0u) == 0ull) continue;  // wave-uniform
+
+                    const int slot = first + row;
+                    const bool owner = (ch == 0) && sel != 0u;
+                    if (p.stats && owner) {
+                        st_sel_any++;
+                        st_sel_pairs += (unsigned long long)__popc(sel);
+                    }
+                    if (!is_queue && (p.dense != nullptr || p.sel_count != nullptr)) {
+                        int idx = slot;
+                        if (owner && p.dense_by_position) idx = p.perm[krow0 + slot];
+#pragma unroll
+                        for (int g = 0; g < GMAX; ++g) {
+                            const bool mine = owner && ((sel >> g) & 1u);
+                            if (p.dense != nullptr && mine)
+                                p.dense[(int64_t)qh[g] * p.dense_stride + idx] = s[g] * sc[g];
+                            if (p.sel_count != nullptr) {
+                                const unsigned long long bal = __ballot(mine);
+                                if (bal != 0ull) {
+                                    int base = 0;
+                                    if (lane == 0)
+                                        base = atomicAdd(&p.sel_count[qh[g]], __popcll(bal));
+                                    base = __shfl(base, 0, 64);
+                                    const int pos =
+                                        base + __popcll(bal & ((1ull << lane) - 1ull));
+                                    if (mine && pos < p.sel_cap) {
+                                        p.sel_index[(int64_t)qh[g] * p.sel_cap + pos] = idx;
+                                        p.sel_score[(int64_t)qh[g] * p.sel_cap + pos] = s[g];
+                                    }
+                                }
+                            }
+                        }
+                    }
+                    if (want_attn && sel != 0u) {
+                        uint4 vraw = make_uint4(0, 0, 0, 0);
+                        if (vchunk_ok) vraw = load_chunk<T>(vbase, (krow0 + slot) * Dv, ch);
+                        float vf[EPL];
+                        unpack<T>(vraw, vf);
+#pragma unroll
+                        for (int g = 0; g < GMAX; ++g) {
+                            if ((sel >> g) & 1u) {
+                                const float z = s[g] * sc[g] * kLog2e;
+                                if (z > mrun[g]) {
+                                    const float f = exp2f(mrun[g] - z);
+                                    lrun[g] = lrun[g] * f + 1.0f;
+#pragma unroll
+                                    for (int e = 0; e < EPL; ++e)
+                                        acc[g][e] = acc[g][e] * f + vf[e];
+                                    mrun[g] = z;
+                                } else {
+                                    const float w = exp2f(z - mrun[g]);
+                                    lrun[g] += w;
+#pragma unroll
+                                    for (int e = 0; e < EPL; ++e) acc[g][e] += w * vf[e];
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    }
+
+    if (p.stats) {
+        unsigned long long* st = p.stats + (size_t)tree * (HIRA_MAX_LEVELS + 2);
+#pragma unroll
+        for (int l = 0; l < HIRA_MAX_LEVELS; ++l)
+            if (st_nodes[l]) atomicAdd(&st[l], st_nodes[l]);
+        if (st_sel_any) atomicAdd(&st[HIRA_MAX_LEVELS], st_sel_any);
+        if (st_sel_pairs) atomicAdd(&st[HIRA_MAX_LEVELS + 1], st_sel_pairs);
+    }
+
+    if (!want_attn) return;  // uniform
+
+    // ---- merge the lane groups of the wave, then the waves of the workgroup -----------
+    float* wsm = smem + (size_t)wave * GMAX * (DVP + 2);
+#pragma unroll
+    for (int g = 0; g < GMAX; ++g) {
+        const float mall = cross_group_max<LPR>(mrun[g]);
+        const float f = (mrun[g] == -INFINITY) ? 0.0f : exp2f(mrun[g] - mall);
+        const float lsum = cross_group_sum<LPR>(lrun[g] * f);
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) {
+            const float a = cross_group_sum<LPR>(acc[g][e] * f);
+            if (rg == 0) wsm[g * (DVP + 2) + ch * EPL + e] = a;
+        }
+        if (lane == 0) {
+            wsm[g * (DVP + 2) + DVP] = mall;
+            wsm[g * (DVP + 2) + DVP + 1] = lsum;
+        }
+    }
+    __syncthreads();
+    for (int t = threadIdx.x; t < G * Dv; t += blockDim.x) {
+        const int g = t / Dv, e = t % Dv;
+        float mall = -INFINITY;
+        for (int w = 0; w < nwaves; ++w)
+            mall = fmaxf(mall, smem[((size_t)w * GMAX + g) * (DVP + 2) + DVP]);
+        float a = 0.0f, lsum = 0.0f;
+        for (int w = 0; w < nwaves; ++w) {
+            const float* ws = smem + ((size_t)w * GMAX + g) * (DVP + 2);
+            const float mw = ws[DVP];
+            const float f = (mw == -INFINITY) ? 0.0f : exp2f(mw - mall);
+            a += ws[e] * f;
+            lsum += ws[DVP + 1] * f;
+        }
+        const int head = p.tree_q_heads[hoff + g];
+        const size_t slot = (size_t)head * p.num_parts + blockIdx.x;
+        p.part_acc[slot * Dv + e] = a;
+        if (e == 0) {
+            p.part_m[slot] = mall;
+            p.part_l[slot] = lsum;
+        }
+    }
+}
+
+// out[h] = sum_p 2^(m_p - M) acc_p / sum_p 2^(m_p - M) l_p over the P partials of head h.
+// Thread t owns a float4 of the output (t % DVL) for the partials p = t / DVL (mod NG).
+__global__ __launch_bounds__(256) void merge_kernel(const float* __restrict__ part_m,
+                                                    const float* __restrict__ part_l,
+                                                    const float* __restrict__ part_acc, int P,
+                                                    int Dv, int dvl, float* __restrict__ out) {
+    __shared__ float red[256];
+    extern __shared__ float smem[];  // (NG, Dv + 1)
+    const int t = threadIdx.x;
+    const int head = blockIdx.x;
+    const float* pm = part_m + (size_t)head * P;
+    const float* pl = part_l + (size_t)head * P;
+    const float* pa = part_acc + (size_t)head * P * Dv;
+
+    float mx = -INFINITY;
+    for (int i = t; i < P; i += 256) mx = fmaxf(mx, pm[i]);
+    mx = wave_max(mx);
+    if ((t & 63) == 0) red[t >> 6] = mx;
+    __syncthreads();
+    const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    if (M == -INFINITY) {  // nothing selected for this head
+        for (int e = t; e < Dv; e += 256) out[(size_t)head * Dv + e] = 0.0f;
+        return;
+    }
+    const int ng = 256 / dvl;
+    const int gi = t / dvl, li = t % dvl;
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+    float lsum = 0.0f;
+    const bool lane_ok = li * 4 < Dv;
+    for (int i = gi; i < P; i += ng) {
+        const float mp = pm[i];
+        if (mp == -INFINITY) continue;
+        const float w = exp2f(mp - M);
+        lsum += w * pl[i];
+        if (lane_ok) {
+            const float4 v = *reinterpret_cast<const float4*>(pa + (size_t)i * Dv + li * 4);
+            a.x += w * v.x;
+            a.y += w * v.y;
+            a.z += w * v.z;
+            a.w += w * v.w;
+        }
+    }
+    float* row = smem + (size_t)gi * (Dv + 1);
+    if (lane_ok) {
+        row[li * 4 + 0] = a.x;
+        row[li * 4 + 1] = a.y;
+        row[li * 4 + 2] = a.z;
+        row[li * 4 + 3] = a.w;
+    }
+    if (li == 0) row[Dv] = lsum;
+    __syncthreads();
+    float ltot = 0.0f;
+    for (int g = 0; g < ng; ++g) ltot += smem[(size_t)g * (Dv + 1) + Dv];
+    for (int e = t; e < Dv; e += 256) {
+        float s = 0.0f;
+        for (int g = 0; g < ng; ++g) s += smem[(size_t)g * (Dv + 1) + e];
+        out[(size_t)head * Dv + e] = s / ltot;
+    }
+}
+
+// ---- host side ------------------------------------------------------------------------
+struct SearchPlan {
+    int lpr;          // lanes per row
+    int gmax;         // heads per pass
+    int threads;      // workgroup size
+    int nodes_per_wave;
+    int num_nodes, num_queue_blocks;
+    int tree_blocks, queue_blocks, head_chunks;
+    size_t smem;
+};
+
+static int round_pow2(int v) {
+    int r = 1;
+    while (r < v) r <<= 1;
+    return r;
+}
+
+static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* queue,
+                     const HiraLaunch* launch, SearchPlan* plan) {
+    HIRA_CHECK_ARG(t && q, "tree and query must not be NULL");
+    HIRA_CHECK_ARG(t->dtype == HIRA_F32 || t->dtype == HIRA_BF16, "dtype %d", t->dtype);
+    const int esize = t->dtype == HIRA_F32 ? 4 : 2;
+    const int epl = 16 / esize;
+    HIRA_CHECK_ARG(t->num_trees >= 1, "num_trees %d", t->num_trees);
+    HIRA_CHECK_ARG(t->num_levels >= 1 && t->num_levels <= HIRA_MAX_LEVELS, "num_levels %d",
+                   t->num_levels);
+    HIRA_CHECK_ARG(t->bf >= 1 && t->bf <= 64, "branching factor %d not in 1..64", t->bf);
+    HIRA_CHECK_ARG(t->dim >= epl && t->dim % epl == 0,
+                   "dim %d: rows must be a multiple of 16 bytes", t->dim);
+    HIRA_CHECK_ARG(t->vdim >= 0 && t->vdim % epl == 0,
+                   "vdim %d: rows must be a multiple of 16 bytes", t->vdim);
+    const int widest = t->dim > t->vdim ? t->dim : t->vdim;
+    int lpr = round_pow2((widest + epl - 1) / epl);
+    if (lpr < 2) lpr = 2;
+    HIRA_CHECK_ARG(lpr <= 64, "dim %d / vdim %d too wide (max %d)", t->dim, t->vdim, 64 * epl);
+    HIRA_CHECK_ARG(t->keys != nullptr, "keys is NULL");
+    for (int l = 0; l < t->num_levels; ++l) {
+        HIRA_CHECK_ARG(t->size[l] >= 0 && t->size[l] <= t->cap[l], "size[%d]=%d cap=%d", l,
+                       t->size[l], t->cap[l]);
+        if (l >= 1) {
+            HIRA_CHECK_ARG(t->centers[l] && t->radii[l] && t->counts[l],
+                           "level %d arrays missing", l);
+            HIRA_CHECK_ARG((int64_t)t->size[l] * t->bf >= t->size[l - 1],
+                           "size[%d]=%d exceeds size[%d]*bf", l - 1, t->size[l - 1], l);
+        }
+    }
+    HIRA_CHECK_ARG(q->num_q_heads >= 1 && q->q && q->tau && q->scaling && q->tree_q_off &&
+                       q->tree_q_heads,
+                   "query arrays missing");
+    HIRA_CHECK_ARG(q->max_group >= 1, "max_group %d", q->max_group);
+    plan->lpr = lpr;
+    plan->gmax = q->max_group <= 1 ? 1 : (q->max_group <= 4 ? 4 : 8);
+    plan->head_chunks = (q->max_group + plan->gmax - 1) / plan->gmax;
+    int threads = launch && launch->block_threads ? launch->block_threads : 256;
+    HIRA_CHECK_ARG(threads == 64 || threads == 128 || threads == 256,
+                   "block_threads %d must be 64, 128 or 256", threads);
+    plan->threads = threads;
+    const int rpw = 64 / lpr;
+    int npw = launch && launch->nodes_per_wave ? launch->nodes_per_wave : rpw;
+    HIRA_CHECK_ARG(npw >= 1, "nodes_per_wave %d", npw);
+    plan->nodes_per_wave = npw;
+    plan->num_nodes = t->num_levels >= 2 ? t->size[1]
+                                         : (t->size[0] + kPseudoBlock - 1) / kPseudoBlock;
+    plan->num_queue_blocks = 0;
+    if (queue && queue->keys && queue->len > 0) {
+        HIRA_CHECK_ARG(queue->len <= queue->cap, "queue len %d > cap %d", queue->len,
+                       queue->cap);
+        plan->num_queue_blocks = (queue->len + kPseudoBlock - 1) / kPseudoBlock;
+    }
+    const int per_block = (threads / 64) * npw;
+    plan->tree_blocks = (plan->num_nodes + per_block - 1) / per_block;
+    plan->queue_blocks = (plan->num_queue_blocks + per_block - 1) / per_block;
+    plan->smem = (size_t)(threads / 64) * plan->gmax * (lpr * epl + 2) * sizeof(float);
+    return HIRA_OK;
+}
+
+template <typename T, int LPR>
+static void launch_search(const SearchPlan& plan, const SearchParams& p, dim3 grid,
+                          hipStream_t s) {
+    const size_t smem = p.part_acc ? plan.smem : 0;
+    switch (plan.gmax) {
+        case 1:
+            hipLaunchKernelGGL((search_kernel<T, LPR, 1>), grid, dim3(plan.threads), smem, s, p);
+            break;
+        case 4:
+            hipLaunchKernelGGL((search_kernel<T, LPR, 4>), grid, dim3(plan.threads), smem, s, p);
+            break;
+        default:
+            hipLaunchKernelGGL((search_kernel<T, LPR, 8>), grid, dim3(plan.threads), smem, s, p);
+            break;
+    }
+}
+
+template <typename T>
+static int dispatch_lpr(const SearchPlan& plan, const SearchParams& p, dim3 grid,
+                        hipStream_t s) {
+    switch (plan.lpr) {
+        case 2: launch_search<T, 2>(plan, p, grid, s); break;
+        case 4: launch_search<T, 4>(plan, p, grid, s); break;
+        case 8: launch_search<T, 8>(plan, p, grid, s); break;
+        case 16: launch_search<T, 16>(plan, p, grid, s); break;
+        case 32: launch_search<T, 32>(plan, p, grid, s); break;
+        case 64: launch_search<T, 64>(plan, p, grid, s); break;
+        default: return fail(HIRA_EINVAL, "unsupported row width");
+    }
+    return HIRA_OK;
+}
+
+}  // namespace hira
+
+using namespace hira;
+
+extern "C" size_t hira_search_workspace_bytes(const HiraTree* tree, const HiraQuery* query,
+                                              const HiraQueue* queue,
+                                              const HiraLaunch* launch) {
+    SearchPlan plan;
+    if (make_plan(tree, query, queue, launch, &plan) != HIRA_OK) return 0;
+    const size_t P = (size_t)plan.tree_blocks + plan.queue_blocks;
+    return (size_t)query->num_q_heads * P * (size_t)(tree->vdim + 2) * sizeof(float);
+}
+
+extern "C" int hira_search(const HiraTree* tree, const HiraQuery* query, const HiraQueue* queue,
+                           const HiraSearchOut* out, const HiraLaunch* launch, void* workspace,
+                           size_t workspace_bytes, void* stream) {
+    SearchPlan plan;
+    int rc = make_plan(tree, query, queue, launch, &plan);
+    if (rc != HIRA_OK) return rc;
+    HIRA_CHECK_ARG(out != nullptr, "out is NULL");
+    const bool attn = out->attn_out != nullptr;
+    if (attn) {
+        HIRA_CHECK_ARG(tree->values != nullptr && tree->vdim > 0,
+                       "attention needs values in the tree");
+        HIRA_CHECK_ARG(tree->vdim % 4 == 0, "vdim %d must be a multiple of 4", tree->vdim);
+        HIRA_CHECK_ARG(plan.num_queue_blocks == 0 || queue->values != nullptr,
+                       "queue values missing");
+    }
+    // by position the row length is the number of keys inserted so far, which only the
+    // caller knows; by slot it must cover every slot in use
+    if (out->dense && !out->dense_by_position)
+        HIRA_CHECK_ARG(out->dense_stride >= tree->size[0], "dense_stride %lld < %d slots",
+                       (long long)out->dense_stride, tree->size[0]);
+    if (out->dense_by_position && (out->dense || out->sel_count))
+        HIRA_CHECK_ARG(tree->perm != nullptr, "perm missing");
+    if (out->sel_count)
+        HIRA_CHECK_ARG(out->sel_index && out->sel_score && out->sel_cap > 0,
+                       "selection list arrays missing");
+
+    SearchParams p;
+    memset(&p, 0, sizeof(p));
+    p.keys = tree->keys;
+    p.values = tree->values;
+    p.perm = tree->perm;
+    for (int l = 0; l < HIRA_MAX_LEVELS; ++l) {
+        p.centers[l] = tree->centers[l];
+        p.radii[l] = tree->radii[l];
+        p.counts[l] = tree->counts[l];
+        p.size[l] = tree->size[l];
+        p.cap[l] = tree->cap[l];
+    }
+    p.num_levels = tree->num_levels;
+    p.bf = tree->bf;
+    p.dim = tree->dim;
+    p.vdim = tree->vdim;
+    p.q = query->q;
+    p.tau = query->tau;
+    p.scaling = query->scaling;
+    p.tree_q_off = query->tree_q_off;
+    p.tree_q_heads = query->tree_q_heads;
+    const bool use_queue = attn && plan.num_queue_blocks > 0;
+    if (use_queue) {
+        p.queue_keys = queue->keys;
+        p.queue_values = queue->values;
+        p.queue_len = queue->len;
+        p.queue_cap = queue->cap;
+    }
+    p.nodes_per_wave = plan.nodes_per_wave;
+    p.tree_blocks = plan.tree_blocks;
+    p.num_nodes = plan.num_nodes;
+    p.num_queue_blocks = use_queue ? plan.num_queue_blocks : 0;
+    p.dense = out->dense;
+    p.dense_stride = out->dense_stride;
+    p.dense_by_position = out->dense_by_position;
+    p.sel_index = out->sel_index;
+    p.sel_score = out->sel_score;
+    p.sel_count = out->sel_count;
+    p.sel_cap = out->sel_cap;
+    p.stats = out->stats;
+
+    const int P = plan.tree_blocks + (use_queue ? plan.queue_blocks : 0);
+    if (P == 0) return HIRA_OK;
+    p.num_parts = P;
+    if (attn) {
+        const size_t need =
+            (size_t)query->num_q_heads * P * (size_t)(tree->vdim + 2) * sizeof(float);
+        if (workspace == nullptr || workspace_bytes < need)
+            return fail(HIRA_EWORKSPACE, "workspace %zu bytes, need %zu", workspace_bytes, need);
+        float* w = reinterpret_cast<float*>(workspace);
+        p.part_acc = w;
+        p.part_m = w + (size_t)query->num_q_heads * P * tree->vdim;
+        p.part_l = p.part_m + (size_t)query->num_q_heads * P;
+    }
+
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    dim3 grid(P, tree->num_trees, plan.head_chunks);
+    rc = tree->dtype == HIRA_F32 ? dispatch_lpr<float>(plan, p, grid, s)
+                                 : dispatch_lpr<bf16_t>(plan, p, grid, s);
+    if (rc != HIRA_OK) return rc;
+    HIRA_CHECK_LAUNCH("search kernel");
+
+    if (attn) {
+        int dvl = round_pow2((tree->vdim + 3) / 4);
+        if (dvl > 256) return fail(HIRA_EINVAL, "vdim %d too wide", tree->vdim);
+        const int ng = 256 / dvl;
+        const size_t smem = (size_t)ng * (tree->vdim + 1) * sizeof(float);
+        hipLaunchKernelGGL(merge_kernel, dim3(query->num_q_heads), dim3(256), smem, s, p.part_m,
+                           p.part_l, p.part_acc, P, tree->vdim, dvl, out->attn_out);
+        HIRA_CHECK_LAUNCH("merge kernel");
+    }
+    return HIRA_OK;
+}

@@ -1,0 +1,258 @@
+"""HIPIndexer: the ball-tree index on one MI355X.
+
+Replaces the reference's GPU indexer (indexer/cuda.py:16-108, 544-701) behind the same
+surface: ``HIPIndexer(num_levels, max_iterations, branching_factor, verbose, pad_value)``,
+``build(keys (1,H,L,D), values)``, ``update(new_keys (1,H,m,D), new_values)``; the
+attributes other code reads (``children``, ``values``, ``parents``, ``parent_radii``,
+``grand_parents``, ``grand_parent_radii``, ``branching_factor``, ``depth``, ``pad_value``,
+``dim``, ``num_heads``, ``_child_counts``, ``_parent_valid``, ``_gp_child_counts``) are
+views of the level arrays.  Differences, all deliberate:
+
+* any depth (the reference GPU indexer stops at three levels, indexer/cuda.py:18-21);
+* keys stay in the model's dtype (bf16 or fp32; the reference up-casts to fp32,
+  indexer/cuda.py:365-368);
+* per-node child counts are authoritative (the reference infers validity from
+  "row is all pad_value", indexer/cuda.py:137-144);
+* ``perm`` maps a key slot to the position the key was inserted at, so results can be
+  reported in the CPU searcher's index space as well;
+* a leading batch dimension B > 1 builds B*H independent trees that one launch searches.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from enum import Enum
+from typing import List, Optional
+
+import torch
+
+from .. import _lib
+from .base import BaseIndexer
+
+DEFAULT_PAD_VALUE = 0.0
+
+_DTYPES = {torch.float32: _lib.HIRA_F32, torch.bfloat16: _lib.HIRA_BF16}
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def level_sizes(n: int, bf: int, num_levels: int) -> List[int]:
+    """Slots per level of the padded tree: K_1 = ceil(n/bf), K_l = ceil(K_{l-1}/bf); the
+    root keeps K_root nodes and each lower level has bf slots per node of the level above
+    (the reference's m = ceil(n/bf), g = ceil(m/bf), children (h, g*bf*bf, d):
+    indexer/cuda.py:223-224, 439-446)."""
+    if num_levels == 1:
+        return [n]
+    k = n
+    for _ in range(1, num_levels):
+        k = max(1, -(-k // bf))
+    sizes = [0] * num_levels
+    sizes[-1] = k
+    for l in range(num_levels - 2, -1, -1):
+        sizes[l] = sizes[l + 1] * bf
+    return sizes
+
+
+class HIPIndexer(BaseIndexer):
+    class DEPTH(Enum):
+        TWO_LEVELS = 2
+        THREE_LEVELS = 3
+
+    def __init__(
+        self,
+        num_levels,
+        max_iterations: int = 1,
+        branching_factor: int = 32,
+        verbose: bool = False,
+        pad_value: float = DEFAULT_PAD_VALUE,
+        *,
+        seed: int = 1234,
+        capacity: Optional[int] = None,
+        device: str = "cuda",
+    ):
+        if isinstance(num_levels, HIPIndexer.DEPTH):
+            num_levels = num_levels.value
+        num_levels = int(num_levels)
+        if not 1 <= num_levels <= _lib.HIRA_MAX_LEVELS:
+            raise ValueError(f"num_levels must be in 1..{_lib.HIRA_MAX_LEVELS}, got {num_levels}")
+        if not 1 <= int(branching_factor) <= 64:
+            raise ValueError(f"branching_factor must be in 1..64, got {branching_factor}")
+        self.num_levels = num_levels
+        self.max_iterations = int(max_iterations)
+        self.branching_factor = int(branching_factor)
+        self.verbose = verbose
+        self.pad_value = pad_value
+        self.seed = int(seed)
+        self.capacity = capacity  # key slots to reserve per tree (room for appends)
+        self.device = torch.device(device)
+
+        self.dim = 0
+        self.vdim = 0
+        self.batch = 1
+        self.num_heads = 0
+        self.num_trees = 0
+        self.num_keys = 0  # keys given to the index so far, per tree
+        self.dtype: Optional[torch.dtype] = None
+        self.size: List[int] = []
+        self.cap: List[int] = []
+        self.keys_buf: Optional[torch.Tensor] = None
+        self.values_buf: Optional[torch.Tensor] = None
+        self.perm: Optional[torch.Tensor] = None
+        self.centers: List[Optional[torch.Tensor]] = []
+        self.radii: List[Optional[torch.Tensor]] = []
+        self.counts: List[Optional[torch.Tensor]] = []
+        self._tree_struct = None
+
+    # ------------------------------------------------------------------ reference views
+    @property
+    def depth(self):
+        try:
+            return HIPIndexer.DEPTH(self.num_levels)
+        except ValueError:
+            return self.num_levels
+
+    def _head_view(self, t: torch.Tensor, n: int) -> torch.Tensor:
+        """(T, cap, ...) -> (H, n, ...) for batch 1, (B, H, n, ...) otherwise."""
+        v = t[:, :n]
+        return v if self.batch == 1 else v.reshape(self.batch, self.num_heads, *v.shape[1:])
+
+    @property
+    def children(self):
+        return None if self.keys_buf is None else self._head_view(self.keys_buf, self.size[0])
+
+    @property
+    def values(self):
+        if self.values_buf is None:
+            return None
+        v = self._head_view(self.values_buf, self.size[0])
+        return v.unsqueeze(0) if self.batch == 1 else v
+
+    def _level(self, arr, l):
+        if l >= self.num_levels or not arr or arr[l] is None:
+            return None
+        return self._head_view(arr[l], self.size[l])
+
+    @property
+    def parents(self):
+        return self._level(self.centers, 1)
+
+    @property
+    def parent_radii(self):
+        return self._level(self.radii, 1)
+
+    @property
+    def grand_parents(self):
+        return self._level(self.centers, 2)
+
+    @property
+    def grand_parent_radii(self):
+        return self._level(self.radii, 2)
+
+    @property
+    def _child_counts(self):
+        return self._level(self.counts, 1)
+
+    @property
+    def _parent_valid(self):
+        c = self._level(self.counts, 1)
+        return None if c is None else c > 0
+
+    @property
+    def _gp_child_counts(self):
+        return self._level(self.counts, 2)
+
+    # ------------------------------------------------------------------ device state
+    def _allocate(self, batch: int, heads: int, n: int, dim: int, vdim: int,
+                  dtype: torch.dtype) -> None:
+        if dtype not in _DTYPES:
+            raise ValueError(f"unsupported key dtype {dtype}: use float32 or bfloat16")
+        esize = 4 if dtype == torch.float32 else 2
+        if (dim * esize) % 16 or (vdim * esize) % 16:
+            raise ValueError(f"dim {dim} / vdim {vdim}: rows must be a multiple of 16 bytes")
+        self.batch, self.num_heads = batch, heads
+        self.num_trees = batch * heads
+        self.dim, self.vdim, self.dtype = dim, vdim, dtype
+        bf, nl = self.branching_factor, self.num_levels
+        self.size = level_sizes(n, bf, nl)
+        want = max(n, int(self.capacity or 0))
+        self.cap = level_sizes(want, bf, nl) if want > n else list(self.size)
+        if nl >= 2 and want > n:
+            # appended keys open new leaf blocks: leave room for one new block per key
+            extra = want - n
+            self.cap = level_sizes(n + extra * bf, bf, nl)
+        dev, t = self.device, self.num_trees
+        self.keys_buf = torch.zeros((t, self.cap[0], dim), dtype=dtype, device=dev)
+        self.values_buf = (
+            torch.zeros((t, self.cap[0], vdim), dtype=dtype, device=dev) if vdim else None)
+        self.perm = torch.full((t, self.cap[0]), -1, dtype=torch.int32, device=dev)
+        self.centers, self.radii, self.counts = [None], [None], [None]
+        for l in range(1, nl):
+            self.centers.append(torch.zeros((t, self.cap[l], dim), dtype=dtype, device=dev))
+            self.radii.append(
+                torch.full((t, self.cap[l]), float("-inf"), dtype=torch.float32, device=dev))
+            self.counts.append(torch.zeros((t, self.cap[l]), dtype=torch.int32, device=dev))
+        self._tree_struct = None
+
+    def tree_struct(self) -> _lib.HiraTree:
+        """The C view of the tree; valid while this indexer's tensors are alive."""
+        if self.keys_buf is None:
+            raise ValueError("Indexer is not built: missing children tensor.")
+        if self._tree_struct is None:
+            t = _lib.HiraTree()
+            t.num_trees = self.num_trees
+            t.num_levels = self.num_levels
+            t.bf = self.branching_factor
+            t.dim, t.vdim = self.dim, self.vdim
+            t.dtype = _DTYPES[self.dtype]
+            for l in range(self.num_levels):
+                t.size[l], t.cap[l] = self.size[l], self.cap[l]
+            t.keys = self.keys_buf.data_ptr()
+            t.values = None if self.values_buf is None else self.values_buf.data_ptr()
+            t.perm = self.perm.data_ptr()
+            for l in range(1, self.num_levels):
+                t.centers[l] = self.centers[l].data_ptr()
+                t.radii[l] = self.radii[l].data_ptr()
+                t.counts[l] = self.counts[l].data_ptr()
+            self._tree_struct = t
+        return self._tree_struct
+
+    # ------------------------------------------------------------------ layouts
+    @classmethod
+    def from_layout(cls, *, bf: int, keys, perm, centers, radii, counts, values=None,
+                    dtype: torch.dtype = torch.float32, batch: int = 1, device: str = "cuda",
+                    num_keys: Optional[int] = None, capacity: Optional[int] = None):
+        """Adopt a padded tree given as host arrays: keys (T, N_pad, D), perm (T, N_pad),
+        and per level l >= 1 (index 0 is None) centers (T, K_l, D), radii (T, K_l), counts
+        (T, K_l); values (T, N_pad, Dv) follow the key slots.  Used to restore a saved index
+        and by tests that walk a tree built on the host."""
+        nl = len(centers)
+        self = cls(nl, 1, bf, device=device, capacity=capacity)
+        keys = torch.as_tensor(keys)
+        t, n_pad, d = keys.shape
+        vdim = 0 if values is None else int(torch.as_tensor(values).shape[-1])
+        self._allocate(batch, t // batch, n_pad, d, vdim, dtype)
+        if self.size[0] != n_pad:
+            raise ValueError(f"keys have {n_pad} slots, layout needs {self.size[0]}")
+        self.keys_buf[:, :n_pad] = keys.to(device=self.device, dtype=dtype)
+        if values is not None:
+            self.values_buf[:, :n_pad] = torch.as_tensor(values).to(device=self.device,
+                                                                    dtype=dtype)
+        perm = torch.as_tensor(perm).to(torch.int32)
+        self.perm[:, :n_pad] = perm.to(self.device)
+        for l in range(1, nl):
+            k = self.size[l]
+            self.centers[l][:, :k] = torch.as_tensor(centers[l]).to(self.device, dtype)
+            self.radii[l][:, :k] = torch.as_tensor(radii[l]).to(self.device, torch.float32)
+            self.counts[l][:, :k] = torch.as_tensor(counts[l]).to(self.device, torch.int32)
+        self.num_keys = int(num_keys if num_keys is not None else (perm[0] >= 0).sum().item())
+        return self
+
+    # ------------------------------------------------------------------ build / update
+    @torch.no_grad()
+    def build(self, keys: torch.Tensor, values: Optional[torch.Tensor] = None):
+        raise NotImplementedError("HIP build is not wired yet")
+
+    @torch.no_grad()
+    def update(self, new_keys: torch.Tensor, new_values: Optional[torch.Tensor] = None):
+        raise NotImplementedError("HIP update is not wired yet")

@@ -1,0 +1,234 @@
+"""HIPSearcher: halfspace range search (and fused sparse attention) on one MI355X.
+
+Replaces the reference's GPU searcher (searcher/cuda.py:15-143) and, through
+``index_space="position"``, the CPU searcher's contract (searcher/cpu.py:44-101):
+``search(query (1,H_q,1,D), threshold (H_q,), indexer, q_head_to_kv=None, scaling=None)``
+returns an ``(H_q, N)`` fp32 tensor holding ``score * scaling`` for every key with
+``q.k >= threshold`` and ``output_fill_value`` elsewhere.
+
+Semantics follow the CPU kernels (keep a node when ``q.c + ||q|| r >= t``, a key when
+``q.k >= t``: kernels/cpp/torch_ext_v3.cpp:182, 212, 238), not the Triton kernels, which
+gate with a strict ``>`` and never filter the leaves (kernels/triton_search_kernels.py:
+49-63).  Like the reference's GPU searcher the dense result lives in a buffer this object
+keeps and reuses: clone it to hold on to a result across calls (searcher/cuda.py:35-54).
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Tuple
+
+import torch
+
+from .. import _lib
+from .base import BaseSearcher
+
+DEFAULT_OUTPUT_FILL_VALUE = 0.0
+
+
+class HIPSearcher(BaseSearcher):
+    def __init__(self, block_c=None, output_fill_value: float = DEFAULT_OUTPUT_FILL_VALUE,
+                 *, index_space: str = "slot", block_threads: int = 0, nodes_per_wave: int = 0,
+                 kernel: int = 0):
+        super().__init__()
+        if index_space not in ("slot", "position"):
+            raise ValueError("index_space must be 'slot' or 'position'")
+        self.block_c = block_c  # accepted for HiraConfig.get_searcher_kwargs(); unused
+        self.output_fill_value = float(output_fill_value)
+        self.index_space = index_space
+        self.launch = _lib.HiraLaunch(int(block_threads), int(nodes_per_wave), int(kernel))
+        self._tmp_out: Optional[torch.Tensor] = None
+        self._map_cache = {}
+        self._workspace: Optional[torch.Tensor] = None
+        self._sel = None
+
+    # -------------------------------------------------------------- input coercion
+    @staticmethod
+    def _coerce_query(query, d: int) -> torch.Tensor:
+        """(H_q, D), (1, H_q, 1, D) or, for B sequences, (B, H_q, 1, D) -> (B*H_q, D)
+        (kernels/triton_search_wrappers.py:9-27)."""
+        if not isinstance(query, torch.Tensor):
+            raise TypeError(f"q must be a torch.Tensor, got {type(query)}")
+        if query.ndim == 4:
+            if query.shape[2] != 1:
+                raise ValueError(f"4D query must be (B,H,1,D), got {tuple(query.shape)}")
+            query = query.squeeze(2).reshape(-1, query.shape[-1])
+        elif query.ndim != 2:
+            raise ValueError(f"q must be (H,d) or (1,H,1,D), got {tuple(query.shape)}")
+        if query.shape[-1] != d:
+            raise ValueError(f"query dim mismatch: expected d={d}, got {query.shape[-1]}")
+        return query
+
+    @staticmethod
+    def _coerce_threshold(t, h: int, device) -> torch.Tensor:
+        """scalar or (H_q,) (kernels/triton_search_wrappers.py:57-71)."""
+        if torch.is_tensor(t):
+            t = t.to(device=device, dtype=torch.float32).reshape(-1)
+        else:
+            t = torch.tensor([float(t)], device=device, dtype=torch.float32)
+        if t.numel() == 1 and h > 1:
+            t = t.expand(h)
+        if t.numel() != h:
+            raise ValueError(f"threshold must be scalar or length H={h}, got {t.numel()}")
+        return t.contiguous()
+
+    @staticmethod
+    def _coerce_scaling(scaling, h: int, device) -> torch.Tensor:
+        """None or (H_q,) (kernels/triton_search_wrappers.py:74-89; the finiteness check
+        there costs a host sync per call and is left to the caller)."""
+        if scaling is None:
+            return torch.ones((h,), device=device, dtype=torch.float32)
+        if not torch.is_tensor(scaling):
+            raise TypeError(f"scaling must be a torch.Tensor with shape (H,), got {type(scaling)}")
+        s = scaling.to(device=device, dtype=torch.float32).reshape(-1)
+        if s.numel() != h:
+            raise ValueError(f"scaling must have length H={h}, got {s.numel()}")
+        return s.contiguous()
+
+    def _head_map(self, h_q: int, indexer, q_head_to_kv) -> Tuple[torch.Tensor, torch.Tensor, int]:
+        """CSR of the query heads of each tree.  Default map: head h of sequence b belongs
+        to tree b*H_kv + h // (H_q/H_kv) (searcher/cuda.py:23-33)."""
+        t, batch, h_kv = indexer.num_trees, indexer.batch, indexer.num_heads
+        key = (h_q, t, batch, None if q_head_to_kv is None
+               else tuple(int(x) for x in torch.as_tensor(q_head_to_kv).reshape(-1).tolist()))
+        hit = self._map_cache.get(key)
+        if hit is not None:
+            return hit
+        if q_head_to_kv is None:
+            if h_q % batch:
+                raise ValueError(f"H_q={h_q} not divisible by batch={batch}")
+            per_seq = h_q // batch
+            if per_seq == h_kv:
+                local = torch.arange(per_seq)
+            else:
+                if per_seq % h_kv:
+                    raise ValueError(
+                        f"Unsupported head mapping: H_q={per_seq} must equal or be divisible "
+                        f"by H_kv={h_kv}")
+                local = torch.arange(per_seq) // (per_seq // h_kv)
+            m = (torch.arange(batch)[:, None] * h_kv + local[None, :]).reshape(-1)
+        else:
+            if not torch.is_tensor(q_head_to_kv):
+                raise TypeError(
+                    f"q_head_to_kv must be a torch.Tensor or None, got {type(q_head_to_kv)}")
+            m = q_head_to_kv.detach().to("cpu", torch.long).reshape(-1)
+            if m.numel() != h_q:
+                raise ValueError(f"q_head_to_kv length mismatch: expected H_q={h_q}, got {m.numel()}")
+            if bool(((m < 0) | (m >= t)).any()):
+                raise ValueError(f"q_head_to_kv values must be in [0, {t - 1}]")
+        order = torch.argsort(m, stable=True)
+        counts = torch.bincount(m, minlength=t)
+        off = torch.zeros(t + 1, dtype=torch.int32)
+        off[1:] = counts.cumsum(0).to(torch.int32)
+        dev = indexer.device
+        val = (off.to(dev), order.to(torch.int32).to(dev), int(counts.max().item()))
+        self._map_cache = {key: val}
+        return val
+
+    def _query_struct(self, query, threshold, indexer, q_head_to_kv, scaling):
+        dev = indexer.device
+        q = self._coerce_query(query, indexer.dim).to(device=dev, dtype=indexer.dtype).contiguous()
+        h_q = q.shape[0]
+        tau = self._coerce_threshold(threshold, h_q, dev)
+        sc = self._coerce_scaling(scaling, h_q, dev)
+        off, heads, gmax = self._head_map(h_q, indexer, q_head_to_kv)
+        qs = _lib.HiraQuery(h_q, q.data_ptr(), tau.data_ptr(), sc.data_ptr(), off.data_ptr(),
+                            heads.data_ptr(), gmax)
+        return qs, (q, tau, sc, off, heads)
+
+    def _get_workspace(self, nbytes: int, device) -> torch.Tensor:
+        if self._workspace is None or self._workspace.numel() < nbytes or \
+                self._workspace.device != device:
+            self._workspace = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
+        return self._workspace
+
+    def _prepare_output_buffer(self, h_q: int, n: int, device) -> torch.Tensor:
+        """searcher/cuda.py:35-54."""
+        if self._tmp_out is None or self._tmp_out.device != device or \
+                tuple(self._tmp_out.shape) != (h_q, n):
+            self._tmp_out = torch.full((h_q, n), self.output_fill_value, device=device,
+                                       dtype=torch.float32)
+        else:
+            self._tmp_out.fill_(self.output_fill_value)
+        return self._tmp_out
+
+    def _run(self, indexer, qs, out: _lib.HiraSearchOut, queue: Optional[_lib.HiraQueue]):
+        lib = _lib.lib()
+        tree = indexer.tree_struct()
+        ws_ptr, ws_bytes, ws = None, 0, None
+        if out.attn_out:
+            ws_bytes = lib.hira_search_workspace_bytes(
+                C.byref(tree), C.byref(qs), C.byref(queue) if queue else None,
+                C.byref(self.launch))
+            ws = self._get_workspace(ws_bytes, indexer.device)
+            ws_ptr = ws.data_ptr()
+        stream = torch.cuda.current_stream(indexer.device).cuda_stream
+        rc = lib.hira_search(C.byref(tree), C.byref(qs), C.byref(queue) if queue else None,
+                             C.byref(out), C.byref(self.launch), ws_ptr, ws_bytes, stream)
+        _lib.check(rc)
+
+    # -------------------------------------------------------------- public API
+    def search(self, query, threshold, indexer, q_head_to_kv: Optional[torch.Tensor] = None,
+               scaling: Optional[torch.Tensor] = None, *, index_space: Optional[str] = None,
+               stats: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if indexer.keys_buf is None:
+            raise ValueError("Indexer is not built: missing children tensor.")
+        space = index_space or self.index_space
+        qs, keep = self._query_struct(query, threshold, indexer, q_head_to_kv, scaling)
+        n = indexer.size[0] if space == "slot" else indexer.num_keys
+        dense = self._prepare_output_buffer(qs.num_q_heads, n, indexer.device)
+        out = _lib.HiraSearchOut()
+        out.dense = dense.data_ptr()
+        out.dense_stride = dense.stride(0)
+        out.dense_by_position = 1 if space == "position" else 0
+        out.stats = None if stats is None else stats.data_ptr()
+        self._run(indexer, qs, out, None)
+        del keep
+        return dense
+
+    def search_compact(self, query, threshold, indexer, q_head_to_kv=None, scaling=None, *,
+                       capacity: Optional[int] = None, index_space: Optional[str] = None):
+        """Compact result: (index (H_q, cap) int32, score (H_q, cap) fp32 raw q.k,
+        count (H_q,) int32); entries of a head are unordered."""
+        space = index_space or self.index_space
+        qs, keep = self._query_struct(query, threshold, indexer, q_head_to_kv, scaling)
+        cap = int(capacity or indexer.size[0])
+        h_q, dev = qs.num_q_heads, indexer.device
+        if self._sel is None or self._sel[0].shape != (h_q, cap) or self._sel[0].device != dev:
+            self._sel = (torch.empty((h_q, cap), dtype=torch.int32, device=dev),
+                         torch.empty((h_q, cap), dtype=torch.float32, device=dev),
+                         torch.zeros((h_q,), dtype=torch.int32, device=dev))
+        idx, score, count = self._sel
+        count.zero_()
+        out = _lib.HiraSearchOut()
+        out.dense_by_position = 1 if space == "position" else 0
+        out.sel_index, out.sel_score, out.sel_count = idx.data_ptr(), score.data_ptr(), count.data_ptr()
+        out.sel_cap = cap
+        self._run(indexer, qs, out, None)
+        del keep
+        return idx, score, count
+
+    def search_attention(self, query, threshold, indexer, q_head_to_kv=None, scaling=None, *,
+                         queue_keys: Optional[torch.Tensor] = None,
+                         queue_values: Optional[torch.Tensor] = None,
+                         out: Optional[torch.Tensor] = None,
+                         stats: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Fused search + softmax(scaling * q.K_S^T) V_S over the selected keys and, when
+        given, every queued key (T, m, D) / value (T, m, Dv).  Returns (H_q, Dv) fp32."""
+        qs, keep = self._query_struct(query, threshold, indexer, q_head_to_kv, scaling)
+        h_q, dev = qs.num_q_heads, indexer.device
+        if out is None:
+            out = torch.empty((h_q, indexer.vdim), dtype=torch.float32, device=dev)
+        so = _lib.HiraSearchOut()
+        so.attn_out = out.data_ptr()
+        so.stats = None if stats is None else stats.data_ptr()
+        queue = None
+        if queue_keys is not None and queue_keys.shape[-2] > 0:
+            qk = queue_keys.reshape(indexer.num_trees, -1, indexer.dim)
+            qv = queue_values.reshape(indexer.num_trees, -1, indexer.vdim)
+            qk = qk.to(device=dev, dtype=indexer.dtype).contiguous()
+            qv = qv.to(device=dev, dtype=indexer.dtype).contiguous()
+            queue = _lib.HiraQueue(qk.data_ptr(), qv.data_ptr(), qk.shape[1], qk.shape[1])
+            keep = keep + (qk, qv)
+        self._run(indexer, qs, so, queue)
+        del keep
+        return out

@@ -1,0 +1,144 @@
+/*
+ * hira_hip.h -- C ABI of libhira_hip.so: the MI355X (gfx950) range-search sparse-attention
+ * hot path: ball-tree index build / append, halfspace tree search, sparse attention.
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer unless its name ends in _host.  The caller owns
+ *     all memory; the library allocates nothing and keeps no state between calls
+ *     (except the thread-local text returned by hira_last_error).
+ *   - Every call only ENQUEUES work on `stream` (a hipStream_t passed as void*) and
+ *     returns; calls that touch the same tree must be ordered by the caller (same stream).
+ *   - Return value: 0 on success, a negative HIRA_E* code otherwise.
+ *   - dtype: HIRA_F32 or HIRA_BF16; it is the storage type of keys, values, centers and
+ *     queries.  All arithmetic accumulates in fp32.
+ *
+ * Tree layout (depth-generic, fixed fan-out; the layout of the reference's GPU indexer,
+ * indexer/cuda.py:338-357, 439-446, generalised to any depth and to many trees):
+ *   level 0 = keys; level l >= 1 = ball centers + radii.  The children of node p of
+ *   level l+1 are the slots [p*bf, (p+1)*bf) of level l, filled from slot 0;
+ *   counts[l+1][p] says how many are in use.  size[l] = slots of level l that may be in
+ *   use (size[l] <= size[l+1]*bf), cap[l] = allocated slots per tree (row stride between
+ *   trees).  A node without children has radius -inf.  perm maps a key slot to the
+ *   position of that key in the order it was given to the index (-1 for an empty slot).
+ */
+#ifndef HIRA_HIP_H
+#define HIRA_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HIRA_ABI_VERSION 1
+#define HIRA_MAX_LEVELS 8
+
+enum { HIRA_F32 = 0, HIRA_BF16 = 1 };
+
+enum {
+    HIRA_OK = 0,
+    HIRA_EINVAL = -1,   /* bad shape / dtype / null pointer: the message names it */
+    HIRA_ELAUNCH = -2,  /* the HIP runtime refused a launch */
+    HIRA_EWORKSPACE = -3 /* workspace too small */
+};
+
+typedef struct HiraTree {
+    int32_t num_trees;  /* T = sequences x KV heads; one independent tree each */
+    int32_t num_levels; /* L >= 1 (L = 1: keys only, every search is a flat scan) */
+    int32_t bf;         /* fan-out, 1..64 */
+    int32_t dim;        /* key / query / center dim D; D*elem_size a multiple of 16 B */
+    int32_t vdim;       /* value dim Dv (0 if there are no values) */
+    int32_t dtype;
+    int32_t size[HIRA_MAX_LEVELS];
+    int32_t cap[HIRA_MAX_LEVELS];
+    void* keys;                      /* (T, cap[0], D) */
+    void* values;                    /* (T, cap[0], Dv) or NULL */
+    int32_t* perm;                   /* (T, cap[0]) */
+    void* centers[HIRA_MAX_LEVELS];  /* [l >= 1] (T, cap[l], D) */
+    float* radii[HIRA_MAX_LEVELS];   /* [l >= 1] (T, cap[l]) */
+    int32_t* counts[HIRA_MAX_LEVELS];/* [l >= 1] (T, cap[l]) */
+} HiraTree;
+
+/* One decode step's queries.  Query head h belongs to tree q2tree order given as CSR:
+ * the heads of tree t are tree_q_heads[tree_q_off[t] .. tree_q_off[t+1]).  This carries
+ * the reference's q_head_to_kv map (searcher/cpu.py:103-109, searcher/cuda.py:23-33),
+ * including maps that are not monotone (tests/test_cpp_kernels.py:529-565). */
+typedef struct HiraQuery {
+    int32_t num_q_heads;         /* H_q (all sequences) */
+    const void* q;               /* (H_q, D), tree dtype */
+    const float* tau;            /* (H_q) threshold on the raw score q.k */
+    const float* scaling;        /* (H_q) factor applied to returned scores / softmax logits */
+    const int32_t* tree_q_off;   /* (T+1) */
+    const int32_t* tree_q_heads; /* (H_q) */
+    int32_t max_group;           /* max heads of one tree (host knows it) */
+} HiraQuery;
+
+/* Keys/values that are cached but not yet in the index (the reference's decode queue,
+ * cache/hira_cache.py:121-140): attention always attends to all of them. */
+typedef struct HiraQueue {
+    const void* keys;   /* (T, cap, D) or NULL */
+    const void* values; /* (T, cap, Dv) */
+    int32_t len;        /* rows in use per tree */
+    int32_t cap;
+} HiraQueue;
+
+/* What a search writes.  Any of the three groups may be absent (NULL pointers). */
+typedef struct HiraSearchOut {
+    /* (1) dense scores, the reference's return value (searcher/cpu.py:44-101,
+     *     searcher/cuda.py:56-143): dense[h*dense_stride + i] = (q_h.k_i)*scaling[h] for
+     *     every selected key, untouched elsewhere (caller pre-fills).  dense_by_position
+     *     != 0: i = position of the key in insertion order (CPU searcher's index space);
+     *     0: i = key slot (GPU searcher's index space). */
+    float* dense;
+    int64_t dense_stride;
+    int32_t dense_by_position;
+    /* (2) compact lists: for head h, sel_count[h] entries (unordered) of
+     *     sel_index[h*sel_cap + j] (slot or position, as above) and sel_score (raw q.k).
+     *     sel_count must be zeroed by the caller; entries beyond sel_cap are counted but
+     *     not stored. */
+    int32_t* sel_index;
+    float* sel_score;
+    int32_t* sel_count;
+    int32_t sel_cap;
+    /* (3) attention over the selected keys (+ the queue): out (H_q, Dv) fp32.
+     *     Heads with an empty selection get zeros. */
+    float* attn_out;
+    /* optional counters, zeroed by the caller: (T, HIRA_MAX_LEVELS+2) uint64:
+     *     [l] nodes of level l evaluated by at least one head of the tree's group
+     *     (l = 0: candidate keys), [HIRA_MAX_LEVELS] keys selected by at least one head,
+     *     [HIRA_MAX_LEVELS+1] (key, head) selections. */
+    unsigned long long* stats;
+} HiraSearchOut;
+
+typedef struct HiraLaunch {
+    int32_t block_threads;  /* 64, 128 or 256; 0 = default */
+    int32_t nodes_per_wave; /* level-1 nodes one wavefront walks; 0 = default */
+    int32_t kernel;         /* 0 = auto, 1 = vector-ALU kernel, 2 = MFMA kernel (bf16) */
+} HiraLaunch;
+
+int hira_abi_version(void);
+const char* hira_last_error(void);
+
+/* Bytes of workspace hira_search needs for this tree/query (attention partials). */
+size_t hira_search_workspace_bytes(const HiraTree* tree, const HiraQuery* query,
+                                   const HiraQueue* queue, const HiraLaunch* launch);
+
+/*
+ * Halfspace range search (+ optional fused sparse attention).
+ * Replaces: fused_tree_search_v3 (kernels/cpp/torch_ext_v3.cpp:36-247),
+ * triton_two_level_filter / triton_three_level_filter (kernels/triton_search_wrappers.py:
+ * 113-211, 214-358; kernels/triton_search_kernels.py:6-148) and the attention function
+ * the reference leaves unwritten (attention/hira_attention.py:1-3).
+ * Semantics: a node is pruned when q.c + ||q||*r < tau; a key is selected when
+ * q.k >= tau (the CPU kernels' comparisons, torch_ext_v3.cpp:182, 212, 238).
+ * queue may be NULL.  workspace is needed only when out->attn_out != NULL.
+ */
+int hira_search(const HiraTree* tree, const HiraQuery* query, const HiraQueue* queue,
+                const HiraSearchOut* out, const HiraLaunch* launch, void* workspace,
+                size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HIRA_HIP_H */

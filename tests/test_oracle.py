@@ -1,0 +1,216 @@
+"""Pins the CPU oracle (oracle/hira_oracle.c) against the reference's golden vectors, the
+reference's own compiled C++ kernels where they are built, and closed forms."""
+import glob
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import hira_oracle as ho
+from oracle.build_ref import load_ref
+from helpers import midpoint_threshold, normalized_keys, random_query
+
+GOLDEN = sorted(glob.glob(str(Path(__file__).parent / "golden" / "*.npz")))
+
+
+def _tree_from_fixture(z) -> ho.CPUTree:
+    keys = z["keys"]
+    h, n, _ = keys.shape
+    nl = int(z["num_levels"])
+    tree = ho.CPUTree()
+    tree.levels.append(ho.Level(0, keys, np.zeros((h, n), np.float32), n,
+                                z["c2p_0"].astype(np.int64) if nl > 1 else None))
+    for l in range(1, nl):
+        c2p = z[f"c2p_{l}"].astype(np.int64) if f"c2p_{l}" in z else None
+        tree.levels.append(ho.Level(l, z[f"centers_{l}"], z[f"radii_{l}"],
+                                    z[f"centers_{l}"].shape[1], c2p))
+    return tree
+
+
+@pytest.mark.parametrize("path", GOLDEN, ids=[Path(p).stem for p in GOLDEN])
+def test_search_v3_matches_reference_golden(path):
+    """Selected set and scores of the oracle's walk == what the compiled reference kernels
+    returned on the same tree (all of v1..v4 agreed when the fixture was written)."""
+    z = np.load(path)
+    tree = _tree_from_fixture(z)
+    out = ho.search_v3(tree, z["query"], z["threshold"], z["scaling"], q2kv=z["q2kv"])
+    n = z["keys"].shape[1]
+    for v in ("v1", "v2", "v3", "v4"):
+        if f"sel_{v}" in z:
+            ref_sel = np.unpackbits(z[f"sel_{v}"], axis=1)[:, :n].astype(bool)
+            assert np.array_equal(out != 0, ref_sel), v
+    np.testing.assert_allclose(out, z["out_v3"], rtol=1e-5, atol=1e-6)
+    # and the closed form the reference's own tests use: where(s >= th, s * sc, 0)
+    bf = ho.brute_force(z["keys"], z["query"], z["threshold"], z["scaling"], z["q2kv"])
+    assert np.array_equal(bf != 0, out != 0)
+
+
+def test_brute_force_matches_numpy_closed_form():
+    keys = normalized_keys(3, 257, 48, seed=5)
+    q = random_query(6, 48, seed=6)
+    q2kv = np.array([2, 2, 0, 1, 1, 0])
+    s = np.einsum("hnd,hd->hn", keys[q2kv], q)
+    th = np.quantile(s, 0.7, axis=1).astype(np.float32)
+    sc = np.linspace(0.5, 2.0, 6).astype(np.float32)
+    out = ho.brute_force(keys, q, th, sc, q2kv)
+    want = np.where(s >= th[:, None], s * sc[:, None], 0.0)
+    band = np.abs(s - th[:, None]) < 1e-6
+    assert np.array_equal((out != 0) | band, (want != 0) | band)
+    np.testing.assert_allclose(out[~band], want[~band], rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("variant", ["v1", "v2", "v3", "v4"])
+def test_oracle_equals_compiled_reference(variant):
+    """Live comparison with the reference's C++ (skipped where oracle/_ref is not built)."""
+    ref = load_ref(f"hira_ref_{variant}")
+    if ref is None:
+        pytest.skip("oracle/_ref not built here")
+    d = 128 if variant == "v4" else 64
+    h_kv, h_q = 2, 6
+    keys = normalized_keys(h_kv, 320, d, seed=77)
+    q = random_query(h_q, d, seed=78)
+    tree = ho.build_cpu_tree(keys, 3, 8, max_iterations=2)
+    offs, chs = ho.csr_levels(tree)
+    q2kv = ho.default_q2kv(h_q, h_kv)
+    s = ho.scores(keys, q, q2kv)
+    th = midpoint_threshold(s, 40)
+    sc = np.full(h_q, 0.125, np.float32)
+    mine = ho.search_v3(tree, q, th, sc, q2kv=q2kv)
+    T = torch.from_numpy
+    base = (T(keys), T(q), T(th), [T(l.ball_centers) for l in tree.levels],
+            [T(l.ball_radii) for l in tree.levels],
+            [T(l.child2parent) if l.child2parent is not None else torch.empty(0, dtype=torch.long)
+             for l in tree.levels], [l.size for l in tree.levels])
+    adj = ([T(o) for o in offs], [T(c) for c in chs])
+    tail = (T(q2kv), T(sc))
+    if variant == "v1":
+        theirs = ref.fused_tree_search(*base, *tail)
+    elif variant == "v2":
+        theirs = ref.fused_tree_search_v2(*base, *tail)
+    elif variant == "v3":
+        theirs = ref.fused_tree_search_v3(*base, *adj, *tail)
+    else:
+        theirs = ref.fused_tree_search_v4(*base, *adj, *tail)
+    theirs = theirs.numpy()
+    assert np.array_equal(theirs != 0, mine != 0)
+    np.testing.assert_allclose(theirs, mine, rtol=1e-5, atol=1e-6)
+
+
+def test_walk_on_padded_tree_equals_brute_force():
+    """The fixed-fan-out (padded) layout the device kernels use, walked by the reference
+    algorithm through CSR lists of the children in use, selects the brute-force set; works
+    when N is not a multiple of bf (pad slots) and with the ||q|| radius scale."""
+    keys = normalized_keys(2, 203, 32, seed=9) * 3.0
+    q = random_query(4, 32, seed=10, normalize=False)
+    ff = ho.fixed_fanout_tree(keys, 4, 4, niter=2)
+    assert ff.sizes == [256, 64, 16, 4]
+    assert int((ff.perm >= 0).sum()) == 2 * 203
+    tree, csr = ho.fixed_fanout_as_cpu_tree(ff)
+    q2kv = ho.default_q2kv(4, 2)
+    s_slot = ho.scores(ff.keys, q, q2kv)
+    valid = ff.perm[q2kv] >= 0
+    th = midpoint_threshold(np.where(valid, s_slot, -1e30), 25)
+    rs = np.linalg.norm(q, axis=1).astype(np.float32)
+    out, st = ho.search_v3(tree, q, th, rscale=rs, q2kv=q2kv, csr=csr, want_stats=True)
+    assert np.array_equal(out != 0, (s_slot >= th[:, None]) & valid)
+    # radius invariant of the reference (tests/test_cpu_indexer_searcher.py:62-81)
+    for l in range(1, ff.num_levels):
+        for h in range(2):
+            cc = ff.keys[h] if l == 1 else ff.centers[l - 1][h]
+            cr = np.zeros(ff.sizes[0], np.float32) if l == 1 else ff.radii[l - 1][h]
+            ok = (ff.perm[h] >= 0) if l == 1 else (ff.counts[l - 1][h] > 0)
+            par = np.repeat(ff.centers[l][h], ff.bf, axis=0)
+            need = np.linalg.norm(cc - par, axis=1) + np.where(ok, cr, 0)
+            have = np.repeat(ff.radii[l][h], ff.bf)
+            assert np.all(have[ok] + 1e-4 >= need[ok])
+
+
+def test_group_traffic_is_union_over_heads():
+    keys = normalized_keys(1, 512, 32, seed=11)
+    q = random_query(4, 32, seed=12)
+    ff = ho.fixed_fanout_tree(keys, 8, 3, niter=2)
+    tree, csr = ho.fixed_fanout_as_cpu_tree(ff)
+    q2kv = np.zeros(4, np.int64)
+    th = midpoint_threshold(ho.scores(ff.keys, q, q2kv), 20)
+    _, st = ho.search_v3(tree, q, th, q2kv=q2kv, csr=csr, want_stats=True)
+    tr = ho.group_traffic(tree, q, th, q2kv=q2kv, csr=csr)
+    assert tr.shape == (1, 4)
+    for col in range(4):
+        assert st[:, col].max() <= tr[0, col] <= st[:, col].sum()
+    assert tr[0, 2] == ff.sizes[2]  # every root node is evaluated
+
+
+def test_build_csr_matches_numpy():
+    rng = np.random.default_rng(0)
+    c2p = rng.integers(0, 7, size=(3, 50))
+    off, ch = ho.build_csr(c2p, 7)
+    for h in range(3):
+        order = np.argsort(c2p[h], kind="stable")
+        assert np.array_equal(ch[h], order)
+        assert np.array_equal(np.diff(off[h]), np.bincount(c2p[h], minlength=7))
+
+
+def test_refine_radii_closed_form_and_empty_parent():
+    rng = np.random.default_rng(1)
+    cc = rng.normal(size=(40, 8)).astype(np.float32)
+    cr = rng.random(40).astype(np.float32)
+    pc = rng.normal(size=(5, 8)).astype(np.float32)
+    assign = rng.integers(0, 4, size=40)  # parent 4 stays empty
+    r = ho.refine_radii(cc, cr, assign, pc)
+    for p in range(4):
+        m = assign == p
+        want = (np.linalg.norm(cc[m] - pc[p], axis=1) + cr[m]).max()
+        assert abs(r[p] - want) < 1e-5
+    assert r[4] == -np.inf  # indexer/cpu.py:300-309: an empty parent is never visited
+
+
+def test_kmeans_special_cases_and_monotone_inertia():
+    rng = np.random.default_rng(2)
+    x = rng.normal(size=(300, 16)).astype(np.float32)
+    c, a, _ = ho.kmeans(x, 1, 3, seed=1)
+    np.testing.assert_allclose(c[0], x.mean(0), atol=1e-5)
+    assert (a == 0).all()
+    c, a, tr = ho.kmeans(x, 300, 2, seed=1)  # K = n: every point its own centroid
+    assert len(set(a.tolist())) == 300 and tr[-1] < 1e-8
+    c, a, tr = ho.kmeans(x, 12, 8, seed=3)
+    assert np.all(np.diff(tr) <= 1e-6 * tr[0])  # Lloyd never increases the inertia
+    d2 = ((x[:, None, :] - c[None]) ** 2).sum(-1)
+    assert np.allclose(d2[np.arange(300), a], d2.min(1), rtol=1e-5, atol=1e-6)
+    # same seed, same result; other seed, other initial sample
+    c2, a2, _ = ho.kmeans(x, 12, 8, seed=3)
+    assert np.array_equal(c, c2) and np.array_equal(a, a2)
+
+
+def test_cpu_tree_level_sizes_follow_reference():
+    """indexer/cpu.py:78-83: N, N//bf, ... stopping when the next size is 0 or at num_levels."""
+    keys = normalized_keys(1, 192, 16, seed=3)
+    assert [l.size for l in ho.build_cpu_tree(keys, 4, 8).levels] == [192, 24, 3]
+    assert [l.size for l in ho.build_cpu_tree(keys, 2, 8).levels] == [192, 24]
+    assert [l.size for l in ho.build_cpu_tree(keys, 1, 8).levels] == [192]
+    t = ho.build_cpu_tree(keys, 3, 8)
+    assert (t.levels[0].ball_radii == 0).all()
+    assert t.levels[0].child2parent.max() < 24 and t.levels[-1].child2parent is None
+
+
+def test_attention_matches_torch_softmax_and_full_selection_is_sdpa():
+    rng = np.random.default_rng(4)
+    keys = rng.normal(size=(2, 64, 16)).astype(np.float32)
+    vals = rng.normal(size=(2, 64, 24)).astype(np.float32)
+    q = rng.normal(size=(4, 16)).astype(np.float32)
+    sc = np.full(4, 0.25, np.float32)
+    q2kv = ho.default_q2kv(4, 2)
+    mask = rng.random((4, 64)) < 0.3
+    mask[3] = False  # empty selection -> zeros
+    out = ho.attention(keys, vals, q, sc, mask, q2kv)
+    K, V, Q = (torch.from_numpy(a).double() for a in (keys, vals, q))
+    for h in range(3):
+        idx = torch.from_numpy(np.nonzero(mask[h])[0])
+        w = torch.softmax(0.25 * (K[q2kv[h]][idx] @ Q[h]), 0)
+        np.testing.assert_allclose(out[h], (w[:, None] * V[q2kv[h]][idx]).sum(0).numpy(), atol=1e-12)
+    assert (out[3] == 0).all()
+    full = ho.attention(keys, vals, q, sc, np.ones((4, 64), bool), q2kv)
+    sdpa = torch.nn.functional.scaled_dot_product_attention(
+        Q.view(2, 2, 1, 16), K.view(2, 1, 64, 16).expand(2, 2, 64, 16),
+        V.view(2, 1, 64, 24).expand(2, 2, 64, 24), scale=0.25).reshape(4, 24)
+    np.testing.assert_allclose(full, sdpa.numpy(), atol=1e-10)
