@@ -38,3 +38,25 @@ def assert_same_selection(got_mask: np.ndarray, scores: np.ndarray, th: np.ndarr
     bad = (got_mask != want) & ~band
     assert not bad.any(), f"{int(bad.sum())} keys differ outside the threshold band"
     return int(band.sum())
+
+
+def clustered_keys(h: int, n: int, d: int, seed: int, clusters: int = 16,
+                   spread: float = 0.15) -> np.ndarray:
+    """Keys around `clusters` well-separated centres, so that ball bounds really prune."""
+    g = torch.Generator().manual_seed(seed)
+    cen = torch.randn((h, clusters, d), generator=g)
+    cen = cen / cen.norm(dim=-1, keepdim=True)
+    which = torch.randint(0, clusters, (h, n), generator=g)
+    x = torch.gather(cen, 1, which[..., None].expand(h, n, d))
+    x = x + spread * torch.randn((h, n, d), generator=g) / d ** 0.5
+    return x.numpy()
+
+
+def bf16_round(a: np.ndarray) -> np.ndarray:
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(torch.bfloat16).float().numpy()
+
+
+def rel_err(got: np.ndarray, ref: np.ndarray) -> float:
+    """max |got - ref| over max |ref|, per row, worst row."""
+    den = np.maximum(np.abs(ref).max(axis=-1), 1e-30)
+    return float((np.abs(got - ref).max(axis=-1) / den).max())

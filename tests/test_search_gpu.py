@@ -1,0 +1,214 @@
+"""GPU parity of the HIP search / sparse-attention path against the CPU oracle, through
+the C ABI (hira_search), on trees built on the host by the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import hira_oracle as ho
+from helpers import (assert_same_selection, bf16_round, clustered_keys, midpoint_threshold,
+                     normalized_keys, random_query, rel_err)
+
+pytestmark = pytest.mark.gpu
+
+
+def _setup(h_kv, h_q, n, d, bf, nl, dtype, seed, keep, clustered=True, q2kv=None, dv=None,
+           unit_q=True, niter=2):
+    from hira_amd.indexer.hip import HIPIndexer
+
+    keys = (clustered_keys if clustered else normalized_keys)(h_kv, n, d, seed)
+    rng = np.random.default_rng(seed)
+    dv = d if dv is None else dv
+    vals = rng.normal(size=(h_kv, n, dv)).astype(np.float32)
+    q = random_query(h_q, d, seed + 1, normalize=unit_q)
+    if not unit_q:
+        q = q * 3.0
+    rnd = bf16_round if dtype == torch.bfloat16 else (lambda a: a)
+    keys, vals, q = rnd(keys), rnd(vals), rnd(q)
+    ff = ho.fixed_fanout_tree(keys, bf, nl, niter=niter, round_fn=rnd if nl > 1 else None)
+    ok = ff.perm >= 0
+    vslot = np.zeros((h_kv, ff.sizes[0], dv), np.float32)
+    for h in range(h_kv):
+        vslot[h][ok[h]] = vals[h][ff.perm[h][ok[h]]]
+    q2kv = ho.default_q2kv(h_q, h_kv) if q2kv is None else np.asarray(q2kv)
+    s = ho.scores(ff.keys, q, q2kv)
+    valid = ok[q2kv]
+    th = midpoint_threshold(np.where(valid, s, -1e30), keep)
+    idx = HIPIndexer.from_layout(bf=bf, keys=ff.keys, perm=ff.perm, centers=ff.centers,
+                                 radii=ff.radii, counts=ff.counts, values=vslot, dtype=dtype,
+                                 num_keys=n)
+    return dict(ff=ff, idx=idx, q=q, th=th, s=s, valid=valid, q2kv=q2kv, keys=keys, vals=vals,
+                vslot=vslot)
+
+
+CASES = [
+    # h_kv, h_q, n, d, bf, levels, dtype, keep
+    (2, 2, 192, 64, 8, 3, torch.float32, 48),
+    (2, 6, 192, 128, 8, 3, torch.float32, 48),
+    (1, 1, 4096, 128, 16, 2, torch.float32, 205),
+    (2, 8, 2048, 128, 32, 3, torch.bfloat16, 41),
+    (2, 16, 1024, 128, 32, 3, torch.bfloat16, 30),   # 8 heads per tree
+    (1, 12, 600, 64, 8, 3, torch.bfloat16, 30),      # 12 heads per tree: two passes
+    (3, 3, 203, 32, 4, 4, torch.float32, 25),        # pad slots, 4 levels
+    (2, 4, 333, 16, 5, 3, torch.float32, 40),        # odd fan-out, narrow rows
+    (2, 4, 333, 16, 5, 3, torch.bfloat16, 40),
+    (1, 2, 500, 256, 16, 2, torch.float32, 50),
+    (1, 2, 500, 256, 16, 2, torch.bfloat16, 50),
+    (2, 2, 300, 64, 8, 1, torch.float32, 30),        # one level: flat scan
+    (1, 4, 70000, 128, 32, 4, torch.bfloat16, 700),
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=[f"hkv{c[0]}_hq{c[1]}_n{c[2]}_d{c[3]}_bf{c[4]}_L{c[5]}_"
+                                               f"{'bf16' if c[6] == torch.bfloat16 else 'f32'}"
+                                               for c in CASES])
+def test_selected_set_and_scores_match_oracle(case, gpu_device):
+    from hira_amd.searcher.hip import HIPSearcher
+
+    h_kv, h_q, n, d, bf, nl, dtype, keep = case
+    print(f"case {case}", flush=True)
+    c = _setup(h_kv, h_q, n, d, bf, nl, dtype, seed=100 + n, keep=keep, niter=1 if n > 5000 else 2)
+    sc = torch.full((h_q,), 0.125)
+    searcher = HIPSearcher()
+    q4 = torch.from_numpy(c["q"]).view(1, h_q, 1, d)
+    out = searcher.search(q4, torch.from_numpy(c["th"]), c["idx"], scaling=sc).cpu().numpy()
+    # slot space: bit-exact set, outside the 1e-5 relative band around the threshold
+    s = np.where(c["valid"], c["s"], -np.inf).astype(np.float32)
+    assert_same_selection(out != 0, s, c["th"])
+    m = out != 0
+    np.testing.assert_allclose(out[m], (c["s"] * 0.125)[m], rtol=2e-5, atol=1e-6)
+    # position space (the CPU searcher's contract): compare with the oracle on the keys in
+    # insertion order
+    pos = searcher.search(q4, torch.from_numpy(c["th"]), c["idx"], scaling=sc,
+                          index_space="position").cpu().numpy()
+    assert pos.shape == (h_q, n)
+    s_pos = ho.scores(c["keys"], c["q"], c["q2kv"])
+    assert_same_selection(pos != 0, s_pos, c["th"])
+    # compact lists carry the same set
+    idx, score, count = searcher.search_compact(q4, torch.from_numpy(c["th"]), c["idx"], scaling=sc)
+    idx, score, count = idx.cpu().numpy(), score.cpu().numpy(), count.cpu().numpy()
+    for h in range(h_q):
+        got = np.sort(idx[h, :count[h]])
+        assert np.array_equal(got, np.nonzero(m[h])[0])
+        order = np.argsort(idx[h, :count[h]])
+        np.testing.assert_allclose(score[h, :count[h]][order] * 0.125, out[h][m[h]], rtol=1e-6)
+
+
+def test_explicit_non_monotone_head_map(gpu_device):
+    """tests/test_cpp_kernels.py:529-565 of the reference: q_head_to_kv = [1, 0, 1, 0]."""
+    from hira_amd.searcher.hip import HIPSearcher
+
+    c = _setup(2, 4, 192, 64, 8, 3, torch.float32, seed=311, keep=38, q2kv=[1, 0, 1, 0])
+    out = HIPSearcher().search(torch.from_numpy(c["q"]), torch.from_numpy(c["th"]), c["idx"],
+                               q_head_to_kv=torch.tensor([1, 0, 1, 0])).cpu().numpy()
+    s = np.where(c["valid"], c["s"], -np.inf).astype(np.float32)
+    assert_same_selection(out != 0, s, c["th"])
+
+
+def test_non_unit_queries_use_norm_scaled_radius(gpu_device):
+    """The gate q.c + ||q|| r stays conservative for ||q|| != 1 (searcher/cpu.py:61-63)."""
+    from hira_amd.searcher.hip import HIPSearcher
+
+    c = _setup(2, 4, 1000, 64, 8, 3, torch.float32, seed=21, keep=60, unit_q=False)
+    out = HIPSearcher().search(torch.from_numpy(c["q"]), torch.from_numpy(c["th"]), c["idx"]).cpu().numpy()
+    s = np.where(c["valid"], c["s"], -np.inf).astype(np.float32)
+    assert_same_selection(out != 0, s, c["th"])
+
+
+def test_low_threshold_returns_every_valid_score_and_zero_scaling_returns_zeros(gpu_device):
+    """tests/test_triton_kernels.py:243-280, tests/test_cpu_pipeline.py:257-267."""
+    from hira_amd.searcher.hip import HIPSearcher
+
+    c = _setup(2, 2, 203, 32, 4, 3, torch.float32, seed=5, keep=10)
+    se = HIPSearcher(output_fill_value=-7.0)
+    out = se.search(torch.from_numpy(c["q"]), -2.0, c["idx"]).cpu().numpy()
+    assert np.all(out[~c["valid"]] == -7.0)
+    np.testing.assert_allclose(out[c["valid"]], c["s"][c["valid"]], rtol=2e-5, atol=1e-6)
+    z = HIPSearcher().search(torch.from_numpy(c["q"]), -2.0, c["idx"], scaling=torch.zeros(2))
+    assert float(z.abs().max()) == 0.0
+
+
+def test_device_counters_match_oracle_traffic(gpu_device):
+    from hira_amd.searcher.hip import HIPSearcher
+    from hira_amd import _lib
+
+    c = _setup(2, 8, 4096, 64, 16, 3, torch.float32, seed=8, keep=40)
+    stats = torch.zeros((2, _lib.HIRA_MAX_LEVELS + 2), dtype=torch.int64, device="cuda")
+    HIPSearcher().search(torch.from_numpy(c["q"]), torch.from_numpy(c["th"]), c["idx"], stats=stats)
+    tree, csr = ho.fixed_fanout_as_cpu_tree(c["ff"])
+    tr = ho.group_traffic(tree, c["q"], c["th"], q2kv=c["q2kv"], csr=csr,
+                          rscale=np.linalg.norm(c["q"], axis=1))
+    st = stats.cpu().numpy()
+    assert np.array_equal(st[:, :3], tr[:, :3])
+    assert np.array_equal(st[:, _lib.HIRA_MAX_LEVELS], tr[:, 3])
+    assert (tr[:, 0] < 4096).all()  # the clustered keys are really pruned
+
+
+ATTN_CASES = [
+    (1, 1, 4096, 128, 16, 2, torch.float32, 205, 1e-5),
+    (2, 8, 2048, 128, 32, 3, torch.bfloat16, 41, 2e-3),
+    (2, 16, 1024, 128, 32, 3, torch.bfloat16, 30, 2e-3),
+    (3, 3, 203, 32, 4, 4, torch.float32, 25, 1e-5),
+    (2, 4, 333, 16, 5, 3, torch.bfloat16, 40, 2e-3),
+    (2, 2, 300, 64, 8, 1, torch.float32, 30, 1e-5),
+]
+
+
+@pytest.mark.parametrize("case", ATTN_CASES, ids=[f"hkv{c[0]}_hq{c[1]}_n{c[2]}_d{c[3]}_L{c[5]}_"
+                                                    f"{'bf16' if c[6] == torch.bfloat16 else 'f32'}"
+                                                    for c in ATTN_CASES])
+def test_fused_attention_matches_fp64_oracle(case, gpu_device):
+    """softmax(scaling q.K_S^T) V_S over the oracle's selected set; tolerance 1e-5 (fp32
+    storage) / 2e-3 (bf16 storage) relative to the largest output component of the head."""
+    from hira_amd.searcher.hip import HIPSearcher
+
+    h_kv, h_q, n, d, bf, nl, dtype, keep, tol = case
+    print(f"case {case}", flush=True)
+    c = _setup(h_kv, h_q, n, d, bf, nl, dtype, seed=300 + n, keep=keep)
+    scale = d ** -0.5
+    sc = torch.full((h_q,), scale)
+    out = HIPSearcher().search_attention(torch.from_numpy(c["q"]), torch.from_numpy(c["th"]),
+                                         c["idx"], scaling=sc).cpu().numpy()
+    mask = (c["s"] >= c["th"][:, None]) & c["valid"]
+    ref = ho.attention(c["ff"].keys, c["vslot"], c["q"], sc.numpy(), mask, c["q2kv"])
+    assert rel_err(out, ref) <= tol, rel_err(out, ref)
+
+
+def test_attention_with_queue_and_empty_selection(gpu_device):
+    from hira_amd.searcher.hip import HIPSearcher
+
+    c = _setup(2, 4, 512, 64, 8, 3, torch.float32, seed=55, keep=20)
+    rng = np.random.default_rng(3)
+    qk = rng.normal(size=(2, 37, 64)).astype(np.float32) * 0.1
+    qv = rng.normal(size=(2, 37, 64)).astype(np.float32)
+    sc = torch.full((4,), 0.5)
+    th = c["th"].copy()
+    th[3] = 1e9  # head 3 selects nothing from the index: only the queue remains
+    out = HIPSearcher().search_attention(
+        torch.from_numpy(c["q"]), torch.from_numpy(th), c["idx"], scaling=sc,
+        queue_keys=torch.from_numpy(qk), queue_values=torch.from_numpy(qv)).cpu().numpy()
+    keys_all = np.concatenate([c["ff"].keys, qk], axis=1)
+    vals_all = np.concatenate([c["vslot"], qv], axis=1)
+    mask = (c["s"] >= th[:, None]) & c["valid"]
+    mask = np.concatenate([mask, np.ones((4, 37), bool)], axis=1)
+    ref = ho.attention(keys_all, vals_all, c["q"], sc.numpy(), mask, c["q2kv"])
+    assert rel_err(out, ref) <= 1e-5
+    # no queue and nothing selected -> zeros
+    z = HIPSearcher().search_attention(torch.from_numpy(c["q"]), 1e9, c["idx"], scaling=sc)
+    assert float(z.abs().max()) == 0.0
+
+
+def test_bad_inputs_raise_value_error(gpu_device):
+    """tests/test_triton_kernels.py:547-601 of the reference."""
+    from hira_amd.searcher.hip import HIPSearcher
+
+    c = _setup(2, 2, 192, 64, 8, 3, torch.float32, seed=1, keep=10)
+    se = HIPSearcher()
+    q = torch.from_numpy(c["q"])
+    with pytest.raises(ValueError):
+        se.search(q[:, :32], torch.from_numpy(c["th"]), c["idx"])       # wrong dim
+    with pytest.raises(ValueError):
+        se.search(q.view(2, 1, 1, 64)[:, :, :, :], torch.zeros(3), c["idx"])  # threshold length
+    with pytest.raises(ValueError):
+        se.search(q, torch.from_numpy(c["th"]), c["idx"], scaling=torch.ones(5))
+    with pytest.raises(ValueError):
+        se.search(torch.zeros(3, 64), torch.zeros(3), c["idx"])         # 3 heads over 2 trees
