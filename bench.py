@@ -1,0 +1,321 @@
+#!/usr/bin/env python3
+"""Decode benchmark: one "step" = index search + sparse attention for one fresh query of every
+head of one layer (32 query / 8 KV heads, d = 128, bf16) over a 32k-token context; keys,
+values, index, queries and thresholds are resident in HBM before the timed region starts.
+
+    python bench.py [--gpus 1] [--steps 256] [--warmup 16] [--config 2]
+
+Prints ONE JSON line.  `value` = microseconds per step (whole layer, all heads) with the K
+steps replayed back to back from one HIP graph; `roofline` prices the search kernel against
+HBM bandwidth using the ALGORITHMIC bytes of the walk (nodes evaluated x (d*e + 4) +
+candidate keys x d*e + selected values x d*e + queries + output; counted by the kernel's
+own counters, which the tests tie to the CPU oracle); `cpu_baseline` times the reference's
+own C++ search kernel (compiled into oracle/_ref) -- or, if that is absent, the C
+restatement in oracle/ -- plus a host softmax-V, on a bounded sample of the same steps.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def algorithmic_bytes(stats, w, num_levels, steps):
+    """Mean algorithmic bytes per step from the device counters summed over `steps` steps.
+    stats: (T, MAX_LEVELS+2) int64."""
+    import numpy as np
+    from hira_amd import _lib
+
+    e = 2 if str(w.dtype).endswith("bfloat16") else 4
+    s = stats.astype(np.float64).sum(0) / steps
+    nodes = sum(s[l] for l in range(1, num_levels))
+    cand = s[0]
+    sel_any = s[_lib.HIRA_MAX_LEVELS]
+    h_q = w.h_q * w.batch
+    b_search = nodes * (w.d * e + 4) + cand * w.d * e
+    b_attn = sel_any * w.d * e + h_q * w.d * 4 + h_q * w.d * e
+    return b_search + b_attn, dict(nodes_per_step=nodes, candidates_per_step=cand,
+                                   selected_union_per_step=sel_any,
+                                   selected_pairs_per_step=s[_lib.HIRA_MAX_LEVELS + 1])
+
+
+def cpu_baseline(w, index, queries, taus, scale, budget_s=20.0):
+    """Reference CPU search (+ host softmax-V) on the same tree, first steps of the same
+    queries, for about `budget_s` seconds of CPU work."""
+    import numpy as np
+    import torch
+    from oracle import hira_oracle as ho
+    from oracle.build_ref import load_ref
+
+    threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")), w.h_q)
+    torch.set_num_threads(threads)
+    n0 = index.size[0]
+    ff = ho.FixedFanoutTree(
+        bf=index.branching_factor,
+        keys=index.keys_buf[:, :n0].float().cpu().numpy(),
+        perm=index.perm[:, :n0].cpu().numpy().astype(np.int64),
+        centers=[None] + [index.centers[l][:, : index.size[l]].float().cpu().numpy()
+                          for l in range(1, index.num_levels)],
+        radii=[None] + [index.radii[l][:, : index.size[l]].cpu().numpy()
+                        for l in range(1, index.num_levels)],
+        counts=[None] + [index.counts[l][:, : index.size[l]].cpu().numpy()
+                         for l in range(1, index.num_levels)],
+        sizes=list(index.size))
+    vals = index.values_buf[:, :n0].float().cpu().numpy()
+    tree, csr = ho.fixed_fanout_as_cpu_tree(ff)
+    ref = None
+    try:
+        ref = load_ref("hira_ref_v3")
+    except Exception as ex:  # noqa: BLE001
+        log(f"[cpu_baseline] compiled reference not loadable ({ex}); timing the C port")
+    q2kv = ho.default_q2kv(w.h_q, w.h_kv)
+    T = torch.from_numpy
+    if ref is not None:
+        os.environ["OMP_NUM_THREADS"] = str(threads)
+        args_tree = ([T(l.ball_centers) for l in tree.levels], [T(l.ball_radii) for l in tree.levels],
+                     [T(l.child2parent) if l.child2parent is not None
+                      else torch.empty(0, dtype=torch.long) for l in tree.levels],
+                     [l.size for l in tree.levels], [T(o) for o in csr[0]], [T(c) for c in csr[1]])
+        keys_t = T(ff.keys)
+
+    def one_step(i):
+        q = queries[i].float().cpu().numpy().reshape(w.h_q, w.d)
+        th = taus[i].cpu().numpy().reshape(w.h_q)
+        qn = np.linalg.norm(q, axis=1).astype(np.float32)
+        sc = np.full(w.h_q, scale, np.float32)
+        t0 = time.perf_counter()
+        if ref is not None:
+            # unit-norm query, threshold and scaling rescaled: the same set, the bound the
+            # reference assumes (searcher/cpu.py:61-63)
+            out = ref.fused_tree_search_v3(keys_t, T(q / qn[:, None]), T(th / qn), *args_tree,
+                                           T(q2kv), T(sc * qn)).numpy()
+        else:
+            out = ho.search_v3(tree, q, th, sc, rscale=qn, q2kv=q2kv, csr=csr, fast=True,
+                               num_threads=threads)
+        # host attention over the selected keys, fp32
+        o = np.zeros((w.h_q, w.d), np.float32)
+        for h in range(w.h_q):
+            idx = np.nonzero(out[h])[0]
+            if idx.size:
+                z = out[h, idx]
+                p = np.exp(z - z.max())
+                o[h] = (p[:, None] * vals[q2kv[h], idx]).sum(0) / p.sum()
+        return time.perf_counter() - t0, out, o
+
+    one_step(0)  # warm-up
+    times = []
+    t_start = time.perf_counter()
+    i = 0
+    while i < len(queries) and (time.perf_counter() - t_start) < budget_s:
+        dt, _, _ = one_step(i)
+        times.append(dt)
+        i += 1
+    times = np.array(times)
+    return dict(value=float(np.median(times) * 1e6), unit="us/layer", cores=threads,
+                kind="reference" if ref is not None else "port",
+                sample=f"first {len(times)} of the timed decode steps (same tree, queries, "
+                       f"thresholds); median; p99 {float(np.percentile(times, 99) * 1e6):.0f} us; "
+                       f"search = reference v3 C++ kernel, attention = numpy fp32")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--config", type=int, default=2)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-budget", type=float, default=20.0)
+    ap.add_argument("--block-threads", type=int, default=0)
+    ap.add_argument("--nodes-per-wave", type=int, default=0)
+    ap.add_argument("--kernel", type=int, default=0)
+    ap.add_argument("--kmeans-iters", type=int, default=-1)
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        log("bench.py: this path is built and measured on ONE GPU (each KV head owns an "
+            "independent tree, so more GPUs would shard by head without any exchange); "
+            "run with --gpus 1")
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from hira_amd import _lib, synth
+    from hira_amd.cache.threshold_finder import exact_topk
+    from hira_amd.indexer import HIPIndexer
+    from hira_amd.searcher import HIPSearcher
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    dev = torch.device("cuda:0")
+    w = synth.WORKLOADS[a.config]
+    K, W = a.steps, a.warmup
+    total = K + W
+    log(f"[bench] workload {w.name}: generating keys/values/queries on the host")
+    keys, values = synth.make_kv(w)
+    queries = synth.make_queries(w, keys, total)  # (total, B, H_q, D)
+    keys_d, values_d = keys.to(dev), values.to(dev)
+    niter = w.kmeans_iters if a.kmeans_iters < 0 else a.kmeans_iters
+    t0 = time.perf_counter()
+    index = HIPIndexer(w.num_levels, niter, w.bf, device="cuda:0").build(keys_d, values_d)
+    torch.cuda.synchronize()
+    build_ms = (time.perf_counter() - t0) * 1e3
+    log(f"[bench] index built in {build_ms:.1f} ms, level sizes {index.size}")
+
+    # thresholds: exactly ceil(p*N) keys per head (midpoint between neighbouring scores)
+    fr = synth.select_fractions(w)
+    q_d = queries.to(dev).reshape(total, w.batch * w.h_q, w.d).contiguous()
+    taus = torch.empty((total, w.batch * w.h_q), dtype=torch.float32, device=dev)
+    ksel = [int(np.ceil(float(fr[b]) * w.n)) for b in range(w.batch)]
+    for b in range(w.batch):
+        hs = slice(b * w.h_q, (b + 1) * w.h_q)
+        for i in range(total):
+            taus[i, hs] = exact_topk(keys_d[b], q_d[i, hs], ksel[b])
+    scale = w.d ** -0.5
+    searcher = HIPSearcher(block_threads=a.block_threads, nodes_per_wave=a.nodes_per_wave,
+                           kernel=a.kernel)
+    h_all = w.batch * w.h_q
+    plan = searcher.plan_attention(index, h_all, scaling=torch.full((h_all,), scale))
+    outs = torch.empty((total, h_all, w.d), dtype=torch.float32, device=dev)
+
+    # ---- warm-up (eager) -----------------------------------------------------------
+    for i in range(W):
+        plan.run(q_d[i], taus[i], outs[i])
+    torch.cuda.synchronize()
+
+    # ---- counters: algorithmic bytes of the K timed steps ---------------------------
+    stats = torch.zeros((index.num_trees, _lib.HIRA_MAX_LEVELS + 2), dtype=torch.int64, device=dev)
+    splan = searcher.plan_attention(index, h_all, scaling=torch.full((h_all,), scale), stats=stats)
+    scratch = torch.empty((h_all, w.d), dtype=torch.float32, device=dev)
+    for i in range(W, total):
+        splan.run(q_d[i], taus[i], scratch)
+    torch.cuda.synchronize()
+    alg_bytes, counts = algorithmic_bytes(stats.cpu().numpy(), w, index.num_levels, K)
+    want_pairs = sum(ksel[b] * w.h_q for b in range(w.batch))
+    if abs(counts["selected_pairs_per_step"] - want_pairs) > 1e-6 * want_pairs:
+        log(f"[bench] WARNING: selected {counts['selected_pairs_per_step']} pairs/step, "
+            f"expected {want_pairs}")
+
+    # ---- timed: K steps captured in one HIP graph, replayed once --------------------
+    stream = torch.cuda.Stream(device=dev)
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            for i in range(W, total):
+                plan.run(q_d[i], taus[i], outs[i])
+        graph.replay()  # untimed: first replay uploads the graph
+        stream.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ev0.record(stream)
+        graph.replay()
+        ev1.record(stream)
+        stream.synchronize()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3
+        graph_ms = ev0.elapsed_time(ev1)
+
+        # eager loop (one library call per step from Python), for comparison
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for i in range(W, total):
+            plan.run(q_d[i], taus[i], outs[i], stream=stream.cuda_stream)
+        e1.record(stream)
+        stream.synchronize()
+        eager_ms = e0.elapsed_time(e1)
+    us_per_step = wall_ms * 1e3 / K
+    kernel_us = graph_ms * 1e3 / K
+
+    # ---- dense comparators ------------------------------------------------------------
+    dense_us = {}
+    try:
+        qd = q_d[W:].reshape(K, w.batch, w.h_q, 1, w.d)
+        kk = keys_d[:, :, None].expand(w.batch, w.h_kv, w.group, w.n, w.d).reshape(
+            w.batch, w.h_q, w.n, w.d)
+        vv = values_d[:, :, None].expand(w.batch, w.h_kv, w.group, w.n, w.d).reshape(
+            w.batch, w.h_q, w.n, w.d)
+        reps = min(K, 32)
+        for name, kw in (("sdpa_gqa", dict(enable_gqa=True)), ("sdpa_expanded", {})):
+            kx, vx = (keys_d, values_d) if kw else (kk, vv)
+            for _ in range(3):
+                torch.nn.functional.scaled_dot_product_attention(qd[0], kx, vx, scale=scale, **kw)
+            torch.cuda.synchronize()
+            d0, d1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            d0.record()
+            for i in range(reps):
+                torch.nn.functional.scaled_dot_product_attention(qd[i], kx, vx, scale=scale, **kw)
+            d1.record()
+            torch.cuda.synchronize()
+            dense_us[name] = d0.elapsed_time(d1) * 1e3 / reps
+    except Exception as ex:  # noqa: BLE001
+        log(f"[bench] dense SDPA comparator failed: {ex}")
+    # our kernel with every key selected (threshold -inf): a dense decode attention
+    ninf = torch.full((h_all,), -3.0e38, dtype=torch.float32, device=dev)
+    for _ in range(3):
+        plan.run(q_d[0], ninf, scratch)
+    torch.cuda.synchronize()
+    d0, d1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    d0.record()
+    for i in range(16):
+        plan.run(q_d[W + i % K], ninf, scratch)
+    d1.record()
+    torch.cuda.synchronize()
+    dense_us["ours_all_selected"] = d0.elapsed_time(d1) * 1e3 / 16
+    dense_best = min(dense_us.values())
+
+    e = 2 if w.dtype == torch.bfloat16 else 4
+    dense_bytes = 2.0 * w.batch * w.h_kv * w.n * w.d * e
+    achieved = alg_bytes / (kernel_us * 1e-6) / 1e9
+    result = {
+        "metric": "decode search+sparse-attn us/layer at 32k ctx; achieved HBM GB/s vs 8 TB/s",
+        "value": round(us_per_step, 3),
+        "unit": "us/layer",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": W,
+        "ms_per_step": round(us_per_step / 1e3, 6),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if w.dtype == torch.bfloat16 else "f32",
+        "data": "synthetic",
+        "config": {"workload": w.name, "h_q": w.h_q, "h_kv": w.h_kv, "context": w.n,
+                   "head_dim": w.d, "batch": w.batch, "levels": w.num_levels, "bf": w.bf,
+                   "select_per_head": ksel, "kmeans_iters": niter},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None},
+        "algorithmic_bytes_per_step": round(alg_bytes),
+        "gpu_us_per_step_events": round(kernel_us, 3),
+        "eager_us_per_step": round(eager_ms * 1e3 / K, 3),
+        "dense_attention_us": {k: round(v, 2) for k, v in dense_us.items()},
+        "dense_attention_bytes": dense_bytes,
+        "frac_of_dense_time": round(kernel_us / dense_best, 4),
+        "counters": {k: round(v, 1) for k, v in counts.items()},
+        "index_build_ms": round(build_ms, 1),
+    }
+    if not a.no_cpu:
+        try:
+            result["cpu_baseline"] = cpu_baseline(w, index, q_d[W:], taus[W:], scale,
+                                                  a.cpu_budget)
+        except Exception as ex:  # noqa: BLE001
+            log(f"[bench] cpu baseline failed: {ex!r}")
+            result["cpu_baseline"] = None
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

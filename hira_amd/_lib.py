@@ -90,6 +90,12 @@ SYMBOLS = {
         [C.POINTER(HiraTree), C.POINTER(HiraQuery), C.POINTER(HiraQueue),
          C.POINTER(HiraSearchOut), C.POINTER(HiraLaunch), _vp, C.c_size_t, _vp],
     ),
+    "hira_build_workspace_bytes": (C.c_size_t, [C.POINTER(HiraTree), C.c_int32]),
+    "hira_build": (
+        C.c_int,
+        [C.POINTER(HiraTree), _vp, _vp, C.c_int32, C.c_int32, C.c_int32, C.c_uint64, _vp,
+         C.c_size_t, _vp],
+    ),
 }
 
 _lib = None

@@ -1,0 +1,96 @@
+"""The attention function the reference leaves unwritten (attention/hira_attention.py:1-3
+only points at transformers' AttentionInterface).
+
+Calling convention of transformers' attention functions:
+
+    fn(module, query (B, H_q, L_q, D), key, value, attention_mask, dropout=0.0,
+       scaling=None, **kwargs) -> (attn_output (B, L_q, H_q, Dv), None)
+
+``key`` is what ``HiraCache.update`` returned in place of the key states: a ``CacheOutput``
+(cache/hira_cache.py:19-26 of the reference).
+
+* prefill (``prefill_keys`` present): ordinary causal attention over the prompt;
+* decode (L_q == 1): out[h] = softmax over {indexed keys with q_h.k >= tau_h} + {queued
+  keys} of scaling * q_h.k, times V -- one fused search + sparse-attention launch.
+
+The threshold comes from ``hira_threshold`` (tensor (B*H_q,) or scalar) or from
+``hira_topk`` (int: select exactly the k best indexed keys per head).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+import torch.nn.functional as F
+
+from hira_amd.cache.threshold_finder import exact_topk
+
+
+def _repeat_kv(x: torch.Tensor, n_rep: int) -> torch.Tensor:
+    if n_rep == 1:
+        return x
+    b, h, l, d = x.shape
+    return x[:, :, None].expand(b, h, n_rep, l, d).reshape(b, h * n_rep, l, d)
+
+
+def _dense(query, key, value, attention_mask, scaling, is_causal):
+    n_rep = query.shape[1] // key.shape[1]
+    out = F.scaled_dot_product_attention(
+        query, _repeat_kv(key, n_rep), _repeat_kv(value, n_rep),
+        attn_mask=attention_mask, scale=scaling,
+        is_causal=is_causal and attention_mask is None and query.shape[2] > 1)
+    return out.transpose(1, 2).contiguous()
+
+
+def index_thresholds(indexer, query: torch.Tensor, topk: int) -> torch.Tensor:
+    """(B*H_q,) thresholds that keep exactly the `topk` best indexed keys of every head."""
+    keys = indexer.keys_buf[:, : indexer.size[0]]  # (T, N_pad, D) slot order
+    q = query.reshape(-1, query.shape[-1])
+    t = indexer.num_trees
+    qg = q.reshape(t, -1, q.shape[-1]).float()
+    s = torch.einsum("tnd,tgd->tgn", keys.float(), qg)
+    s = s.masked_fill((indexer.perm[:, None, : indexer.size[0]] < 0), float("-inf"))
+    s = s.reshape(q.shape[0], -1)
+    k = max(1, min(int(topk), indexer.num_keys))
+    top = s.topk(min(k + 1, s.shape[-1]), dim=-1).values
+    if top.shape[-1] == k or k == indexer.num_keys:
+        return top[:, k - 1].contiguous()
+    return ((top[:, k - 1].double() + top[:, k].double()) * 0.5).float()
+
+
+def hira_attention_forward(module, query, key, value, attention_mask=None, dropout: float = 0.0,
+                           scaling: Optional[float] = None, hira_threshold=None,
+                           hira_topk: Optional[int] = None, **kwargs):
+    d = query.shape[-1]
+    if scaling is None:
+        scaling = getattr(module, "scaling", None) or d ** -0.5
+    if not hasattr(key, "indexer"):  # plain tensors: no cache in use
+        return _dense(query, key, value, attention_mask, scaling, True), None
+    cache = key
+    if cache.prefill_keys is not None:
+        return _dense(query, cache.prefill_keys, cache.prefill_values, attention_mask, scaling,
+                      True), None
+    if query.shape[2] != 1:
+        raise ValueError("sparse decode expects one query position per step")
+    indexer, searcher = cache.indexer, cache.searcher
+    b, h_q = query.shape[0], query.shape[1]
+    if hira_threshold is None:
+        hira_threshold = getattr(module, "hira_threshold", None)
+    if hira_threshold is None:
+        topk = hira_topk or getattr(module, "hira_topk", None) or max(1, indexer.num_keys // 100)
+        hira_threshold = index_thresholds(indexer, query, topk)
+    scale = torch.full((b * h_q,), float(scaling), dtype=torch.float32, device=query.device)
+    qk, qv = cache.queued_keys, cache.queued_values
+    out = searcher.search_attention(
+        query, hira_threshold, indexer, scaling=scale,
+        queue_keys=qk if qk is not None and qk.shape[-2] > 0 else None,
+        queue_values=qv if qv is not None and qv.shape[-2] > 0 else None)
+    return out.reshape(b, 1, h_q, -1).to(query.dtype), None
+
+
+def register_hira_attention(name: str = "hira") -> str:
+    """Make the function selectable as ``attn_implementation=name``."""
+    from transformers import AttentionInterface
+
+    AttentionInterface.register(name, hira_attention_forward)
+    return name

@@ -1,0 +1,190 @@
+"""HiraCache / HiraCacheLayer: HuggingFace cache objects that own one index per layer.
+
+Mirrors the reference's cache/hira_cache.py:19-249: the first ``update`` of a layer
+(prefill) builds the index and returns the prefill tensors untouched; later updates queue
+the new keys/values and fold the queue into the index every ``update_every`` tokens.
+``update`` returns ``(CacheOutput, None)``, as the reference does, and the attention
+function (attention/hira_attention.py) reads indexer, searcher and queue from it.
+
+Both spellings of the two methods whose name or signature changed between transformers
+releases are provided: ``get_max_cache_shape`` (reference, cache/hira_cache.py:167-168) /
+``get_max_length``, and ``get_mask_sizes(cache_position tensor | query_length int)``.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any
+
+import torch
+from transformers.cache_utils import Cache, CacheLayerMixin
+
+from hira_amd.cache.hira_config import DeviceMode, HiraConfig
+from hira_amd.indexer import HIPIndexer
+from hira_amd.searcher import HIPSearcher
+
+# names the reference binds in this module (tests patch them there)
+CUDAIndexer = HIPIndexer
+CUDASearcher = HIPSearcher
+
+
+@dataclass
+class CacheOutput:
+    queued_keys: torch.Tensor
+    queued_values: torch.Tensor
+    prefill_keys: torch.Tensor | None
+    prefill_values: torch.Tensor | None
+    indexer: Any
+    searcher: Any
+
+
+class HiraCacheLayer(CacheLayerMixin):
+    """One layer, all KV heads.  key_states / value_states: (B, H_kv, L, D)."""
+
+    def __init__(
+        self,
+        device_mode: str,
+        update_every: int,
+        indexer_kwargs: dict[str, Any],
+        searcher_kwargs: dict[str, Any],
+    ):
+        super().__init__()
+        self.device_mode = device_mode
+        self.update_every = update_every
+        self.indexer_kwargs = indexer_kwargs
+        self.searcher_kwargs = searcher_kwargs
+        if self.device_mode == DeviceMode.CUDA_ONLY:
+            # looked up at call time so that the module-level names can be replaced
+            import hira_amd.cache.hira_cache as me
+
+            self.indexer_cls = me.CUDAIndexer
+            self.searcher_cls = me.CUDASearcher
+        elif self.device_mode == DeviceMode.CPU_ONLY:
+            raise NotImplementedError(
+                "cpu_only is the reference's host path; this package is the MI355X path "
+                "(device_mode='cuda_only')")
+        else:
+            raise NotImplementedError(f"Device mode {self.device_mode} not supported yet")
+        self.indexed_len = 0
+        self.queued_len = 0
+
+    def _empty_queue(self):
+        return torch.empty((self.batch, self.H_kv, 0, self.dim), dtype=self.dtype,
+                           device=self.device)
+
+    def lazy_initialization(self, key_states, value_states):
+        self.dim = key_states.shape[-1]
+        self.H_kv = key_states.shape[-3]
+        self.batch = key_states.shape[0] if key_states.ndim == 4 else 1
+        self.dtype = key_states.dtype
+        self.device = key_states.device
+        self.indexer = self.indexer_cls(**self.indexer_kwargs)
+        self.searcher = self.searcher_cls(**self.searcher_kwargs)
+        self.queued_keys = self._empty_queue()
+        self.queued_values = self._empty_queue()
+        self.queued_len = 0
+        self.keys = None  # the index holds the keys
+        self.values = None
+        self.is_initialized = True
+
+    def update(self, key_states: torch.Tensor, value_states: torch.Tensor,
+               cache_kwargs: dict[str, Any] | None = None, *args, **kwargs):
+        if not self.is_initialized:
+            self.lazy_initialization(key_states, value_states)
+            self.indexer.build(key_states, value_states)
+            self.indexed_len = key_states.shape[-2]
+            return (
+                CacheOutput(
+                    queued_keys=self.queued_keys,
+                    queued_values=self.queued_values,
+                    prefill_keys=key_states,
+                    prefill_values=value_states,
+                    indexer=self.indexer,
+                    searcher=self.searcher,
+                ),
+                None,
+            )
+        self.queued_keys = torch.cat([self.queued_keys, key_states], dim=-2)
+        self.queued_values = torch.cat([self.queued_values, value_states], dim=-2)
+        self.queued_len += key_states.shape[-2]
+        if self.queued_len >= self.update_every:
+            self.update_index()
+        return (
+            CacheOutput(
+                queued_keys=self.queued_keys,
+                queued_values=self.queued_values,
+                prefill_keys=None,
+                prefill_values=None,
+                indexer=self.indexer,
+                searcher=self.searcher,
+            ),
+            None,
+        )
+
+    def update_index(self):
+        self.indexer.update(self.queued_keys, self.queued_values)
+        self.queued_keys = self._empty_queue()
+        self.queued_values = self._empty_queue()
+        self.indexed_len += self.queued_len
+        self.queued_len = 0
+
+    def get_mask_sizes(self, cache_position):
+        kv_offset = 0
+        query_length = (int(cache_position) if isinstance(cache_position, int)
+                        else cache_position.shape[0])
+        return self.get_seq_length() + query_length, kv_offset
+
+    def get_seq_length(self):
+        if not self.is_initialized:
+            return 0
+        return self.indexed_len + self.queued_len
+
+    def get_max_cache_shape(self):
+        return -1
+
+    def get_max_length(self):
+        return -1
+
+    def reset(self):
+        if self.is_initialized:
+            self.indexer = self.indexer_cls(**self.indexer_kwargs)
+            self.queued_keys = self._empty_queue()
+            self.queued_values = self._empty_queue()
+            self.queued_len = 0
+            self.indexed_len = 0
+            self.is_initialized = False
+        if hasattr(self, "cumulative_length"):
+            self.cumulative_length = 0
+
+
+class HiraCache(Cache):
+    """HuggingFace ``Cache`` whose layers are HiraCacheLayer (cache/hira_cache.py:187-249)."""
+
+    def __init__(self, cache_config, hira_config: HiraConfig):
+        self.device_mode = hira_config.device_mode
+        self.update_every = hira_config.update_every
+        config = cache_config.get_text_config(decoder=True)
+        layer_types = getattr(config, "layer_types", None)
+        if layer_types is None:
+            if getattr(config, "sliding_window", None) is not None:
+                layer_types = ["sliding_attention" for _ in range(config.num_hidden_layers)]
+            elif getattr(config, "attention_chunk_size", None) is not None:
+                layer_types = ["chunked_attention" for _ in range(config.num_hidden_layers)]
+            else:
+                layer_types = ["full_attention" for _ in range(config.num_hidden_layers)]
+        if hasattr(config, "num_kv_shared_layers"):
+            layer_types = layer_types[: -config.num_kv_shared_layers]
+        layers = [
+            HiraCacheLayer(
+                device_mode=self.device_mode,
+                update_every=self.update_every,
+                indexer_kwargs=hira_config.get_indexer_kwargs(),
+                searcher_kwargs=hira_config.get_searcher_kwargs(),
+            )
+            for _ in layer_types
+        ]
+        super().__init__(layers=layers, offloading=False)
+
+    def update(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int,
+               cache_kwargs: dict[str, Any] | None = None, *args, **kwargs):
+        cache_output, _ = self.layers[layer_idx].update(key_states, value_states, cache_kwargs)
+        return cache_output, None

@@ -438,7 +438,10 @@ __global__ void k_compose_order(const int32_t* order_parent, int size_parent, in
     const int s = i / bf, j = i % bf;
     int node = order_parent ? order_parent[(size_t)t * size_parent + s] : (s < K_parent ? s : -1);
     int v = -1;
-    if (node >= 0) v = slots[((size_t)t * K_parent + node) * bf + j];
+    if (slots == nullptr)
+        v = node;  // bf == 1: plain copy / identity
+    else if (node >= 0)
+        v = slots[((size_t)t * K_parent + node) * bf + j];
     order_child[(size_t)t * size_parent * bf + i] = v;
 }
 

@@ -69,6 +69,7 @@ class HIPIndexer(BaseIndexer):
         *,
         seed: int = 1234,
         capacity: Optional[int] = None,
+        pack_rounds: int = 8,
         device: str = "cuda",
     ):
         if isinstance(num_levels, HIPIndexer.DEPTH):
@@ -84,6 +85,7 @@ class HIPIndexer(BaseIndexer):
         self.verbose = verbose
         self.pad_value = pad_value
         self.seed = int(seed)
+        self.pack_rounds = int(pack_rounds)
         self.capacity = capacity  # key slots to reserve per tree (room for appends)
         self.device = torch.device(device)
 
@@ -251,7 +253,36 @@ class HIPIndexer(BaseIndexer):
     # ------------------------------------------------------------------ build / update
     @torch.no_grad()
     def build(self, keys: torch.Tensor, values: Optional[torch.Tensor] = None):
-        raise NotImplementedError("HIP build is not wired yet")
+        """keys (1, H, L, D) (or (B, H, L, D): one tree per sequence and KV head), values
+        (1, H, L, Dv) aligned with the keys or None.  Runs on the current stream and
+        returns self without waiting (indexer/cuda.py:56-108)."""
+        if keys.ndim != 4:
+            raise ValueError(f"keys must be (B,H,L,D), got {tuple(keys.shape)}")
+        if values is not None and values.shape[:3] != keys.shape[:3]:
+            raise ValueError("values must be aligned with keys: (B,H,L,Dv)")
+        b, h, n, d = keys.shape
+        dtype = keys.dtype if keys.dtype in _DTYPES else torch.float32
+        vdim = 0 if values is None else int(values.shape[-1])
+        self._allocate(b, h, n, d, vdim, dtype)
+        kin = keys.to(device=self.device, dtype=dtype).reshape(b * h, n, d).contiguous()
+        vin = None
+        if values is not None:
+            vin = values.to(device=self.device, dtype=dtype).reshape(b * h, n, vdim).contiguous()
+        lib = _lib.lib()
+        tree = self.tree_struct()
+        need = lib.hira_build_workspace_bytes(C.byref(tree), n)
+        if need == 0:
+            _lib.check(-1)
+        ws = torch.empty(need, dtype=torch.uint8, device=self.device)
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        rc = lib.hira_build(C.byref(tree), kin.data_ptr(), None if vin is None else vin.data_ptr(),
+                            n, self.max_iterations, self.pack_rounds, self.seed, ws.data_ptr(),
+                            need, stream)
+        _lib.check(rc)
+        self.num_keys = n
+        if self.verbose:
+            print(f"built {self.num_trees} trees, level sizes {self.size}")
+        return self
 
     @torch.no_grad()
     def update(self, new_keys: torch.Tensor, new_values: Optional[torch.Tensor] = None):

@@ -232,3 +232,47 @@ class HIPSearcher(BaseSearcher):
         self._run(indexer, qs, so, queue)
         del keep
         return out
+
+    def plan_attention(self, indexer, num_q_heads: int, scaling=None, q_head_to_kv=None,
+                       stats: Optional[torch.Tensor] = None) -> "DecodePlan":
+        """Pre-resolve everything that does not change between decode steps (head map,
+        scaling, workspace) so that a step is one library call on ready device tensors."""
+        return DecodePlan(self, indexer, num_q_heads, scaling, q_head_to_kv, stats)
+
+
+class DecodePlan:
+    """One fused search + attention call per ``run``: ``query`` (H_q, D) in the tree dtype,
+    ``threshold`` (H_q,) fp32 and ``out`` (H_q, Dv) fp32 must be contiguous device tensors."""
+
+    def __init__(self, searcher: HIPSearcher, indexer, num_q_heads: int, scaling, q_head_to_kv,
+                 stats):
+        self.indexer = indexer
+        self.lib = _lib.lib()
+        dev = indexer.device
+        self.scaling = searcher._coerce_scaling(scaling, num_q_heads, dev)
+        off, heads, gmax = searcher._head_map(num_q_heads, indexer, q_head_to_kv)
+        self._keep = (off, heads, stats)
+        self.query = _lib.HiraQuery(num_q_heads, None, None, self.scaling.data_ptr(),
+                                    off.data_ptr(), heads.data_ptr(), gmax)
+        self.out = _lib.HiraSearchOut()
+        self.out.stats = None if stats is None else stats.data_ptr()
+        self.launch = searcher.launch
+        self.tree = indexer.tree_struct()
+        fake_q = _lib.HiraQuery(num_q_heads, 1, 1, 1, 1, 1, gmax)  # sizes only
+        self.ws_bytes = self.lib.hira_search_workspace_bytes(
+            C.byref(self.tree), C.byref(fake_q), None, C.byref(self.launch))
+        self.ws = torch.empty(max(self.ws_bytes, 1), dtype=torch.uint8, device=dev)
+        self._refs = (C.byref(self.tree), C.byref(self.query), C.byref(self.out),
+                      C.byref(self.launch))
+
+    def run(self, query: torch.Tensor, threshold: torch.Tensor, out: torch.Tensor,
+            stream: Optional[int] = None) -> None:
+        self.query.q = query.data_ptr()
+        self.query.tau = threshold.data_ptr()
+        self.out.attn_out = out.data_ptr()
+        if stream is None:
+            stream = torch.cuda.current_stream(self.indexer.device).cuda_stream
+        t, q, o, l = self._refs
+        rc = self.lib.hira_search(t, q, None, o, l, self.ws.data_ptr(), self.ws_bytes, stream)
+        if rc:
+            _lib.check(rc)

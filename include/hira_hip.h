@@ -138,6 +138,27 @@ int hira_search(const HiraTree* tree, const HiraQuery* query, const HiraQueue* q
                 const HiraSearchOut* out, const HiraLaunch* launch, void* workspace,
                 size_t workspace_bytes, void* stream);
 
+/*
+ * Index build.  Replaces CUDAIndexer.build and its helpers (indexer/cuda.py:56-108,
+ * 200-336, 338-538: centroid choice, nearest-centroid assignment, closest-first packing into
+ * blocks of bf, layout of the levels, radii from the layout, indexer/cuda.py:114-198) and,
+ * for the Lloyd rounds, CPUIndexer._sample_centroids_faiss (indexer/cpu.py:223-261).
+ *   tree       buffers for the result; tree->size[] must be the padded layout of n keys:
+ *              size[L-1] = K_{L-1}, size[l] = size[l+1]*bf with K_0 = n,
+ *              K_l = ceil(K_{l-1}/bf); cap[l] >= size[l].  Slots beyond size[] are not
+ *              touched.
+ *   keys_in    (T, n, D), values_in (T, n, Dv) or NULL, in insertion order, tree dtype.
+ *   niter      Lloyd rounds per level (the reference's max_iterations); 0 = sampled points
+ *              as centroids, as the reference's GPU build does.
+ *   pack_rounds rounds of "propose to the nearest centroid with room" before leftovers
+ *              are placed in order; >= 1.
+ *   seed       picks the initial centroids.
+ */
+size_t hira_build_workspace_bytes(const HiraTree* tree, int32_t n);
+int hira_build(const HiraTree* tree, const void* keys_in, const void* values_in, int32_t n,
+               int32_t niter, int32_t pack_rounds, uint64_t seed, void* workspace,
+               size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

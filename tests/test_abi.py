@@ -1,0 +1,61 @@
+"""The C-ABI library loads and exports every symbol include/hira_hip.h declares (no
+compute calls: this runs without a GPU)."""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+from hira_amd import _lib
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+def _declared_symbols():
+    text = (ROOT / "include" / "hira_hip.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(hira_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_symbols()
+    assert "hira_search" in names and "hira_build" in names
+    lib = ctypes.CDLL(str(_lib.LIB_PATH))
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in hira_hip.h but not exported"
+    assert set(names) == set(_lib.SYMBOLS), "binding table and header disagree"
+
+
+def test_abi_version_and_error_text():
+    lib = _lib.lib()
+    assert lib.hira_abi_version() == _lib.HIRA_ABI_VERSION
+    assert isinstance(lib.hira_last_error(), bytes)
+
+
+def test_argument_validation_needs_no_gpu():
+    """Bad descriptors are rejected before anything is launched."""
+    lib = _lib.lib()
+    t = _lib.HiraTree()
+    t.num_trees, t.num_levels, t.bf, t.dim, t.dtype = 1, 2, 99, 64, _lib.HIRA_F32
+    assert lib.hira_build_workspace_bytes(ctypes.byref(t), 100) == 0
+    assert b"branching factor" in lib.hira_last_error()
+    rc = lib.hira_build(ctypes.byref(t), None, None, 100, 1, 4, 0, None, 0, None)
+    assert rc == -1
+    with pytest.raises(ValueError):
+        _lib.check(rc)
+    t.bf, t.dim = 8, 6  # rows not a multiple of 16 bytes
+    assert lib.hira_build_workspace_bytes(ctypes.byref(t), 100) == 0
+    t.dim = 64
+    t.size[0], t.size[1], t.cap[0], t.cap[1] = 104, 13, 104, 13
+    assert lib.hira_build_workspace_bytes(ctypes.byref(t), 100) > 0
+    t.size[1] = 12  # not the padded layout of 100 keys
+    assert lib.hira_build_workspace_bytes(ctypes.byref(t), 100) == 0
+
+
+def test_struct_layout_matches_header():
+    """ctypes mirrors of the header structs: field order and sizes."""
+    assert ctypes.sizeof(_lib.HiraTree) == 6 * 4 + 2 * 8 * 4 + 3 * 8 + 3 * 8 * 8
+    assert ctypes.sizeof(_lib.HiraQueue) == 24
+    assert ctypes.sizeof(_lib.HiraLaunch) == 12
+    assert _lib.HiraQuery.max_group.offset == 48
+    assert _lib.HiraSearchOut.attn_out.offset == 56

@@ -1,0 +1,146 @@
+"""Host-side logic that needs no GPU: layout sizes, head maps, input coercion, config,
+threshold rules, synthetic workloads."""
+import numpy as np
+import pytest
+import torch
+
+from hira_amd import synth
+from hira_amd.cache import hira_config, threshold_finder
+from hira_amd.indexer.hip import HIPIndexer, level_sizes
+from hira_amd.searcher.hip import HIPSearcher
+from oracle import hira_oracle as ho
+
+
+def test_level_sizes_match_the_benchmark_shapes():
+    assert level_sizes(4096, 16, 2) == [4096, 256]
+    assert level_sizes(8192, 32, 3) == [8192, 256, 8]
+    assert level_sizes(32768, 32, 3) == [32768, 1024, 32]
+    assert level_sizes(131072, 32, 4) == [131072, 4096, 128, 4]
+    assert level_sizes(203, 4, 4) == [256, 64, 16, 4]
+    assert level_sizes(20, 32, 3) == [1024, 32, 1]
+    assert level_sizes(100, 1, 2) == [100, 100]
+    for n, bf, nl in [(203, 4, 4), (769, 8, 3), (5, 64, 2), (4096, 16, 2)]:
+        assert level_sizes(n, bf, nl) == ho.fixed_fanout_sizes(n, bf, nl)
+
+
+class _FakeIndexer:
+    def __init__(self, batch, heads):
+        self.batch, self.num_heads, self.num_trees = batch, heads, batch * heads
+        self.device = torch.device("cpu")
+
+
+def test_default_head_map_is_gqa_grouping():
+    off, heads, gmax = HIPSearcher()._head_map(32, _FakeIndexer(1, 8), None)
+    assert gmax == 4 and off.tolist() == list(range(0, 33, 4))
+    assert heads.tolist() == list(range(32))
+    # two sequences of 4 query / 2 KV heads: tree = b*H_kv + h // 2
+    off, heads, gmax = HIPSearcher()._head_map(8, _FakeIndexer(2, 2), None)
+    assert off.tolist() == [0, 2, 4, 6, 8] and heads.tolist() == list(range(8))
+
+
+def test_explicit_head_map_and_its_errors():
+    se = HIPSearcher()
+    off, heads, gmax = se._head_map(4, _FakeIndexer(1, 2), torch.tensor([1, 0, 1, 0]))
+    assert off.tolist() == [0, 2, 4] and heads.tolist() == [1, 3, 0, 2] and gmax == 2
+    with pytest.raises(ValueError):
+        se._head_map(4, _FakeIndexer(1, 2), torch.tensor([0, 1, 2, 0]))  # out of range
+    with pytest.raises(ValueError):
+        se._head_map(4, _FakeIndexer(1, 2), torch.tensor([0, 1]))        # wrong length
+    with pytest.raises(TypeError):
+        se._head_map(4, _FakeIndexer(1, 2), [0, 1, 0, 1])
+    with pytest.raises(ValueError):
+        se._head_map(3, _FakeIndexer(1, 2), None)                        # 3 heads over 2 trees
+
+
+def test_input_coercion_errors_follow_the_reference_wrappers():
+    """kernels/triton_search_wrappers.py:9-110 of the reference."""
+    se = HIPSearcher
+    assert se._coerce_query(torch.zeros(1, 4, 1, 16), 16).shape == (4, 16)
+    assert se._coerce_query(torch.zeros(3, 4, 1, 16), 16).shape == (12, 16)
+    with pytest.raises(TypeError):
+        se._coerce_query([[0.0]], 1)
+    with pytest.raises(ValueError):
+        se._coerce_query(torch.zeros(1, 4, 2, 16), 16)
+    with pytest.raises(ValueError):
+        se._coerce_query(torch.zeros(4, 8), 16)
+    with pytest.raises(ValueError):
+        se._coerce_query(torch.zeros(16), 16)
+    assert se._coerce_threshold(0.5, 3, "cpu").tolist() == [0.5] * 3
+    assert se._coerce_threshold(torch.tensor(2.0), 2, "cpu").tolist() == [2.0, 2.0]
+    with pytest.raises(ValueError):
+        se._coerce_threshold(torch.zeros(2), 3, "cpu")
+    assert se._coerce_scaling(None, 2, "cpu").tolist() == [1.0, 1.0]
+    with pytest.raises(ValueError):
+        se._coerce_scaling(torch.ones(5), 2, "cpu")
+    with pytest.raises(TypeError):
+        se._coerce_scaling(1.0, 2, "cpu")
+    with pytest.raises(ValueError):
+        HIPSearcher(index_space="token")
+
+
+def test_indexer_constructor_contract():
+    idx = HIPIndexer(num_levels=3, max_iterations=2, branching_factor=8)
+    assert idx.depth == HIPIndexer.DEPTH.THREE_LEVELS and idx.children is None
+    assert HIPIndexer(HIPIndexer.DEPTH.TWO_LEVELS, 1, 4).num_levels == 2
+    assert HIPIndexer(5, 1, 4).depth == 5  # deeper than the reference's enum goes
+    with pytest.raises(ValueError):
+        idx.tree_struct()  # not built
+
+
+def test_config_kwargs_and_loaders(tmp_path):
+    """cache/hira_config.py:35-46 of the reference + the loaders it leaves unwritten."""
+    cfg = hira_config.HiraConfig(device_mode=hira_config.DeviceMode.CUDA_ONLY, num_levels=3,
+                                 max_iterations=2, branching_factor=32)
+    assert cfg.get_indexer_kwargs() == {"num_levels": 3, "max_iterations": 2,
+                                        "branching_factor": 32}
+    assert cfg.get_searcher_kwargs() == {"block_c": 32}
+    cpu = hira_config.HiraConfig(device_mode=hira_config.DeviceMode.CPU_ONLY)
+    assert cpu.get_searcher_kwargs() == {"chunk_size": 8192}
+    HIPIndexer(**cfg.get_indexer_kwargs())
+    HIPSearcher(**cfg.get_searcher_kwargs())
+    d = hira_config.HiraConfig.from_dict({"num_levels": 4, "update_every": 64})
+    assert d.num_levels == 4 and d.update_every == 64 and d.branching_factor == 10
+    with pytest.raises(ValueError):
+        hira_config.HiraConfig.from_dict({"cuda_memory_limit": 1})
+    p = tmp_path / "c.yml"
+    p.write_text("device_mode: cuda_only\nnum_levels: 3\nbranching_factor: 16\n")
+    y = hira_config.HiraConfig.from_yaml(str(p))
+    assert (y.device_mode, y.num_levels, y.branching_factor) == ("cuda_only", 3, 16)
+
+
+def test_threshold_rules():
+    g = torch.Generator().manual_seed(0)
+    keys = torch.randn((2, 500, 16), generator=g)
+    q = torch.randn((4, 16), generator=g)
+    s = torch.einsum("hnd,hd->hn", keys.repeat_interleave(2, 0), q)
+    t = threshold_finder.exact_topk(keys, q, 25)
+    assert ((s >= t[:, None]).sum(1) == 25).all()
+    t2 = threshold_finder.exact_topk(keys, q.view(1, 4, 1, 16), 25, midpoint=False)
+    assert torch.equal(t2, s.topk(25, dim=1).values[:, -1])
+    assert torch.allclose(threshold_finder.sample_max(keys, q), s.max(1).values)
+    assert torch.allclose(threshold_finder.sample_mean_topk(keys, q, 10),
+                          s.topk(10, dim=1).values.mean(1))
+    m = torch.tensor([1, 0, 1, 0])
+    s2 = torch.einsum("hnd,hd->hn", keys[m], q)
+    assert torch.allclose(threshold_finder.sample_max(keys, q, m), s2.max(1).values)
+    assert set(threshold_finder.THRESHOLD_METHODS) >= {"sample_max", "sample_mean_topk"}
+
+
+def test_synthetic_workloads_are_seeded_and_shaped():
+    w = synth.WORKLOADS[0]
+    k1, v1 = synth.make_kv(w)
+    k2, _ = synth.make_kv(w)
+    assert k1.shape == (1, 1, 4096, 128) and k1.dtype == torch.float32 and torch.equal(k1, k2)
+    q = synth.make_queries(w, k1, 3)
+    assert q.shape == (3, 1, 1, 128)
+    w2 = synth.WORKLOADS[2]
+    d = synth.head_dist(w2, 0, 3)
+    assert d.massive.numel() == 8
+    k, _ = synth.make_kv(w2, n=256)
+    assert k.dtype == torch.bfloat16 and k.shape == (1, 8, 256, 128)
+    big = k[0, 3].float().abs().mean(0)
+    others = torch.ones(128, dtype=torch.bool)
+    others[d.massive] = False
+    assert big[d.massive].min() > 3 * big[others].mean()  # the 8 boosted channels stand out
+    fr = synth.select_fractions(synth.WORKLOADS[3])
+    assert fr.shape == (16,) and 0.005 <= float(fr.min()) and float(fr.max()) <= 0.05
