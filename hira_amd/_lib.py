@@ -15,6 +15,7 @@ LIB_PATH = CSRC / "libhira_hip.so"
 
 HIRA_MAX_LEVELS = 8
 HIRA_F32, HIRA_BF16 = 0, 1
+HIRA_ROW_MAJOR, HIRA_TILE16 = 0, 1
 HIRA_ABI_VERSION = 1
 
 _vp = C.c_void_p
@@ -28,6 +29,8 @@ class HiraTree(C.Structure):
         ("dim", C.c_int32),
         ("vdim", C.c_int32),
         ("dtype", C.c_int32),
+        ("layout", C.c_int32),
+        ("reserved_", C.c_int32),
         ("size", C.c_int32 * HIRA_MAX_LEVELS),
         ("cap", C.c_int32 * HIRA_MAX_LEVELS),
         ("keys", _vp),

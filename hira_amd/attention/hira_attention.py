@@ -44,7 +44,7 @@ def _dense(query, key, value, attention_mask, scaling, is_causal):
 
 def index_thresholds(indexer, query: torch.Tensor, topk: int) -> torch.Tensor:
     """(B*H_q,) thresholds that keep exactly the `topk` best indexed keys of every head."""
-    keys = indexer.keys_buf[:, : indexer.size[0]]  # (T, N_pad, D) slot order
+    keys = indexer.keys_rowmajor()  # (T, N_pad, D) slot order
     q = query.reshape(-1, query.shape[-1])
     t = indexer.num_trees
     qg = q.reshape(t, -1, q.shape[-1]).float()

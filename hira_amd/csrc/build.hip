@@ -18,7 +18,7 @@
 // layout: r_p = max over children (||c_child - c_p|| + r_child), the bound of
 // indexer/cpu.py:286-309 / indexer/cuda.py:114-198, against the ROUNDED centres and
 // nudged up by a few ulp so that rounding never makes a ball too small.
-#include "common.hip.h"
+#include "search.h"
 
 namespace hira {
 
@@ -449,7 +449,7 @@ __global__ void k_compose_order(const int32_t* order_parent, int size_parent, in
 // per element.  perm_out != NULL: also writes perm.
 template <typename T>
 __global__ void k_gather_rows(const void* src, size_t src_tree_stride, const int32_t* order,
-                              int size, int D, void* dst, size_t dst_tree_stride,
+                              int size, int D, void* dst, size_t dst_tree_stride, int dst_layout,
                               int32_t* perm_out, size_t perm_tree_stride) {
     const int t = blockIdx.y;
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -458,7 +458,7 @@ __global__ void k_gather_rows(const void* src, size_t src_tree_stride, const int
     const int o = order[(size_t)t * size + s];
     float v = 0.0f;
     if (o >= 0) v = load_elem<T>(src, ((size_t)t * src_tree_stride + o) * D + j);
-    store_elem<T>(dst, ((size_t)t * dst_tree_stride + s) * D + j, v);
+    store_elem<T>(dst, (size_t)t * dst_tree_stride * D + elem_index(dst_layout, D, (size_t)s, j), v);
     if (perm_out && j == 0) perm_out[(size_t)t * perm_tree_stride + s] = o;
 }
 
@@ -470,7 +470,7 @@ __global__ __launch_bounds__(64) void k_radii(const void* child, size_t child_tr
                                               size_t child_radii_stride,
                                               const int32_t* child_order, int size_child,
                                               const void* centers, size_t center_tree_stride,
-                                              int size, int bf, int D, float* radii,
+                                              int size, int bf, int D, int layout, float* radii,
                                               int32_t* counts, size_t out_stride) {
     const int p = blockIdx.x, t = blockIdx.y;
     const int lane = threadIdx.x;
@@ -483,8 +483,9 @@ __global__ __launch_bounds__(64) void k_radii(const void* child, size_t child_tr
         ++c;
         float ss = 0.0f;
         for (int e = lane; e < D; e += 64) {
-            const float df = load_elem<T>(child, ((size_t)t * child_tree_stride + s) * D + e) -
-                             load_elem<T>(centers, ((size_t)t * center_tree_stride + p) * D + e);
+            const float df =
+                load_elem<T>(child, (size_t)t * child_tree_stride * D + elem_index(layout, D, (size_t)s, e)) -
+                load_elem<T>(centers, (size_t)t * center_tree_stride * D + elem_index(layout, D, (size_t)p, e));
             ss += df * df;
         }
         ss = group_sum<64>(ss);
@@ -687,18 +688,18 @@ static int build_impl(const HiraTree* t, const void* keys_in, const void* values
         const size_t tot = (size_t)t->size[0] * D;
         hipLaunchKernelGGL((k_gather_rows<T>), dim3((unsigned)((tot + 255) / 256), NT), dim3(256),
                            0, s, keys_in, (size_t)n, w.order[0], t->size[0], D, t->keys,
-                           (size_t)t->cap[0], t->perm, (size_t)t->cap[0]);
+                           (size_t)t->cap[0], t->layout, t->perm, (size_t)t->cap[0]);
         if (values_in && t->values) {
             const size_t totv = (size_t)t->size[0] * t->vdim;
             hipLaunchKernelGGL((k_gather_rows<T>), dim3((unsigned)((totv + 255) / 256), NT),
                                dim3(256), 0, s, values_in, (size_t)n, w.order[0], t->size[0],
-                               t->vdim, t->values, (size_t)t->cap[0], nullptr, (size_t)0);
+                               t->vdim, t->values, (size_t)t->cap[0], (int)HIRA_ROW_MAJOR, nullptr, (size_t)0);
         }
         for (int l = 1; l < L; ++l) {
             const size_t totc = (size_t)t->size[l] * D;
             hipLaunchKernelGGL((k_gather_rows<T>), dim3((unsigned)((totc + 255) / 256), NT),
                                dim3(256), 0, s, w.cent_t[l], (size_t)K[l], w.order[l], t->size[l], D,
-                               t->centers[l], (size_t)t->cap[l], nullptr, (size_t)0);
+                               t->centers[l], (size_t)t->cap[l], t->layout, nullptr, (size_t)0);
         }
     }
     // radii and counts, bottom-up
@@ -708,7 +709,7 @@ static int build_impl(const HiraTree* t, const void* keys_in, const void* values
         hipLaunchKernelGGL((k_radii<T>), dim3(t->size[l], NT), dim3(64), 0, s, child,
                            (size_t)t->cap[l - 1], crad, (size_t)t->cap[l - 1], w.order[l - 1],
                            t->size[l - 1], t->centers[l], (size_t)t->cap[l], t->size[l], bf, D,
-                           t->radii[l], t->counts[l], (size_t)t->cap[l]);
+                           t->layout, t->radii[l], t->counts[l], (size_t)t->cap[l]);
     }
     HIRA_CHECK_LAUNCH("build layout");
     return HIRA_OK;
@@ -725,6 +726,14 @@ static int check_build_args(const HiraTree* t, int n) {
     HIRA_CHECK_ARG(t->dim >= epl && t->dim % epl == 0 && t->dim <= 64 * epl,
                    "dim %d: rows must be a multiple of 16 bytes", t->dim);
     HIRA_CHECK_ARG(n >= 1, "need at least one key, got %d", n);
+    HIRA_CHECK_ARG(t->layout == HIRA_ROW_MAJOR || t->layout == HIRA_TILE16, "layout %d", t->layout);
+    if (t->layout == HIRA_TILE16) {
+        HIRA_CHECK_ARG(t->dtype == HIRA_BF16 && t->dim % 32 == 0,
+                       "the tiled layout needs bf16 rows of a multiple of 32 columns");
+        for (int l = 0; l < t->num_levels; ++l)
+            HIRA_CHECK_ARG(t->cap[l] % 16 == 0, "tiled layout: cap[%d]=%d not a multiple of 16", l,
+                           t->cap[l]);
+    }
     int K[HIRA_MAX_LEVELS];
     cluster_counts(n, t->bf, t->num_levels, K);
     // padded sizes the layout needs

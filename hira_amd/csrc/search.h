@@ -1,0 +1,91 @@
+// Kernel arguments and launch plan shared by the two search kernels (vector-ALU: any
+// dtype/row width/fan-out, row-major or tiled keys; MFMA: bf16, tiled keys).
+#pragma once
+
+#include "common.hip.h"
+
+namespace hira {
+
+constexpr int kPseudoBlock = 32;  // rows per block when there is no level-1 node (flat scan, queue)
+
+struct SearchParams {
+    // tree
+    const void* keys;
+    const void* values;
+    const int32_t* perm;
+    const void* centers[HIRA_MAX_LEVELS];
+    const float* radii[HIRA_MAX_LEVELS];
+    const int32_t* counts[HIRA_MAX_LEVELS];
+    int32_t size[HIRA_MAX_LEVELS];
+    int32_t cap[HIRA_MAX_LEVELS];
+    int32_t num_levels, bf, dim, vdim;
+    int32_t layout;  // HIRA_ROW_MAJOR or HIRA_TILE16 (keys and centers)
+    // queries
+    const void* q;
+    const float* tau;
+    const float* scaling;
+    const int32_t* tree_q_off;
+    const int32_t* tree_q_heads;
+    // queue (always row-major)
+    const void* queue_keys;
+    const void* queue_values;
+    int32_t queue_len, queue_cap;
+    // work split
+    int32_t nodes_per_wave;  // level-1 nodes (or pseudo blocks) per wave
+    int32_t tree_blocks;     // workgroups that walk the tree; the rest scan the queue
+    int32_t num_nodes;       // level-1 nodes (or pseudo blocks over the keys when L == 1)
+    int32_t num_queue_blocks;
+    // outputs
+    float* dense;
+    int64_t dense_stride;
+    int32_t dense_by_position;
+    int32_t* sel_index;
+    float* sel_score;
+    int32_t* sel_count;
+    int32_t sel_cap;
+    float* part_m;    // (H_q, P)
+    float* part_l;    // (H_q, P)
+    float* part_acc;  // (H_q, P, Dv)
+    int32_t num_parts;  // P = gridDim.x
+    int32_t gmax_state; // MFMA kernel: heads per pass its LDS state rows are sized for
+    unsigned long long* stats;
+};
+
+struct SearchPlan {
+    int kernel;       // 1 = vector-ALU, 2 = MFMA
+    int lpr;          // lanes per row (vector-ALU kernel)
+    int gmax;         // heads per pass
+    int threads;      // workgroup size
+    int nodes_per_wave;
+    int num_nodes, num_queue_blocks;
+    int tree_blocks, queue_blocks, head_chunks;
+    size_t smem;
+};
+
+// search_mfma.hip
+bool mfma_search_supported(const HiraTree* t, const HiraQueue* queue);
+int launch_search_mfma(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
+
+// Element index of (row, column j) inside one tree's (cap, D) matrix.
+//   row-major: row*D + j
+//   tiled (16 rows x 32 columns per tile, 16-byte chunks stored lane-major so that one
+//   wave-wide 128-bit load fetches a whole MFMA A-operand tile):
+//     chunk (tile = row/16, s = j/32, kb = (j%32)/8, i = row%16) at ((tile*KS + s)*64 + kb*16 + i)
+__device__ __host__ __forceinline__ size_t elem_index(int layout, int D, size_t row, int j) {
+    if (layout == HIRA_ROW_MAJOR) return row * (size_t)D + j;
+    const size_t ks = (size_t)D / 32;
+    const size_t chunk = ((row / 16) * ks + (size_t)(j / 32)) * 64 + (size_t)((j % 32) / 8) * 16 + row % 16;
+    return chunk * 8 + (size_t)(j % 8);
+}
+
+// 16-byte load of chunk `c` (8 bf16 or 4 fp32) of row `row` of one tree's matrix.
+template <typename T>
+__device__ __forceinline__ uint4 load_row_chunk(const void* base, int layout, int D,
+                                                size_t tree_row0, size_t row, int c) {
+    constexpr int EPL = Elem<T>::kPerChunk;
+    const T* p = reinterpret_cast<const T*>(base) + tree_row0 * (size_t)D;
+    if (layout == HIRA_ROW_MAJOR) return *reinterpret_cast<const uint4*>(p + row * (size_t)D + c * EPL);
+    return *reinterpret_cast<const uint4*>(p + elem_index(layout, D, row, c * EPL));
+}
+
+}  // namespace hira

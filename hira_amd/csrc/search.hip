@@ -15,53 +15,11 @@
 // Semantics (reference: kernels/cpp/torch_ext_v3.cpp:172-242, with the conservative
 // non-unit-query bound of searcher/cpu.py:61-63): keep a node when q.c + ||q||*r >= tau,
 // select a key when q.k >= tau.
-#include "common.hip.h"
+#include "search.h"
 
 namespace hira {
 
-constexpr int kUnroll = 8;        // row loads in flight per lane while scanning a block
-constexpr int kPseudoBlock = 32;  // rows per block when there is no level-1 node (flat scan, queue)
-
-struct SearchParams {
-    // tree
-    const void* keys;
-    const void* values;
-    const int32_t* perm;
-    const void* centers[HIRA_MAX_LEVELS];
-    const float* radii[HIRA_MAX_LEVELS];
-    const int32_t* counts[HIRA_MAX_LEVELS];
-    int32_t size[HIRA_MAX_LEVELS];
-    int32_t cap[HIRA_MAX_LEVELS];
-    int32_t num_levels, bf, dim, vdim;
-    // queries
-    const void* q;
-    const float* tau;
-    const float* scaling;
-    const int32_t* tree_q_off;
-    const int32_t* tree_q_heads;
-    // queue
-    const void* queue_keys;
-    const void* queue_values;
-    int32_t queue_len, queue_cap;
-    // work split
-    int32_t nodes_per_wave;  // level-1 nodes (or pseudo blocks) per wave
-    int32_t tree_blocks;     // workgroups that walk the tree; the rest scan the queue
-    int32_t num_nodes;       // level-1 nodes (or pseudo blocks over the keys when L == 1)
-    int32_t num_queue_blocks;
-    // outputs
-    float* dense;
-    int64_t dense_stride;
-    int32_t dense_by_position;
-    int32_t* sel_index;
-    float* sel_score;
-    int32_t* sel_count;
-    int32_t sel_cap;
-    float* part_m;    // (H_q, P)
-    float* part_l;    // (H_q, P)
-    float* part_acc;  // (H_q, P, Dv)
-    int32_t num_parts;  // P = gridDim.x
-    unsigned long long* stats;
-};
+constexpr int kUnroll = 8;  // row loads in flight per lane while scanning a block
 
 template <typename T, int LPR, int GMAX>
 __global__ __launch_bounds__(256) void search_kernel(const SearchParams p) {
@@ -135,6 +93,7 @@ __global__ __launch_bounds__(256) void search_kernel(const SearchParams p) {
     const size_t krow0 = (size_t)tree * (is_queue ? p.queue_cap : p.cap[0]);
     const int n_rows = is_queue ? p.queue_len : p.size[0];
     const int block_rows = real_nodes ? p.bf : kPseudoBlock;
+    const int klayout = is_queue ? HIRA_ROW_MAJOR : p.layout;
 
     for (int n0 = node_first; n0 < node_last; n0 += RPW) {
         // -------- gates: lane group rg owns node n0 + rg -----------------------------
@@ -157,7 +116,9 @@ __global__ __launch_bounds__(256) void search_kernel(const SearchParams p) {
                     arad[l - 2] = 0.0f;
                     if (l < L && node_ok) {
                         const size_t r = (size_t)tree * p.cap[l] + id;
-                        if (chunk_ok) araw[l - 2] = load_chunk<T>(p.centers[l], r * D, ch);
+                        if (chunk_ok)
+                            araw[l - 2] = load_row_chunk<T>(p.centers[l], p.layout, D,
+                                                            (size_t)tree * p.cap[l], id, ch);
                         arad[l - 2] = p.radii[l][r];
                     }
                 }
@@ -166,7 +127,7 @@ __global__ __launch_bounds__(256) void search_kernel(const SearchParams p) {
 #pragma unroll
             for (int l = HIRA_MAX_LEVELS - 1; l >= 2; --l) {
                 if (l < L) {
-                    if (p.stats && alive && ch == 0) {
+                    if (p.stats && alive && ch == 0 && arad[l - 2] > -INFINITY) {
                         // count the node once: by its first level-1 descendant
                         int span = 1;
                         for (int t = 1; t < l; ++t) span *= p.bf;
@@ -190,10 +151,12 @@ __global__ __launch_bounds__(256) void search_kernel(const SearchParams p) {
             if (alive) {
                 const size_t r = (size_t)tree * p.cap[1] + node;
                 uint4 raw = make_uint4(0, 0, 0, 0);
-                if (chunk_ok) raw = load_chunk<T>(p.centers[1], r * D, ch);
+                if (chunk_ok)
+                    raw = load_row_chunk<T>(p.centers[1], p.layout, D, (size_t)tree * p.cap[1],
+                                            node, ch);
                 const float rad = p.radii[1][r];
                 cnt = p.counts[1][r];
-                if (p.stats && ch == 0) st_nodes[1]++;
+                if (p.stats && ch == 0 && rad > -INFINITY) st_nodes[1]++;
                 float kf[EPL];
                 unpack<T>(raw, kf);
                 unsigned pass = 0;
@@ -229,7 +192,7 @@ __global__ __launch_bounds__(256) void search_kernel(const SearchParams p) {
                     const int row = i0 + u * RPW + rg;
                     raw[u] = make_uint4(0, 0, 0, 0);
                     if (row < bcnt && chunk_ok)
-                        raw[u] = load_chunk<T>(kbase, (krow0 + first + row) * D, ch);
+                        raw[u] = load_row_chunk<T>(kbase, klayout, D, krow0, first + row, ch);
                 }
 #pragma unroll
                 for (int u = 0; u < kUnroll; ++u) {
@@ -423,16 +386,6 @@ __global__ __launch_bounds__(256) void merge_kernel(const float* __restrict__ pa
 }
 
 // ---- host side ------------------------------------------------------------------------
-struct SearchPlan {
-    int lpr;          // lanes per row
-    int gmax;         // heads per pass
-    int threads;      // workgroup size
-    int nodes_per_wave;
-    int num_nodes, num_queue_blocks;
-    int tree_blocks, queue_blocks, head_chunks;
-    size_t smem;
-};
-
 static int round_pow2(int v) {
     int r = 1;
     while (r < v) r <<= 1;
@@ -472,7 +425,44 @@ static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* que
                        q->tree_q_heads,
                    "query arrays missing");
     HIRA_CHECK_ARG(q->max_group >= 1, "max_group %d", q->max_group);
+    HIRA_CHECK_ARG(t->layout == HIRA_ROW_MAJOR || t->layout == HIRA_TILE16, "layout %d",
+                   t->layout);
+    if (t->layout == HIRA_TILE16) {
+        HIRA_CHECK_ARG(t->dtype == HIRA_BF16 && t->dim % 32 == 0,
+                       "the tiled layout needs bf16 rows of a multiple of 32 columns");
+        for (int l = 0; l < t->num_levels; ++l)
+            HIRA_CHECK_ARG(t->cap[l] % 16 == 0, "tiled layout: cap[%d]=%d not a multiple of 16",
+                           l, t->cap[l]);
+    }
+    plan->num_queue_blocks = 0;
+    if (queue && queue->keys && queue->len > 0) {
+        HIRA_CHECK_ARG(queue->len <= queue->cap, "queue len %d > cap %d", queue->len,
+                       queue->cap);
+        plan->num_queue_blocks = (queue->len + kPseudoBlock - 1) / kPseudoBlock;
+    }
+    const int want = launch ? launch->kernel : 0;
+    HIRA_CHECK_ARG(want >= 0 && want <= 2, "kernel %d", want);
+    const bool mfma_ok = mfma_search_supported(t, queue);
+    HIRA_CHECK_ARG(want != 2 || mfma_ok,
+                   "the MFMA kernel needs bf16, tiled layout, >= 2 levels, fan-out 16/32/48/64, "
+                   "dim = vdim in {64,128,256} and no queue");
+    plan->kernel = (want == 2 || (want == 0 && mfma_ok)) ? 2 : 1;
     plan->lpr = lpr;
+    if (plan->kernel == 2) {
+        // one workgroup per tile of 16 level-1 nodes; heads in passes of 16
+        plan->gmax = q->max_group < 16 ? q->max_group : 16;
+        plan->head_chunks = (q->max_group + 15) / 16;
+        int threads = launch && launch->block_threads ? launch->block_threads : 512;
+        HIRA_CHECK_ARG(threads >= 64 && threads <= 512 && threads % 64 == 0,
+                       "block_threads %d must be a multiple of 64 up to 512", threads);
+        plan->threads = threads;
+        plan->nodes_per_wave = 0;
+        plan->num_nodes = t->size[1];
+        plan->tree_blocks = (t->size[1] + 15) / 16;
+        plan->queue_blocks = 0;
+        plan->smem = (size_t)(threads / 64) * plan->gmax * (t->dim + 2) * sizeof(float);
+        return HIRA_OK;
+    }
     plan->gmax = q->max_group <= 1 ? 1 : (q->max_group <= 4 ? 4 : 8);
     plan->head_chunks = (q->max_group + plan->gmax - 1) / plan->gmax;
     int threads = launch && launch->block_threads ? launch->block_threads : 256;
@@ -485,12 +475,6 @@ static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* que
     plan->nodes_per_wave = npw;
     plan->num_nodes = t->num_levels >= 2 ? t->size[1]
                                          : (t->size[0] + kPseudoBlock - 1) / kPseudoBlock;
-    plan->num_queue_blocks = 0;
-    if (queue && queue->keys && queue->len > 0) {
-        HIRA_CHECK_ARG(queue->len <= queue->cap, "queue len %d > cap %d", queue->len,
-                       queue->cap);
-        plan->num_queue_blocks = (queue->len + kPseudoBlock - 1) / kPseudoBlock;
-    }
     const int per_block = (threads / 64) * npw;
     plan->tree_blocks = (plan->num_nodes + per_block - 1) / per_block;
     plan->queue_blocks = (plan->num_queue_blocks + per_block - 1) / per_block;
@@ -585,6 +569,7 @@ extern "C" int hira_search(const HiraTree* tree, const HiraQuery* query, const H
     p.bf = tree->bf;
     p.dim = tree->dim;
     p.vdim = tree->vdim;
+    p.layout = tree->layout;
     p.q = query->q;
     p.tau = query->tau;
     p.scaling = query->scaling;
@@ -626,8 +611,12 @@ extern "C" int hira_search(const HiraTree* tree, const HiraQuery* query, const H
 
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     dim3 grid(P, tree->num_trees, plan.head_chunks);
-    rc = tree->dtype == HIRA_F32 ? dispatch_lpr<float>(plan, p, grid, s)
-                                 : dispatch_lpr<bf16_t>(plan, p, grid, s);
+    p.gmax_state = plan.gmax;
+    if (plan.kernel == 2)
+        rc = launch_search_mfma(plan, p, grid, s);
+    else
+        rc = tree->dtype == HIRA_F32 ? dispatch_lpr<float>(plan, p, grid, s)
+                                     : dispatch_lpr<bf16_t>(plan, p, grid, s);
     if (rc != HIRA_OK) return rc;
     HIRA_CHECK_LAUNCH("search kernel");
 

@@ -37,6 +37,22 @@ def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else C.c_void_p(t.data_ptr())
 
 
+def to_tiled(x: torch.Tensor) -> torch.Tensor:
+    """(T, R, D) row-major -> the same shape holding the HIRA_TILE16 arrangement: the
+    16-byte chunk with columns [32 s + 8 kb, +8) of row 16 t + i moves to chunk index
+    (t*(D/32) + s)*64 + kb*16 + i.  R must be a multiple of 16, D of 32."""
+    t, r, d = x.shape
+    v = x.reshape(t, r // 16, 16, d // 32, 4, 8).permute(0, 1, 3, 4, 2, 5)
+    return v.contiguous().reshape(t, r, d)
+
+
+def from_tiled(x: torch.Tensor) -> torch.Tensor:
+    """Inverse of to_tiled."""
+    t, r, d = x.shape
+    v = x.reshape(t, r // 16, d // 32, 4, 16, 8).permute(0, 1, 4, 2, 3, 5)
+    return v.contiguous().reshape(t, r, d)
+
+
 def level_sizes(n: int, bf: int, num_levels: int) -> List[int]:
     """Slots per level of the padded tree: K_1 = ceil(n/bf), K_l = ceil(K_{l-1}/bf); the
     root keeps K_root nodes and each lower level has bf slots per node of the level above
@@ -70,6 +86,7 @@ class HIPIndexer(BaseIndexer):
         seed: int = 1234,
         capacity: Optional[int] = None,
         pack_rounds: int = 8,
+        layout: str = "auto",
         device: str = "cuda",
     ):
         if isinstance(num_levels, HIPIndexer.DEPTH):
@@ -86,6 +103,10 @@ class HIPIndexer(BaseIndexer):
         self.pad_value = pad_value
         self.seed = int(seed)
         self.pack_rounds = int(pack_rounds)
+        if layout not in ("auto", "row_major", "tiled"):
+            raise ValueError("layout must be 'auto', 'row_major' or 'tiled'")
+        self.layout_request = layout
+        self.tiled = False  # keys / centers stored in the MFMA tile arrangement
         self.capacity = capacity  # key slots to reserve per tree (room for appends)
         self.device = torch.device(device)
 
@@ -114,14 +135,26 @@ class HIPIndexer(BaseIndexer):
         except ValueError:
             return self.num_levels
 
-    def _head_view(self, t: torch.Tensor, n: int) -> torch.Tensor:
-        """(T, cap, ...) -> (H, n, ...) for batch 1, (B, H, n, ...) otherwise."""
+    def _head_view(self, t: torch.Tensor, n: int, rows: bool = False) -> torch.Tensor:
+        """(T, cap, ...) -> (H, n, ...) for batch 1, (B, H, n, ...) otherwise.  `rows`: t is
+        a key / centre matrix; it is returned row-major (a copy when the index is tiled)."""
+        if rows and self.tiled:
+            t = from_tiled(t)
         v = t[:, :n]
         return v if self.batch == 1 else v.reshape(self.batch, self.num_heads, *v.shape[1:])
 
     @property
     def children(self):
-        return None if self.keys_buf is None else self._head_view(self.keys_buf, self.size[0])
+        return None if self.keys_buf is None else self._head_view(self.keys_buf, self.size[0], True)
+
+    def keys_rowmajor(self) -> torch.Tensor:
+        """(T, N_pad, D) keys in slot order, row-major (a copy when the index is tiled)."""
+        k = from_tiled(self.keys_buf) if self.tiled else self.keys_buf
+        return k[:, : self.size[0]]
+
+    def centers_rowmajor(self, l: int) -> torch.Tensor:
+        c = from_tiled(self.centers[l]) if self.tiled else self.centers[l]
+        return c[:, : self.size[l]]
 
     @property
     def values(self):
@@ -130,14 +163,14 @@ class HIPIndexer(BaseIndexer):
         v = self._head_view(self.values_buf, self.size[0])
         return v.unsqueeze(0) if self.batch == 1 else v
 
-    def _level(self, arr, l):
+    def _level(self, arr, l, rows: bool = False):
         if l >= self.num_levels or not arr or arr[l] is None:
             return None
-        return self._head_view(arr[l], self.size[l])
+        return self._head_view(arr[l], self.size[l], rows)
 
     @property
     def parents(self):
-        return self._level(self.centers, 1)
+        return self._level(self.centers, 1, True)
 
     @property
     def parent_radii(self):
@@ -145,7 +178,7 @@ class HIPIndexer(BaseIndexer):
 
     @property
     def grand_parents(self):
-        return self._level(self.centers, 2)
+        return self._level(self.centers, 2, True)
 
     @property
     def grand_parent_radii(self):
@@ -179,10 +212,15 @@ class HIPIndexer(BaseIndexer):
         self.size = level_sizes(n, bf, nl)
         want = max(n, int(self.capacity or 0))
         self.cap = level_sizes(want, bf, nl) if want > n else list(self.size)
-        if nl >= 2 and want > n:
-            # appended keys open new leaf blocks: leave room for one new block per key
-            extra = want - n
-            self.cap = level_sizes(n + extra * bf, bf, nl)
+        tile_ok = (dtype == torch.bfloat16 and dim % 32 == 0)
+        if self.layout_request == "tiled" and not tile_ok:
+            raise ValueError("the tiled layout needs bfloat16 keys with dim a multiple of 32")
+        self.tiled = tile_ok and (
+            self.layout_request == "tiled"
+            or (self.layout_request == "auto" and nl >= 2 and bf % 16 == 0
+                and dim in (64, 128, 256) and vdim in (0, dim)))
+        if self.tiled:
+            self.cap = [-(-c // 16) * 16 for c in self.cap]
         dev, t = self.device, self.num_trees
         self.keys_buf = torch.zeros((t, self.cap[0], dim), dtype=dtype, device=dev)
         self.values_buf = (
@@ -207,6 +245,7 @@ class HIPIndexer(BaseIndexer):
             t.bf = self.branching_factor
             t.dim, t.vdim = self.dim, self.vdim
             t.dtype = _DTYPES[self.dtype]
+            t.layout = _lib.HIRA_TILE16 if self.tiled else _lib.HIRA_ROW_MAJOR
             for l in range(self.num_levels):
                 t.size[l], t.cap[l] = self.size[l], self.cap[l]
             t.keys = self.keys_buf.data_ptr()
@@ -223,13 +262,14 @@ class HIPIndexer(BaseIndexer):
     @classmethod
     def from_layout(cls, *, bf: int, keys, perm, centers, radii, counts, values=None,
                     dtype: torch.dtype = torch.float32, batch: int = 1, device: str = "cuda",
-                    num_keys: Optional[int] = None, capacity: Optional[int] = None):
+                    num_keys: Optional[int] = None, capacity: Optional[int] = None,
+                    layout: str = "auto"):
         """Adopt a padded tree given as host arrays: keys (T, N_pad, D), perm (T, N_pad),
         and per level l >= 1 (index 0 is None) centers (T, K_l, D), radii (T, K_l), counts
         (T, K_l); values (T, N_pad, Dv) follow the key slots.  Used to restore a saved index
         and by tests that walk a tree built on the host."""
         nl = len(centers)
-        self = cls(nl, 1, bf, device=device, capacity=capacity)
+        self = cls(nl, 1, bf, device=device, capacity=capacity, layout=layout)
         keys = torch.as_tensor(keys)
         t, n_pad, d = keys.shape
         vdim = 0 if values is None else int(torch.as_tensor(values).shape[-1])
@@ -237,6 +277,8 @@ class HIPIndexer(BaseIndexer):
         if self.size[0] != n_pad:
             raise ValueError(f"keys have {n_pad} slots, layout needs {self.size[0]}")
         self.keys_buf[:, :n_pad] = keys.to(device=self.device, dtype=dtype)
+        if self.tiled:
+            self.keys_buf.copy_(to_tiled(self.keys_buf))
         if values is not None:
             self.values_buf[:, :n_pad] = torch.as_tensor(values).to(device=self.device,
                                                                     dtype=dtype)
@@ -245,6 +287,8 @@ class HIPIndexer(BaseIndexer):
         for l in range(1, nl):
             k = self.size[l]
             self.centers[l][:, :k] = torch.as_tensor(centers[l]).to(self.device, dtype)
+            if self.tiled:
+                self.centers[l].copy_(to_tiled(self.centers[l]))
             self.radii[l][:, :k] = torch.as_tensor(radii[l]).to(self.device, torch.float32)
             self.counts[l][:, :k] = torch.as_tensor(counts[l]).to(self.device, torch.int32)
         self.num_keys = int(num_keys if num_keys is not None else (perm[0] >= 0).sum().item())

@@ -36,6 +36,14 @@ extern "C" {
 
 enum { HIRA_F32 = 0, HIRA_BF16 = 1 };
 
+/* How the keys and the centers of every level are stored inside one tree's (cap, D)
+ * matrix.  HIRA_TILE16 (bf16 only, D a multiple of 32, every cap a multiple of 16): rows
+ * are grouped in tiles of 16, columns in steps of 32; the 16-byte chunk holding columns
+ * [32 s + 8 kb, +8) of row 16 tile + i sits at chunk index (tile*(D/32) + s)*64 + kb*16 + i,
+ * i.e. one wave-wide 128-bit load fetches a complete 16x32 MFMA operand tile from 1 KiB of
+ * contiguous memory.  Values, radii, counts and perm are never tiled. */
+enum { HIRA_ROW_MAJOR = 0, HIRA_TILE16 = 1 };
+
 enum {
     HIRA_OK = 0,
     HIRA_EINVAL = -1,   /* bad shape / dtype / null pointer: the message names it */
@@ -50,12 +58,14 @@ typedef struct HiraTree {
     int32_t dim;        /* key / query / center dim D; D*elem_size a multiple of 16 B */
     int32_t vdim;       /* value dim Dv (0 if there are no values) */
     int32_t dtype;
+    int32_t layout;     /* HIRA_ROW_MAJOR or HIRA_TILE16 */
+    int32_t reserved_;  /* keeps the arrays below 8-byte aligned; must be 0 */
     int32_t size[HIRA_MAX_LEVELS];
     int32_t cap[HIRA_MAX_LEVELS];
-    void* keys;                      /* (T, cap[0], D) */
+    void* keys;                      /* (T, cap[0], D), stored as `layout` says */
     void* values;                    /* (T, cap[0], Dv) or NULL */
     int32_t* perm;                   /* (T, cap[0]) */
-    void* centers[HIRA_MAX_LEVELS];  /* [l >= 1] (T, cap[l], D) */
+    void* centers[HIRA_MAX_LEVELS];  /* [l >= 1] (T, cap[l], D), stored as `layout` says */
     float* radii[HIRA_MAX_LEVELS];   /* [l >= 1] (T, cap[l]) */
     int32_t* counts[HIRA_MAX_LEVELS];/* [l >= 1] (T, cap[l]) */
 } HiraTree;

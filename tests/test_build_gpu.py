@@ -15,13 +15,13 @@ pytestmark = pytest.mark.gpu
 
 def _download(idx):
     n0 = idx.size[0]
-    out = dict(keys=idx.keys_buf[:, :n0].float().cpu().numpy(),
+    out = dict(keys=idx.keys_rowmajor().float().cpu().numpy(),
                perm=idx.perm[:, :n0].cpu().numpy().astype(np.int64),
                values=None if idx.values_buf is None else idx.values_buf[:, :n0].float().cpu().numpy(),
                centers=[None], radii=[None], counts=[None])
     for l in range(1, idx.num_levels):
         k = idx.size[l]
-        out["centers"].append(idx.centers[l][:, :k].float().cpu().numpy())
+        out["centers"].append(idx.centers_rowmajor(l).float().cpu().numpy())
         out["radii"].append(idx.radii[l][:, :k].cpu().numpy())
         out["counts"].append(idx.counts[l][:, :k].cpu().numpy())
     return out
@@ -80,6 +80,8 @@ BUILD_CASES = [
     (2, 20, 32, 32, 3, torch.float32, 1),      # fewer keys than one block
     (1, 500, 256, 16, 2, torch.bfloat16, 1),
     (8, 8192, 128, 32, 3, torch.bfloat16, 1),
+    (2, 1000, 64, 16, 3, torch.bfloat16, 1),   # tiled layout, partial tiles at every level
+    (1, 3000, 256, 48, 2, torch.bfloat16, 1),
 ]
 
 
@@ -118,6 +120,7 @@ def test_build_is_reproducible_and_seed_dependent(gpu_device):
     b = HIPIndexer(3, 2, 8, seed=5).build(keys)
     c = HIPIndexer(3, 2, 8, seed=6).build(keys)
     torch.cuda.synchronize()
+    assert not a.tiled
     assert torch.equal(a.perm, b.perm) and torch.equal(a.centers[2], b.centers[2])
     assert torch.equal(a.radii[1], b.radii[1])
     assert not torch.equal(a.perm, c.perm)
@@ -131,6 +134,27 @@ def test_lloyd_rounds_tighten_the_balls(gpu_device):
     r0 = HIPIndexer(2, 0, 32).build(keys).radii[1].sum().item()
     r5 = HIPIndexer(2, 5, 32).build(keys).radii[1].sum().item()
     assert r5 < r0
+
+
+def test_tiled_and_row_major_builds_hold_the_same_tree(gpu_device):
+    """The tile arrangement only moves 16-byte chunks around: same tree, same answers."""
+    from hira_amd.indexer.hip import HIPIndexer, from_tiled, to_tiled
+
+    keys = torch.from_numpy(bf16_round(clustered_keys(2, 2000, 128, seed=4)))[None].to(torch.bfloat16)
+    a = HIPIndexer(3, 1, 32, layout="tiled").build(keys, keys.clone())
+    b = HIPIndexer(3, 1, 32, layout="row_major").build(keys, keys.clone())
+    torch.cuda.synchronize()
+    assert a.tiled and not b.tiled and a.cap[0] % 16 == 0
+    assert torch.equal(a.perm[:, : a.size[0]], b.perm[:, : b.size[0]])
+    assert torch.equal(a.keys_rowmajor(), b.keys_rowmajor())
+    assert torch.equal(a.children, b.children) and torch.equal(a.parents, b.parents)
+    for l in (1, 2):
+        assert torch.equal(a.centers_rowmajor(l), b.centers_rowmajor(l))
+        assert torch.equal(a.radii[l][:, : a.size[l]], b.radii[l][:, : b.size[l]])
+        assert torch.equal(a.counts[l][:, : a.size[l]], b.counts[l][:, : b.size[l]])
+    assert torch.equal(a.values, b.values)
+    x = torch.randn(3, 48, 96)
+    assert torch.equal(from_tiled(to_tiled(x)), x)
 
 
 def test_reference_attribute_views(gpu_device):

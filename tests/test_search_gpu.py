@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 
 
 def _setup(h_kv, h_q, n, d, bf, nl, dtype, seed, keep, clustered=True, q2kv=None, dv=None,
-           unit_q=True, niter=2):
+           unit_q=True, niter=2, layout="auto"):
     from hira_amd.indexer.hip import HIPIndexer
 
     keys = (clustered_keys if clustered else normalized_keys)(h_kv, n, d, seed)
@@ -35,7 +35,7 @@ def _setup(h_kv, h_q, n, d, bf, nl, dtype, seed, keep, clustered=True, q2kv=None
     th = midpoint_threshold(np.where(valid, s, -1e30), keep)
     idx = HIPIndexer.from_layout(bf=bf, keys=ff.keys, perm=ff.perm, centers=ff.centers,
                                  radii=ff.radii, counts=ff.counts, values=vslot, dtype=dtype,
-                                 num_keys=n)
+                                 num_keys=n, layout=layout)
     return dict(ff=ff, idx=idx, q=q, th=th, s=s, valid=valid, q2kv=q2kv, keys=keys, vals=vals,
                 vslot=vslot)
 
@@ -91,6 +91,74 @@ def test_selected_set_and_scores_match_oracle(case, gpu_device):
         assert np.array_equal(got, np.nonzero(m[h])[0])
         order = np.argsort(idx[h, :count[h]])
         np.testing.assert_allclose(score[h, :count[h]][order] * 0.125, out[h][m[h]], rtol=1e-6)
+
+
+MFMA_CASES = [
+    # h_kv, h_q, n, d, bf, levels, keep
+    (2, 8, 2048, 128, 32, 3, 41),
+    (1, 1, 1500, 128, 32, 2, 30),       # one head per tree, ragged last block
+    (2, 16, 1024, 128, 32, 3, 30),      # 8 heads per tree
+    (1, 16, 1100, 64, 16, 3, 33),       # 16 heads per tree, d = 64, fan-out 16
+    (1, 20, 900, 64, 16, 2, 27),        # 20 heads per tree: two passes of the head loop
+    (1, 4, 3000, 256, 48, 2, 60),       # d = 256, fan-out 48 (3 tiles per block)
+    (1, 4, 5000, 128, 64, 3, 50),       # fan-out 64
+    (2, 8, 40000, 128, 32, 4, 400),     # four levels
+]
+
+
+@pytest.mark.parametrize("case", MFMA_CASES, ids=[f"hkv{c[0]}_hq{c[1]}_n{c[2]}_d{c[3]}_bf{c[4]}_L{c[5]}"
+                                                    for c in MFMA_CASES])
+def test_mfma_kernel_matches_oracle_and_vector_kernel(case, gpu_device):
+    """bf16 trees in the tiled layout: the MFMA kernel (kernel=2), the vector-ALU kernel on
+    the same tiled tree (kernel=1) and the oracle select the same keys; attention agrees
+    with the fp64 oracle to 2e-3; the device counters of both kernels agree."""
+    from hira_amd import _lib
+    from hira_amd.searcher.hip import HIPSearcher
+
+    h_kv, h_q, n, d, bf, nl, keep = case
+    print(f"case {case}", flush=True)
+    c = _setup(h_kv, h_q, n, d, bf, nl, torch.bfloat16, seed=500 + n, keep=keep,
+               niter=1 if n > 5000 else 2, layout="tiled")
+    assert c["idx"].tiled
+    q, th = torch.from_numpy(c["q"]), torch.from_numpy(c["th"])
+    scale = d ** -0.5
+    sc = torch.full((h_q,), scale)
+    s = np.where(c["valid"], c["s"], -np.inf).astype(np.float32)
+    mask = (c["s"] >= c["th"][:, None]) & c["valid"]
+    ref = ho.attention(c["ff"].keys, c["vslot"], c["q"], sc.numpy(), mask, c["q2kv"])
+    stats = {}
+    for kernel in (2, 1):
+        se = HIPSearcher(kernel=kernel)
+        st = torch.zeros((h_kv, _lib.HIRA_MAX_LEVELS + 2), dtype=torch.int64, device="cuda")
+        out = se.search(q, th, c["idx"], scaling=sc, stats=st).cpu().numpy()
+        assert_same_selection(out != 0, s, c["th"])
+        m = out != 0
+        np.testing.assert_allclose(out[m], (c["s"] * scale)[m], rtol=2e-5, atol=1e-6)
+        pos = se.search(q, th, c["idx"], scaling=sc, index_space="position").cpu().numpy()
+        assert_same_selection(pos != 0, ho.scores(c["keys"], c["q"], c["q2kv"]), c["th"])
+        idx, score, count = (t.cpu().numpy() for t in se.search_compact(q, th, c["idx"], scaling=sc))
+        for h in range(h_q):
+            assert np.array_equal(np.sort(idx[h, :count[h]]), np.nonzero(m[h])[0])
+        att = se.search_attention(q, th, c["idx"], scaling=sc).cpu().numpy()
+        assert rel_err(att, ref) <= 2e-3, (kernel, rel_err(att, ref))
+        stats[kernel] = st.cpu().numpy()
+    if h_q // h_kv <= 8:  # both kernels cover the group in one pass: same counters
+        assert np.array_equal(stats[1], stats[2])
+    pairs = int(mask.sum())
+    assert stats[1][:, _lib.HIRA_MAX_LEVELS + 1].sum() == pairs == stats[2][:, _lib.HIRA_MAX_LEVELS + 1].sum()
+    # every key selected: dense attention through the sparse path
+    full = HIPSearcher(kernel=2).search_attention(q, -3e38, c["idx"], scaling=sc).cpu().numpy()
+    ref_full = ho.attention(c["ff"].keys, c["vslot"], c["q"], sc.numpy(), c["valid"], c["q2kv"])
+    assert rel_err(full, ref_full) <= 2e-3
+
+
+def test_mfma_kernel_is_refused_where_it_does_not_apply(gpu_device):
+    from hira_amd.searcher.hip import HIPSearcher
+
+    c = _setup(2, 4, 333, 16, 5, 3, torch.bfloat16, seed=9, keep=20)
+    assert not c["idx"].tiled
+    with pytest.raises(ValueError):
+        HIPSearcher(kernel=2).search(torch.from_numpy(c["q"]), torch.from_numpy(c["th"]), c["idx"])
 
 
 def test_explicit_non_monotone_head_map(gpu_device):
