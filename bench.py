@@ -52,6 +52,19 @@ def algorithmic_bytes(stats, w, num_levels, steps):
                                    selected_pairs_per_step=s[_lib.HIRA_MAX_LEVELS + 1])
 
 
+def measured_traffic(workload_name):
+    """HBM bytes per launch of the search kernel from the committed rocprofv3 --pmc summary
+    (FETCH_SIZE + WRITE_SIZE, each scaled by what the same counter reads for a kernel of
+    known traffic), or None when no summary for this workload is committed."""
+    f = ROOT / "profiles" / f"search_traffic_{workload_name}.json"
+    if not f.exists():
+        return None
+    try:
+        return json.loads(f.read_text())["hbm_bytes_per_launch"]
+    except Exception:  # noqa: BLE001
+        return None
+
+
 def cpu_baseline(w, index, queries, taus, scale, budget_s=20.0):
     """Reference CPU search (+ host softmax-V) on the same tree, first steps of the same
     queries, for about `budget_s` seconds of CPU work."""
@@ -65,9 +78,9 @@ def cpu_baseline(w, index, queries, taus, scale, budget_s=20.0):
     n0 = index.size[0]
     ff = ho.FixedFanoutTree(
         bf=index.branching_factor,
-        keys=index.keys_buf[:, :n0].float().cpu().numpy(),
+        keys=index.keys_rowmajor().float().cpu().numpy(),
         perm=index.perm[:, :n0].cpu().numpy().astype(np.int64),
-        centers=[None] + [index.centers[l][:, : index.size[l]].float().cpu().numpy()
+        centers=[None] + [index.centers_rowmajor(l).float().cpu().numpy()
                           for l in range(1, index.num_levels)],
         radii=[None] + [index.radii[l][:, : index.size[l]].cpu().numpy()
                         for l in range(1, index.num_levels)],
@@ -143,6 +156,11 @@ def main():
     ap.add_argument("--nodes-per-wave", type=int, default=0)
     ap.add_argument("--kernel", type=int, default=0)
     ap.add_argument("--kmeans-iters", type=int, default=-1)
+    ap.add_argument("--separate-merge", action="store_true",
+                    help="fold the attention partials in a second launch")
+    ap.add_argument("--counters", action="store_true",
+                    help="run the steps once, untimed, plus a kernel of known traffic "
+                         "(for rocprofv3 --pmc runs)")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         log("bench.py: this path is built and measured on ONE GPU (each KV head owns an "
@@ -185,7 +203,7 @@ def main():
             taus[i, hs] = exact_topk(keys_d[b], q_d[i, hs], ksel[b])
     scale = w.d ** -0.5
     searcher = HIPSearcher(block_threads=a.block_threads, nodes_per_wave=a.nodes_per_wave,
-                           kernel=a.kernel)
+                           kernel=a.kernel, separate_merge=a.separate_merge)
     h_all = w.batch * w.h_q
     plan = searcher.plan_attention(index, h_all, scaling=torch.full((h_all,), scale))
     outs = torch.empty((total, h_all, w.d), dtype=torch.float32, device=dev)
@@ -194,6 +212,22 @@ def main():
     for i in range(W):
         plan.run(q_d[i], taus[i], outs[i])
     torch.cuda.synchronize()
+
+    if a.counters:
+        # For `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`: K plain launches of the
+        # search kernel and one elementwise kernel of known traffic (reads 256 MiB, writes
+        # 256 MiB in a single dispatch) that scales the counters; nothing is timed.
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        torch.add(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        for i in range(W, total):
+            plan.run(q_d[i], taus[i], outs[i])
+        torch.cuda.synchronize()
+        print(json.dumps({"mode": "counters", "steps": K,
+                          "calibration_kernel_bytes_read": src.numel() * 4,
+                          "calibration_kernel_bytes_written": dst.numel() * 4}), flush=True)
+        return
 
     # ---- counters: algorithmic bytes of the K timed steps ---------------------------
     stats = torch.zeros((index.num_trees, _lib.HIRA_MAX_LEVELS + 2), dtype=torch.int64, device=dev)
@@ -297,7 +331,8 @@ def main():
                    "head_dim": w.d, "batch": w.batch, "levels": w.num_levels, "bf": w.bf,
                    "select_per_head": ksel, "kmeans_iters": niter},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None},
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": measured_traffic(w.name)},
         "algorithmic_bytes_per_step": round(alg_bytes),
         "gpu_us_per_step_events": round(kernel_us, 3),
         "eager_us_per_step": round(eager_ms * 1e3 / K, 3),

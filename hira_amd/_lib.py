@@ -51,6 +51,7 @@ class HiraQuery(C.Structure):
         ("tree_q_off", _vp),
         ("tree_q_heads", _vp),
         ("max_group", C.c_int32),
+        ("group_size", C.c_int32),
     ]
 
 
@@ -77,6 +78,7 @@ class HiraLaunch(C.Structure):
         ("block_threads", C.c_int32),
         ("nodes_per_wave", C.c_int32),
         ("kernel", C.c_int32),
+        ("separate_merge", C.c_int32),
     ]
 
 

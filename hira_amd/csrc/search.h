@@ -26,6 +26,7 @@ struct SearchParams {
     const float* scaling;
     const int32_t* tree_q_off;
     const int32_t* tree_q_heads;
+    int32_t group_size;  // > 0: head h belongs to tree h / group_size (the CSR is not read)
     // queue (always row-major)
     const void* queue_keys;
     const void* queue_values;
@@ -48,6 +49,8 @@ struct SearchParams {
     float* part_acc;  // (H_q, P, Dv)
     int32_t num_parts;  // P = gridDim.x
     int32_t gmax_state; // MFMA kernel: heads per pass its LDS state rows are sized for
+    float* attn_out;    // (H_q, Dv): written by the kernel itself when `done` is set
+    int32_t* done;      // (T, passes) arrival counters, zero between launches; NULL: no fold
     unsigned long long* stats;
 };
 
@@ -64,6 +67,7 @@ struct SearchPlan {
 
 // search_mfma.hip
 bool mfma_search_supported(const HiraTree* t, const HiraQueue* queue);
+size_t mfma_search_smem(int threads, int gmax, int dim, int bf);
 int launch_search_mfma(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
 
 // Element index of (row, column j) inside one tree's (cap, D) matrix.

@@ -460,7 +460,7 @@ static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* que
         plan->num_nodes = t->size[1];
         plan->tree_blocks = (t->size[1] + 15) / 16;
         plan->queue_blocks = 0;
-        plan->smem = (size_t)(threads / 64) * plan->gmax * (t->dim + 2) * sizeof(float);
+        plan->smem = mfma_search_smem(threads, plan->gmax, t->dim, t->bf);
         return HIRA_OK;
     }
     plan->gmax = q->max_group <= 1 ? 1 : (q->max_group <= 4 ? 4 : 8);
@@ -518,13 +518,20 @@ static int dispatch_lpr(const SearchPlan& plan, const SearchParams& p, dim3 grid
 
 using namespace hira;
 
+// partials (acc, m, l) followed by the arrival counters of the fused fold
+static size_t workspace_need(int h_q, size_t P, int vdim, int trees, int passes) {
+    size_t b = (size_t)h_q * P * (size_t)(vdim + 2) * sizeof(float);
+    b = (b + 255) & ~(size_t)255;
+    return b + (size_t)trees * passes * sizeof(int32_t);
+}
+
 extern "C" size_t hira_search_workspace_bytes(const HiraTree* tree, const HiraQuery* query,
                                               const HiraQueue* queue,
                                               const HiraLaunch* launch) {
     SearchPlan plan;
     if (make_plan(tree, query, queue, launch, &plan) != HIRA_OK) return 0;
     const size_t P = (size_t)plan.tree_blocks + plan.queue_blocks;
-    return (size_t)query->num_q_heads * P * (size_t)(tree->vdim + 2) * sizeof(float);
+    return workspace_need(query->num_q_heads, P, tree->vdim, tree->num_trees, plan.head_chunks);
 }
 
 extern "C" int hira_search(const HiraTree* tree, const HiraQuery* query, const HiraQueue* queue,
@@ -599,28 +606,40 @@ extern "C" int hira_search(const HiraTree* tree, const HiraQuery* query, const H
     if (P == 0) return HIRA_OK;
     p.num_parts = P;
     if (attn) {
-        const size_t need =
-            (size_t)query->num_q_heads * P * (size_t)(tree->vdim + 2) * sizeof(float);
+        const size_t need = workspace_need(query->num_q_heads, (size_t)P, tree->vdim,
+                                           tree->num_trees, plan.head_chunks);
         if (workspace == nullptr || workspace_bytes < need)
             return fail(HIRA_EWORKSPACE, "workspace %zu bytes, need %zu", workspace_bytes, need);
         float* w = reinterpret_cast<float*>(workspace);
         p.part_acc = w;
         p.part_m = w + (size_t)query->num_q_heads * P * tree->vdim;
         p.part_l = p.part_m + (size_t)query->num_q_heads * P;
+        p.attn_out = out->attn_out;
+        // the MFMA kernel folds the partials itself (the last workgroup of a tree to arrive
+        // does it) unless the caller asks for the second launch
+        if (plan.kernel == 2 && !(launch && launch->separate_merge))
+            p.done = reinterpret_cast<int32_t*>(
+                reinterpret_cast<char*>(workspace) + need -
+                (size_t)tree->num_trees * plan.head_chunks * sizeof(int32_t));
     }
+    p.group_size = query->group_size > 0 ? query->group_size : 0;
+    if (p.group_size > 0)
+        HIRA_CHECK_ARG((int64_t)p.group_size * tree->num_trees == query->num_q_heads,
+                       "group_size %d x %d trees != %d heads", p.group_size, tree->num_trees,
+                       query->num_q_heads);
 
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     dim3 grid(P, tree->num_trees, plan.head_chunks);
     p.gmax_state = plan.gmax;
     if (plan.kernel == 2)
-        rc = launch_search_mfma(plan, p, grid, s);
+        rc = launch_search_mfma(plan, p, dim3(tree->num_trees, P, plan.head_chunks), s);
     else
         rc = tree->dtype == HIRA_F32 ? dispatch_lpr<float>(plan, p, grid, s)
                                      : dispatch_lpr<bf16_t>(plan, p, grid, s);
     if (rc != HIRA_OK) return rc;
     HIRA_CHECK_LAUNCH("search kernel");
 
-    if (attn) {
+    if (attn && p.done == nullptr) {
         int dvl = round_pow2((tree->vdim + 3) / 4);
         if (dvl > 256) return fail(HIRA_EINVAL, "vdim %d too wide", tree->vdim);
         const int ng = 256 / dvl;

@@ -28,14 +28,15 @@ DEFAULT_OUTPUT_FILL_VALUE = 0.0
 class HIPSearcher(BaseSearcher):
     def __init__(self, block_c=None, output_fill_value: float = DEFAULT_OUTPUT_FILL_VALUE,
                  *, index_space: str = "slot", block_threads: int = 0, nodes_per_wave: int = 0,
-                 kernel: int = 0):
+                 kernel: int = 0, separate_merge: bool = False):
         super().__init__()
         if index_space not in ("slot", "position"):
             raise ValueError("index_space must be 'slot' or 'position'")
         self.block_c = block_c  # accepted for HiraConfig.get_searcher_kwargs(); unused
         self.output_fill_value = float(output_fill_value)
         self.index_space = index_space
-        self.launch = _lib.HiraLaunch(int(block_threads), int(nodes_per_wave), int(kernel))
+        self.launch = _lib.HiraLaunch(int(block_threads), int(nodes_per_wave), int(kernel),
+                                      int(bool(separate_merge)))
         self._tmp_out: Optional[torch.Tensor] = None
         self._map_cache = {}
         self._workspace: Optional[torch.Tensor] = None
@@ -84,7 +85,7 @@ class HIPSearcher(BaseSearcher):
             raise ValueError(f"scaling must have length H={h}, got {s.numel()}")
         return s.contiguous()
 
-    def _head_map(self, h_q: int, indexer, q_head_to_kv) -> Tuple[torch.Tensor, torch.Tensor, int]:
+    def _head_map(self, h_q: int, indexer, q_head_to_kv) -> Tuple[torch.Tensor, torch.Tensor, int, int]:
         """CSR of the query heads of each tree.  Default map: head h of sequence b belongs
         to tree b*H_kv + h // (H_q/H_kv) (searcher/cuda.py:23-33)."""
         t, batch, h_kv = indexer.num_trees, indexer.batch, indexer.num_heads
@@ -93,6 +94,7 @@ class HIPSearcher(BaseSearcher):
         hit = self._map_cache.get(key)
         if hit is not None:
             return hit
+        group = 0
         if q_head_to_kv is None:
             if h_q % batch:
                 raise ValueError(f"H_q={h_q} not divisible by batch={batch}")
@@ -106,6 +108,7 @@ class HIPSearcher(BaseSearcher):
                         f"by H_kv={h_kv}")
                 local = torch.arange(per_seq) // (per_seq // h_kv)
             m = (torch.arange(batch)[:, None] * h_kv + local[None, :]).reshape(-1)
+            group = per_seq // h_kv  # head h of the launch belongs to tree h // group
         else:
             if not torch.is_tensor(q_head_to_kv):
                 raise TypeError(
@@ -120,7 +123,7 @@ class HIPSearcher(BaseSearcher):
         off = torch.zeros(t + 1, dtype=torch.int32)
         off[1:] = counts.cumsum(0).to(torch.int32)
         dev = indexer.device
-        val = (off.to(dev), order.to(torch.int32).to(dev), int(counts.max().item()))
+        val = (off.to(dev), order.to(torch.int32).to(dev), int(counts.max().item()), group)
         self._map_cache = {key: val}
         return val
 
@@ -130,15 +133,17 @@ class HIPSearcher(BaseSearcher):
         h_q = q.shape[0]
         tau = self._coerce_threshold(threshold, h_q, dev)
         sc = self._coerce_scaling(scaling, h_q, dev)
-        off, heads, gmax = self._head_map(h_q, indexer, q_head_to_kv)
+        off, heads, gmax, group = self._head_map(h_q, indexer, q_head_to_kv)
         qs = _lib.HiraQuery(h_q, q.data_ptr(), tau.data_ptr(), sc.data_ptr(), off.data_ptr(),
-                            heads.data_ptr(), gmax)
+                            heads.data_ptr(), gmax, group)
         return qs, (q, tau, sc, off, heads)
 
     def _get_workspace(self, nbytes: int, device) -> torch.Tensor:
         if self._workspace is None or self._workspace.numel() < nbytes or \
                 self._workspace.device != device:
-            self._workspace = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
+            # zero once: the arrival counters inside must start at zero and are left at
+            # zero by every call
+            self._workspace = torch.zeros(max(nbytes, 1), dtype=torch.uint8, device=device)
         return self._workspace
 
     def _prepare_output_buffer(self, h_q: int, n: int, device) -> torch.Tensor:
@@ -250,18 +255,18 @@ class DecodePlan:
         self.lib = _lib.lib()
         dev = indexer.device
         self.scaling = searcher._coerce_scaling(scaling, num_q_heads, dev)
-        off, heads, gmax = searcher._head_map(num_q_heads, indexer, q_head_to_kv)
+        off, heads, gmax, group = searcher._head_map(num_q_heads, indexer, q_head_to_kv)
         self._keep = (off, heads, stats)
         self.query = _lib.HiraQuery(num_q_heads, None, None, self.scaling.data_ptr(),
-                                    off.data_ptr(), heads.data_ptr(), gmax)
+                                    off.data_ptr(), heads.data_ptr(), gmax, group)
         self.out = _lib.HiraSearchOut()
         self.out.stats = None if stats is None else stats.data_ptr()
         self.launch = searcher.launch
         self.tree = indexer.tree_struct()
-        fake_q = _lib.HiraQuery(num_q_heads, 1, 1, 1, 1, 1, gmax)  # sizes only
+        fake_q = _lib.HiraQuery(num_q_heads, 1, 1, 1, 1, 1, gmax, group)  # sizes only
         self.ws_bytes = self.lib.hira_search_workspace_bytes(
             C.byref(self.tree), C.byref(fake_q), None, C.byref(self.launch))
-        self.ws = torch.empty(max(self.ws_bytes, 1), dtype=torch.uint8, device=dev)
+        self.ws = torch.zeros(max(self.ws_bytes, 1), dtype=torch.uint8, device=dev)
         self._refs = (C.byref(self.tree), C.byref(self.query), C.byref(self.out),
                       C.byref(self.launch))
 

@@ -82,6 +82,9 @@ typedef struct HiraQuery {
     const int32_t* tree_q_off;   /* (T+1) */
     const int32_t* tree_q_heads; /* (H_q) */
     int32_t max_group;           /* max heads of one tree (host knows it) */
+    int32_t group_size;          /* > 0: the default map, head h belongs to tree
+                                    h / group_size (H_q = T * group_size); the kernels then
+                                    skip the CSR lookup.  0: use the CSR above. */
 } HiraQuery;
 
 /* Keys/values that are cached but not yet in the index (the reference's decode queue,
@@ -125,12 +128,17 @@ typedef struct HiraLaunch {
     int32_t block_threads;  /* 64, 128 or 256; 0 = default */
     int32_t nodes_per_wave; /* level-1 nodes one wavefront walks; 0 = default */
     int32_t kernel;         /* 0 = auto, 1 = vector-ALU kernel, 2 = MFMA kernel (bf16) */
+    int32_t separate_merge; /* != 0: fold the attention partials in a second launch even
+                               where the search kernel could do it itself */
 } HiraLaunch;
 
 int hira_abi_version(void);
 const char* hira_last_error(void);
 
-/* Bytes of workspace hira_search needs for this tree/query (attention partials). */
+/* Bytes of workspace hira_search needs for this tree/query (attention partials + arrival
+ * counters).  The workspace must be ZERO before its first use; every completed call leaves
+ * the counters zero again, so it can be reused without clearing.  Two calls that may run
+ * concurrently need separate workspaces. */
 size_t hira_search_workspace_bytes(const HiraTree* tree, const HiraQuery* query,
                                    const HiraQueue* queue, const HiraLaunch* launch);
 

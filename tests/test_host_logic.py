@@ -30,18 +30,18 @@ class _FakeIndexer:
 
 
 def test_default_head_map_is_gqa_grouping():
-    off, heads, gmax = HIPSearcher()._head_map(32, _FakeIndexer(1, 8), None)
-    assert gmax == 4 and off.tolist() == list(range(0, 33, 4))
+    off, heads, gmax, group = HIPSearcher()._head_map(32, _FakeIndexer(1, 8), None)
+    assert gmax == 4 and group == 4 and off.tolist() == list(range(0, 33, 4))
     assert heads.tolist() == list(range(32))
     # two sequences of 4 query / 2 KV heads: tree = b*H_kv + h // 2
-    off, heads, gmax = HIPSearcher()._head_map(8, _FakeIndexer(2, 2), None)
-    assert off.tolist() == [0, 2, 4, 6, 8] and heads.tolist() == list(range(8))
+    off, heads, gmax, group = HIPSearcher()._head_map(8, _FakeIndexer(2, 2), None)
+    assert off.tolist() == [0, 2, 4, 6, 8] and heads.tolist() == list(range(8)) and group == 2
 
 
 def test_explicit_head_map_and_its_errors():
     se = HIPSearcher()
-    off, heads, gmax = se._head_map(4, _FakeIndexer(1, 2), torch.tensor([1, 0, 1, 0]))
-    assert off.tolist() == [0, 2, 4] and heads.tolist() == [1, 3, 0, 2] and gmax == 2
+    off, heads, gmax, group = se._head_map(4, _FakeIndexer(1, 2), torch.tensor([1, 0, 1, 0]))
+    assert off.tolist() == [0, 2, 4] and heads.tolist() == [1, 3, 0, 2] and gmax == 2 and group == 0
     with pytest.raises(ValueError):
         se._head_map(4, _FakeIndexer(1, 2), torch.tensor([0, 1, 2, 0]))  # out of range
     with pytest.raises(ValueError):
