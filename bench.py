@@ -158,6 +158,9 @@ def main():
     ap.add_argument("--kmeans-iters", type=int, default=-1)
     ap.add_argument("--separate-merge", action="store_true",
                     help="fold the attention partials in a second launch")
+    ap.add_argument("--profile", action="store_true",
+                    help="only the warm-up and the timed steps (no counter pass, no dense or "
+                         "CPU comparators): every launch a profiler sees is the measured one")
     ap.add_argument("--counters", action="store_true",
                     help="run the steps once, untimed, plus a kernel of known traffic "
                          "(for rocprofv3 --pmc runs)")
@@ -233,9 +236,10 @@ def main():
     stats = torch.zeros((index.num_trees, _lib.HIRA_MAX_LEVELS + 2), dtype=torch.int64, device=dev)
     splan = searcher.plan_attention(index, h_all, scaling=torch.full((h_all,), scale), stats=stats)
     scratch = torch.empty((h_all, w.d), dtype=torch.float32, device=dev)
-    for i in range(W, total):
-        splan.run(q_d[i], taus[i], scratch)
-    torch.cuda.synchronize()
+    if not a.profile:
+        for i in range(W, total):
+            splan.run(q_d[i], taus[i], scratch)
+        torch.cuda.synchronize()
     alg_bytes, counts = algorithmic_bytes(stats.cpu().numpy(), w, index.num_levels, K)
     want_pairs = sum(ksel[b] * w.h_q for b in range(w.batch))
     if abs(counts["selected_pairs_per_step"] - want_pairs) > 1e-6 * want_pairs:
@@ -276,6 +280,11 @@ def main():
 
     # ---- dense comparators ------------------------------------------------------------
     dense_us = {}
+    if a.profile:
+        print(json.dumps({"mode": "profile", "steps": K, "us_per_step_wall": round(us_per_step, 3),
+                          "us_per_step_events": round(kernel_us, 3),
+                          "eager_us_per_step": round(eager_ms * 1e3 / K, 3)}), flush=True)
+        return
     try:
         qd = q_d[W:].reshape(K, w.batch, w.h_q, 1, w.d)
         kk = keys_d[:, :, None].expand(w.batch, w.h_kv, w.group, w.n, w.d).reshape(
