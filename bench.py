@@ -56,7 +56,7 @@ def measured_traffic(workload_name):
     """HBM bytes per launch of the search kernel from the committed rocprofv3 --pmc summary
     (FETCH_SIZE + WRITE_SIZE, each scaled by what the same counter reads for a kernel of
     known traffic), or None when no summary for this workload is committed."""
-    f = ROOT / "profiles" / f"search_traffic_{workload_name}.json"
+    f = ROOT / "profiles" / f"search_traffic_{workload_name}.txt"
     if not f.exists():
         return None
     try:
