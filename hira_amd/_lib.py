@@ -101,6 +101,7 @@ SYMBOLS = {
         [C.POINTER(HiraTree), _vp, _vp, C.c_int32, C.c_int32, C.c_int32, C.c_uint64, _vp,
          C.c_size_t, _vp],
     ),
+    "hira_update": (C.c_int, [C.POINTER(HiraTree), _vp, _vp, C.c_int32, _vp, _vp]),
 }
 
 _lib = None

@@ -18,7 +18,7 @@
 // layout: r_p = max over children (||c_child - c_p|| + r_child), the bound of
 // indexer/cpu.py:286-309 / indexer/cuda.py:114-198, against the ROUNDED centres and
 // nudged up by a few ulp so that rounding never makes a ball too small.
-#include "search.h"
+#include "rows.h"
 
 namespace hira {
 
@@ -30,37 +30,6 @@ __device__ __forceinline__ uint64_t mix64(uint64_t z) {
     z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
     z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
     return z ^ (z >> 31);
-}
-
-template <typename T>
-__device__ __forceinline__ float load_elem(const void* base, size_t i);
-template <>
-__device__ __forceinline__ float load_elem<float>(const void* base, size_t i) {
-    return reinterpret_cast<const float*>(base)[i];
-}
-template <>
-__device__ __forceinline__ float load_elem<bf16_t>(const void* base, size_t i) {
-    return bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(base)[i]);
-}
-template <typename T>
-__device__ __forceinline__ void store_elem(void* base, size_t i, float v);
-template <>
-__device__ __forceinline__ void store_elem<float>(void* base, size_t i, float v) {
-    reinterpret_cast<float*>(base)[i] = v;
-}
-template <>
-__device__ __forceinline__ void store_elem<bf16_t>(void* base, size_t i, float v) {
-    reinterpret_cast<uint16_t*>(base)[i] = f32_to_bf16_bits(v);
-}
-template <typename T>
-__device__ __forceinline__ float round_to(float v);
-template <>
-__device__ __forceinline__ float round_to<float>(float v) {
-    return v;
-}
-template <>
-__device__ __forceinline__ float round_to<bf16_t>(float v) {
-    return bf16_bits_to_f32(f32_to_bf16_bits(v));
 }
 
 __global__ void k_fill_i32(int32_t* p, size_t n, int32_t v) {

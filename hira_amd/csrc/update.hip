@@ -1,0 +1,315 @@
+// Append-on-decode index update: m new keys/values per tree go into the existing tree.
+//
+// Replaces CUDAIndexer.update and its Triton kernels (indexer/cuda.py:544-701, 707-1231;
+// kernels/triton_update_kernels.py:6-123, 126-235, 238-326) with one launch: one workgroup
+// per tree walks that tree's new keys in insertion order, so slots, counts and radii need
+// no global atomics and the result is reproducible.  For every key:
+//   1. nearest level-1 node that still has a free child slot (exact fp32 L2 distance over
+//      the nodes in use; full nodes are skipped before their centre is read) -- the
+//      reference's nearest_l2 + valid-mask step;
+//   2. the key takes the node's next slot (the reference's atomic slot reservation), the
+//      node's radius grows to cover it (its atomic-max step) and every ancestor's radius is
+//      re-inflated: R_a = max(R_a, ||c_child - c_a|| + r_child) (indexer/cuda.py:1200-1231);
+//      centres never move, radii only grow, exactly as in the reference;
+//   3. if no node has room the key opens a new level-1 node whose centre is the key itself
+//      (the reference draws its new parents from the orphans, indexer/cuda.py:612-635); the
+//      new node is attached the same way one level up: nearest level-2 node with a free
+//      child slot, else a new level-2 node, ... up to the root level, which simply grows.
+// Child counts stay authoritative (the reference over-counts on overflow and repairs the
+// counters with an O(N D) rescan after every update, indexer/cuda.py:1233-1298).
+//
+// state (T, HIRA_MAX_LEVELS + 2) int32: [l] = slots of level l in use (l >= 1; the host keeps
+// the maximum over the trees as size[l]), [HIRA_MAX_LEVELS] = keys inserted so far,
+// [HIRA_MAX_LEVELS + 1] = error flag (1: a level ran out of capacity; the key was dropped).
+#include "rows.h"
+
+namespace hira {
+
+constexpr int kUpdThreads = 256;
+
+struct UpdateParams {
+    void* keys;
+    void* values;
+    int32_t* perm;
+    void* centers[HIRA_MAX_LEVELS];
+    float* radii[HIRA_MAX_LEVELS];
+    int32_t* counts[HIRA_MAX_LEVELS];
+    int32_t cap[HIRA_MAX_LEVELS];
+    int32_t num_levels, bf, dim, vdim, layout;
+    const void* new_keys;    // (T, m, D)
+    const void* new_values;  // (T, m, Dv) or NULL
+    int32_t m;
+    int32_t* state;
+};
+
+__device__ __forceinline__ float block_sum(float v, float* red) {
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) v += __shfl_xor(v, off, 64);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return red[0] + red[1] + red[2] + red[3];
+}
+
+// ||x - row||_2 with x in LDS (fp32) and row = node `node` of a tree matrix; whole workgroup
+template <typename T>
+__device__ __forceinline__ float block_dist(const float* x, const void* mat, size_t tree_base,
+                                            int layout, int D, size_t node, float* red) {
+    float ss = 0.0f;
+    for (int j = threadIdx.x; j < D; j += kUpdThreads) {
+        const float df = x[j] - load_elem<T>(mat, tree_base + elem_index(layout, D, node, j));
+        ss += df * df;
+    }
+    return sqrtf(block_sum(ss, red));
+}
+
+// a bound must survive the fp32 rounding of the sums that produced it
+__device__ __forceinline__ float pad_up(float r) { return r > 0.0f ? r * (1.0f + 4.0f * 1.1920929e-7f) + 1e-30f : r; }
+
+// Nearest node of level l (among the first `used` ones) with a free child slot; -1 if none.
+// Wave w scans nodes w, w+4, ...; a full node costs one count read.  Ties go to the lowest id.
+template <typename T>
+__device__ int nearest_with_room(const UpdateParams& p, int tree, int l, int used, const float* x,
+                                 float* red_f, int* red_i) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int D = p.dim;
+    const size_t base = (size_t)tree * p.cap[l];
+    const int32_t* cnt = p.counts[l] + base;
+    float best = INFINITY;
+    int arg = -1;
+    for (int n0 = wave * 64; n0 < used; n0 += 4 * 64) {
+        const int n = n0 + lane;
+        // a node in use with a free slot; count 0 marks a pad slot, which is not a node yet
+        const bool room = n < used && cnt[n] > 0 && cnt[n] < p.bf;
+        unsigned long long bal = __ballot(room);
+        while (bal != 0ull) {  // uniform in the wave
+            const int b = __ffsll((long long)bal) - 1;
+            bal &= bal - 1ull;
+            const int node = n0 + b;
+            float ss = 0.0f;
+            for (int j = lane; j < D; j += 64) {
+                const float df =
+                    x[j] - load_elem<T>(p.centers[l], base * D + elem_index(p.layout, D, (size_t)node, j));
+                ss += df * df;
+            }
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) ss += __shfl_xor(ss, off, 64);
+            if (ss < best) {  // nodes come in increasing order inside a wave
+                best = ss;
+                arg = node;
+            }
+        }
+    }
+    __syncthreads();
+    if (lane == 0) {
+        red_f[wave] = best;
+        red_i[wave] = arg;
+    }
+    __syncthreads();
+    float b = red_f[0];
+    int a = red_i[0];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {
+        const float bw = red_f[w];
+        const int aw = red_i[w];
+        if (aw >= 0 && (a < 0 || bw < b || (bw == b && aw < a))) {
+            b = bw;
+            a = aw;
+        }
+    }
+    __syncthreads();
+    return a;
+}
+
+template <typename T>
+__global__ __launch_bounds__(kUpdThreads) void k_update(const UpdateParams p) {
+    extern __shared__ float sm[];
+    float* x = sm;              // (D) the new key, fp32
+    float* cbuf = sm + p.dim;   // (D) centre of the node being attached upwards
+    __shared__ float red_f[4];
+    __shared__ int red_i[4];
+    const int tree = blockIdx.x;
+    const int t = threadIdx.x;
+    const int D = p.dim, Dv = p.vdim, L = p.num_levels, bf = p.bf;
+    int32_t* st = p.state + (size_t)tree * (HIRA_MAX_LEVELS + 2);
+    const size_t base0 = (size_t)tree * p.cap[0];
+
+    for (int i = 0; i < p.m; ++i) {
+        const size_t src = ((size_t)tree * p.m + i) * D;
+        for (int j = t; j < D; j += kUpdThreads) x[j] = load_elem<T>(p.new_keys, src + j);
+        __syncthreads();
+        const int position = st[HIRA_MAX_LEVELS];
+
+        long long slot = -1;  // key slot
+        int node1 = -1;       // level-1 node that took the key (L >= 2)
+        if (L == 1) {
+            slot = position < p.cap[0] ? position : -1;
+        } else {
+            node1 = nearest_with_room<T>(p, tree, 1, st[1], x, red_f, red_i);
+            if (node1 < 0) {
+                // ---- open a new level-1 node; attach it upwards -----------------------
+                // child_c = centre of the node being attached (the key itself at level 1)
+                for (int j = t; j < D; j += kUpdThreads) cbuf[j] = x[j];
+                __syncthreads();
+                int lvl = 1;          // level of the node that needs a parent
+                int parent = -1;      // node of level lvl+1 that takes it
+                int opened_top = 0;   // levels 1..opened_top get a brand-new node
+                // find the lowest level that has a parent with room
+                while (true) {
+                    if (lvl == L - 1) {  // the root level grows
+                        parent = -1;
+                        break;
+                    }
+                    parent = nearest_with_room<T>(p, tree, lvl + 1, st[lvl + 1], cbuf, red_f, red_i);
+                    if (parent >= 0) break;
+                    ++lvl;
+                }
+                opened_top = lvl;
+                // index of the new node at level opened_top
+                long long idx;
+                if (parent >= 0) {
+                    idx = (long long)parent * bf + p.counts[opened_top + 1][(size_t)tree * p.cap[opened_top + 1] + parent];
+                } else {
+                    idx = st[opened_top];
+                }
+                // every new node below it is the first child of the new node above
+                bool fits = true;
+                long long id = idx;
+                for (int l = opened_top; l >= 1; --l) {
+                    if (id >= p.cap[l]) fits = false;
+                    id *= bf;
+                }
+                if (id >= p.cap[0]) fits = false;
+                __syncthreads();  // everybody has read the counters the writes below change
+                if (!fits) {
+                    if (t == 0) st[HIRA_MAX_LEVELS + 1] = 1;
+                    __syncthreads();
+                    continue;  // uniform: the key is dropped, the host sees the flag
+                }
+                id = idx;
+                for (int l = opened_top; l >= 1; --l) {
+                    const size_t bl = (size_t)tree * p.cap[l];
+                    for (int j = t; j < D; j += kUpdThreads)
+                        store_elem<T>(p.centers[l], bl * D + elem_index(p.layout, D, (size_t)id, j), x[j]);
+                    if (t == 0) {
+                        p.radii[l][bl + id] = 0.0f;
+                        p.counts[l][bl + id] = (l == 1) ? 0 : 1;  // level 1 gets its key below
+                        if (id + 1 > st[l]) st[l] = (int)(id + 1);
+                    }
+                    id *= bf;
+                }
+                if (t == 0 && parent >= 0)
+                    p.counts[opened_top + 1][(size_t)tree * p.cap[opened_top + 1] + parent] += 1;
+                __syncthreads();
+                node1 = (int)(id / bf);  // the new level-1 node (id is now its first key slot)
+            }
+            // the key takes the next slot of node1
+            const size_t b1 = (size_t)tree * p.cap[1];
+            const int c = p.counts[1][b1 + node1];
+            slot = (long long)node1 * bf + c;
+            __syncthreads();
+            if (t == 0) p.counts[1][b1 + node1] = c + 1;
+        }
+        if (slot < 0 || slot >= p.cap[0]) {
+            if (t == 0) st[HIRA_MAX_LEVELS + 1] = 1;
+            __syncthreads();
+            continue;
+        }
+        // ---- write key, value, perm -------------------------------------------------------
+        {
+            const T* dummy = nullptr;
+            (void)dummy;
+            for (int j = t; j < D; j += kUpdThreads)
+                store_elem<T>(p.keys, base0 * D + elem_index(p.layout, D, (size_t)slot, j), x[j]);
+            if (p.new_values && p.values) {
+                const size_t vs = ((size_t)tree * p.m + i) * Dv;
+                for (int j = t; j < Dv; j += kUpdThreads)
+                    store_elem<T>(p.values, (base0 + slot) * Dv + j, load_elem<T>(p.new_values, vs + j));
+            }
+            if (t == 0) {
+                p.perm[base0 + slot] = position;
+                st[HIRA_MAX_LEVELS] = position + 1;
+                if (L == 1 && slot + 1 > st[0]) st[0] = (int)(slot + 1);
+            }
+        }
+        // ---- radii: the leaf parent covers the key, every ancestor covers its child -----
+        if (L >= 2) {
+            size_t child = (size_t)node1;
+            const size_t b1 = (size_t)tree * p.cap[1];
+            float r_child = p.radii[1][b1 + child];
+            {
+                const float dk = block_dist<T>(x, p.centers[1], b1 * D, p.layout, D, child, red_f);
+                const float rn = fmaxf(r_child, pad_up(dk));
+                if (t == 0) p.radii[1][b1 + child] = rn;
+                r_child = rn;
+            }
+            for (int l = 2; l < L; ++l) {
+                const size_t anc = child / bf;
+                const size_t bl = (size_t)tree * p.cap[l], bc = (size_t)tree * p.cap[l - 1];
+                // cbuf := centre of the child
+                __syncthreads();
+                for (int j = t; j < D; j += kUpdThreads)
+                    cbuf[j] = load_elem<T>(p.centers[l - 1], bc * D + elem_index(p.layout, D, child, j));
+                __syncthreads();
+                const float dc = block_dist<T>(cbuf, p.centers[l], bl * D, p.layout, D, anc, red_f);
+                const float ra = p.radii[l][bl + anc];
+                const float rn = fmaxf(ra, pad_up(dc + r_child));
+                __syncthreads();
+                if (t == 0) p.radii[l][bl + anc] = rn;
+                r_child = rn;
+                child = anc;
+            }
+        }
+        __syncthreads();
+    }
+}
+
+}  // namespace hira
+
+using namespace hira;
+
+/* see include/hira_hip.h */
+extern "C" int hira_update(const HiraTree* tree, const void* new_keys, const void* new_values,
+                           int32_t m, int32_t* state, void* stream) {
+    HIRA_CHECK_ARG(tree != nullptr && new_keys != nullptr && state != nullptr,
+                   "tree / new_keys / state missing");
+    HIRA_CHECK_ARG(tree->dtype == HIRA_F32 || tree->dtype == HIRA_BF16, "dtype %d", tree->dtype);
+    HIRA_CHECK_ARG(tree->num_levels >= 1 && tree->num_levels <= HIRA_MAX_LEVELS, "num_levels %d",
+                   tree->num_levels);
+    HIRA_CHECK_ARG(tree->bf >= 1 && tree->bf <= 64, "branching factor %d", tree->bf);
+    HIRA_CHECK_ARG(m >= 0, "m = %d", m);
+    HIRA_CHECK_ARG(tree->keys && tree->perm, "keys / perm missing");
+    HIRA_CHECK_ARG((new_values == nullptr) || tree->values != nullptr,
+                   "values given but the index holds none");
+    if (m == 0) return HIRA_OK;
+    UpdateParams p;
+    memset(&p, 0, sizeof(p));
+    p.keys = tree->keys;
+    p.values = tree->values;
+    p.perm = tree->perm;
+    for (int l = 0; l < HIRA_MAX_LEVELS; ++l) {
+        p.centers[l] = tree->centers[l];
+        p.radii[l] = tree->radii[l];
+        p.counts[l] = tree->counts[l];
+        p.cap[l] = tree->cap[l];
+    }
+    for (int l = 1; l < tree->num_levels; ++l)
+        HIRA_CHECK_ARG(p.centers[l] && p.radii[l] && p.counts[l], "level %d arrays missing", l);
+    p.num_levels = tree->num_levels;
+    p.bf = tree->bf;
+    p.dim = tree->dim;
+    p.vdim = tree->vdim;
+    p.layout = tree->layout;
+    p.new_keys = new_keys;
+    p.new_values = new_values;
+    p.m = m;
+    p.state = state;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const size_t smem = 2 * (size_t)tree->dim * sizeof(float);
+    if (tree->dtype == HIRA_F32)
+        hipLaunchKernelGGL(k_update<float>, dim3(tree->num_trees), dim3(kUpdThreads), smem, s, p);
+    else
+        hipLaunchKernelGGL(k_update<bf16_t>, dim3(tree->num_trees), dim3(kUpdThreads), smem, s, p);
+    HIRA_CHECK_LAUNCH("update kernel");
+    return HIRA_OK;
+}

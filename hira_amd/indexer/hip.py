@@ -126,6 +126,7 @@ class HIPIndexer(BaseIndexer):
         self.radii: List[Optional[torch.Tensor]] = []
         self.counts: List[Optional[torch.Tensor]] = []
         self._tree_struct = None
+        self._state: Optional[torch.Tensor] = None  # device-side bookkeeping of update()
 
     # ------------------------------------------------------------------ reference views
     @property
@@ -233,6 +234,7 @@ class HIPIndexer(BaseIndexer):
                 torch.full((t, self.cap[l]), float("-inf"), dtype=torch.float32, device=dev))
             self.counts.append(torch.zeros((t, self.cap[l]), dtype=torch.int32, device=dev))
         self._tree_struct = None
+        self._state = None
 
     def tree_struct(self) -> _lib.HiraTree:
         """The C view of the tree; valid while this indexer's tensors are alive."""
@@ -328,6 +330,98 @@ class HIPIndexer(BaseIndexer):
             print(f"built {self.num_trees} trees, level sizes {self.size}")
         return self
 
+    def _needed_caps(self, m: int) -> List[int]:
+        """Slots every level may need after m more keys: at most ceil(m/bf)+1 new level-1
+        nodes, ceil(that/bf)+1 new level-2 nodes, ...; a new node's children sit at
+        position node*bf, so a level below must reach (nodes above)*bf."""
+        bf, nl = self.branching_factor, self.num_levels
+        if nl == 1:
+            return [self.num_keys + m]
+        need = [0] * nl
+        new = m
+        for l in range(1, nl):
+            new = -(-new // bf) + 1
+            need[l] = self.size[l] + new
+        for l in range(nl - 2, -1, -1):
+            need[l] = max(need[l], need[l + 1] * bf)
+        return need
+
+    def _grow(self, need: List[int]) -> None:
+        """Re-allocate the level arrays with at least `need` slots (doubling), keeping the
+        contents.  A tile of 16 rows is contiguous, so a tiled matrix grows by rows too."""
+        caps = []
+        for l, (c, n) in enumerate(zip(self.cap, need)):
+            c2 = c if n <= c else max(n, 2 * c)
+            caps.append(-(-c2 // 16) * 16 if self.tiled else c2)
+        if caps == self.cap:
+            return
+
+        def grown(old, cap, fill):
+            new = torch.full((old.shape[0], cap) + tuple(old.shape[2:]), fill, dtype=old.dtype,
+                             device=old.device)
+            new[:, : old.shape[1]] = old
+            return new
+
+        self.keys_buf = grown(self.keys_buf, caps[0], 0)
+        if self.values_buf is not None:
+            self.values_buf = grown(self.values_buf, caps[0], 0)
+        self.perm = grown(self.perm, caps[0], -1)
+        for l in range(1, self.num_levels):
+            self.centers[l] = grown(self.centers[l], caps[l], 0)
+            self.radii[l] = grown(self.radii[l], caps[l], float("-inf"))
+            self.counts[l] = grown(self.counts[l], caps[l], 0)
+        self.cap = caps
+        self._tree_struct = None
+
     @torch.no_grad()
     def update(self, new_keys: torch.Tensor, new_values: Optional[torch.Tensor] = None):
-        raise NotImplementedError("HIP update is not wired yet")
+        """Append new_keys (1, H, m, D) (and new_values (1, H, m, Dv)) in order
+        (indexer/cuda.py:544-701).  One launch; afterwards the level sizes are read back
+        (one small device-to-host copy), as the next search needs them."""
+        if self.keys_buf is None:
+            raise ValueError("Indexer is not built: call build() first.")
+        if new_keys.ndim != 4 or new_keys.shape[0] != self.batch or \
+                new_keys.shape[1] != self.num_heads or new_keys.shape[3] != self.dim:
+            raise ValueError(
+                f"new_keys must be ({self.batch},{self.num_heads},m,{self.dim}), got "
+                f"{tuple(new_keys.shape)}")
+        if (new_values is None) != (self.values_buf is None):
+            raise ValueError("values must be given exactly when the index was built with values")
+        m = int(new_keys.shape[2])
+        if new_values is not None and tuple(new_values.shape[:3]) != tuple(new_keys.shape[:3]):
+            raise ValueError("new_values must be aligned with new_keys")
+        if m == 0:
+            return self
+        self._grow(self._needed_caps(m))
+        t = self.num_trees
+        if self._state is None:
+            st = torch.zeros((t, _lib.HIRA_MAX_LEVELS + 2), dtype=torch.int32)
+            for l in range(self.num_levels):
+                st[:, l] = self.size[l]
+            st[:, _lib.HIRA_MAX_LEVELS] = self.num_keys
+            self._state = st.to(self.device)
+        kin = new_keys.to(device=self.device, dtype=self.dtype).reshape(t, m, self.dim).contiguous()
+        vin = None
+        if new_values is not None:
+            vin = new_values.to(device=self.device, dtype=self.dtype).reshape(
+                t, m, self.vdim).contiguous()
+        tree = self.tree_struct()
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        rc = _lib.lib().hira_update(C.byref(tree), kin.data_ptr(),
+                                    None if vin is None else vin.data_ptr(), m,
+                                    self._state.data_ptr(), stream)
+        _lib.check(rc)
+        st = self._state.cpu()
+        if int(st[:, _lib.HIRA_MAX_LEVELS + 1].max()) != 0:
+            raise RuntimeError("index update ran out of capacity")
+        self.num_keys += m
+        if self.num_levels == 1:
+            self.size = [self.num_keys]
+        else:
+            size = [0] * self.num_levels
+            for l in range(1, self.num_levels):
+                size[l] = int(st[:, l].max())
+            size[0] = size[1] * self.branching_factor
+            self.size = size
+        self._tree_struct = None
+        return self

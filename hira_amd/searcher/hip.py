@@ -272,6 +272,15 @@ class DecodePlan:
 
     def run(self, query: torch.Tensor, threshold: torch.Tensor, out: torch.Tensor,
             stream: Optional[int] = None) -> None:
+        if self.indexer.tree_struct() is not self.tree:  # the index grew since the plan was made
+            self.tree = self.indexer.tree_struct()
+            need = self.lib.hira_search_workspace_bytes(
+                C.byref(self.tree), C.byref(self.query), None, C.byref(self.launch))
+            if need > self.ws_bytes:
+                self.ws = torch.zeros(need, dtype=torch.uint8, device=self.indexer.device)
+            self.ws_bytes = need
+            self._refs = (C.byref(self.tree), C.byref(self.query), C.byref(self.out),
+                          C.byref(self.launch))
         self.query.q = query.data_ptr()
         self.query.tau = threshold.data_ptr()
         self.out.attn_out = out.data_ptr()

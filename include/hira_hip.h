@@ -177,6 +177,26 @@ int hira_build(const HiraTree* tree, const void* keys_in, const void* values_in,
                int32_t niter, int32_t pack_rounds, uint64_t seed, void* workspace,
                size_t workspace_bytes, void* stream);
 
+/*
+ * Append m new keys (and values) per tree to an existing index, in insertion order.
+ * Replaces CUDAIndexer.update (indexer/cuda.py:544-701) and its kernels nearest_l2 (kernels/
+ * triton_update_kernels.py:6-123, 329-418), fill_existing_children_atomic (:126-235) and
+ * update_parent_radii_atomic (:238-326): a key joins the nearest level-1 node with a free
+ * slot (radius and ancestors' radii grow, centres never move); when none has room it opens
+ * a new level-1 node centred on itself, attached upwards by the same rule.
+ *   tree       the index; cap[] must leave room: per call at most ceil(m/bf)+1 new nodes
+ *              appear at level 1, ceil(that/bf)+1 at level 2, ... (tree->size[] is not read)
+ *   new_keys   (T, m, D), new_values (T, m, Dv) or NULL, tree dtype, row-major
+ *   state      (T, HIRA_MAX_LEVELS+2) int32, kept by the caller across calls:
+ *              [l] = slots of level l in use (initially size[l]; [0] is only kept for
+ *              one-level indexes), [HIRA_MAX_LEVELS] = keys inserted so far (initially n),
+ *              [HIRA_MAX_LEVELS+1] = set to 1 if a key was dropped for lack of capacity.
+ * After the call the caller sets size[l] = max over trees of state[.][l] (level 0:
+ * size[0] = size[1]*bf) before the next search.
+ */
+int hira_update(const HiraTree* tree, const void* new_keys, const void* new_values, int32_t m,
+                int32_t* state, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

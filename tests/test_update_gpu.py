@@ -1,0 +1,167 @@
+"""GPU tests of the append path (hira_update through HIPIndexer.update): every key present
+exactly once, counts and radii stay valid bounds, search after update == brute force
+(tests/test_cuda_indexer_searcher.py:205-262, 594-607 and tests/test_cuda_pipeline.py:215-226
+of the reference)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import hira_oracle as ho
+from helpers import (assert_same_selection, bf16_round, clustered_keys, midpoint_threshold,
+                     random_query, rel_err)
+
+pytestmark = pytest.mark.gpu
+
+
+def _check_tree(idx, keys_all, vals_all):
+    """Structure after updates: perm is a permutation of the inserted positions, rows follow
+    their slot, children packed from slot 0, every radius covers its subtree."""
+    t, n, d = keys_all.shape
+    bf, nl = idx.branching_factor, idx.num_levels
+    kr = idx.keys_rowmajor().float().cpu().numpy()
+    perm = idx.perm[:, : idx.size[0]].cpu().numpy().astype(np.int64)
+    vals = idx.values_buf[:, : idx.size[0]].float().cpu().numpy()
+    for h in range(t):
+        ok = perm[h] >= 0
+        assert np.array_equal(np.sort(perm[h][ok]), np.arange(n))
+        assert np.array_equal(kr[h][ok], keys_all[h][perm[h][ok]])
+        assert np.array_equal(vals[h][ok], vals_all[h][perm[h][ok]])
+        if nl == 1:
+            continue
+        child_c, child_r, child_ok = kr[h], np.zeros(idx.size[0], np.float32), ok
+        for l in range(1, nl):
+            k = idx.size[l]
+            cen = idx.centers_rowmajor(l)[h].float().cpu().numpy()
+            rad = idx.radii[l][h, :k].cpu().numpy()
+            cnt = idx.counts[l][h, :k].cpu().numpy()
+            short = k * bf - len(child_ok)      # slots past the level's size are absent
+            if short > 0:
+                child_c = np.concatenate([child_c, np.zeros((short, d), np.float32)])
+                child_r = np.concatenate([child_r, np.zeros(short, np.float32)])
+                child_ok = np.concatenate([child_ok, np.zeros(short, bool)])
+            blk = child_ok[: k * bf].reshape(k, bf)
+            assert np.array_equal(cnt, blk.sum(1)), f"counts level {l}"
+            assert np.all(blk[:, :-1] >= blk[:, 1:])
+            need = ho.radii_from_layout(child_c[: k * bf], child_r[: k * bf], child_ok[: k * bf], cen, bf)
+            has = cnt > 0
+            assert np.all(rad[has] >= need[has] * (1 - 1e-6) - 1e-6), f"radius level {l}"
+            child_c, child_r, child_ok = cen, np.where(has, rad, 0).astype(np.float32), has
+
+
+UPDATE_CASES = [
+    # trees, n0, appended chunks, d, bf, levels, dtype
+    (2, 128, [1, 1, 1, 7, 64, 30], 32, 8, 3, torch.float32),
+    (2, 2048, [1] * 40 + [64, 500], 128, 32, 3, torch.bfloat16),    # tiled, full blocks at build
+    (1, 1000, [33, 1, 1, 200], 64, 16, 4, torch.bfloat16),          # pad slots inside blocks
+    (3, 50, [5, 5, 100], 64, 4, 2, torch.float32),
+    (2, 40, [1, 2, 3, 50], 32, 8, 1, torch.float32),                # one level: plain append
+    (1, 64, [1] * 70, 128, 32, 4, torch.bfloat16),                  # tree smaller than a block
+]
+
+
+@pytest.mark.parametrize("case", UPDATE_CASES, ids=[f"t{c[0]}_n{c[1]}_m{sum(c[2])}_d{c[3]}_bf{c[4]}_L{c[5]}_"
+                                                      f"{'bf16' if c[6] == torch.bfloat16 else 'f32'}"
+                                                      for c in UPDATE_CASES])
+def test_update_keeps_tree_valid_and_search_exact(case, gpu_device):
+    from hira_amd.indexer.hip import HIPIndexer
+    from hira_amd.searcher.hip import HIPSearcher
+
+    t, n0, chunks, d, bf, nl, dtype = case
+    print(f"case {case}", flush=True)
+    n = n0 + sum(chunks)
+    rnd = bf16_round if dtype == torch.bfloat16 else (lambda x: x)
+    keys = rnd(clustered_keys(t, n, d, seed=17 + n, clusters=max(2, n // 50)))
+    vals = rnd(np.random.default_rng(n).normal(size=(t, n, d)).astype(np.float32))
+    K, V = torch.from_numpy(keys)[None].to(dtype), torch.from_numpy(vals)[None].to(dtype)
+    idx = HIPIndexer(nl, 1, bf).build(K[:, :, :n0], V[:, :, :n0])
+    searcher = HIPSearcher(index_space="position")
+    h_q = 2 * t
+    q2kv = ho.default_q2kv(h_q, t)
+    at = n0
+    for ci, m in enumerate(chunks):
+        ret = idx.update(K[:, :, at:at + m], V[:, :, at:at + m])
+        assert ret is idx
+        at += m
+        if ci % 7 and m == 1 and ci < len(chunks) - 1:
+            continue  # check after some of the single-key steps only
+        assert idx.num_keys == at
+        _check_tree(idx, keys[:, :at], vals[:, :at])
+        q = rnd(random_query(h_q, d, seed=at))
+        s = ho.scores(keys[:, :at], q, q2kv)
+        th = midpoint_threshold(s, max(1, at // 20))
+        out = searcher.search(torch.from_numpy(q), torch.from_numpy(th), idx).cpu().numpy()
+        assert out.shape == (h_q, at)
+        assert_same_selection(out != 0, s, th)
+    # attention over the final index
+    sc = torch.full((h_q,), d ** -0.5)
+    att = HIPSearcher().search_attention(torch.from_numpy(q), torch.from_numpy(th), idx,
+                                         scaling=sc).cpu().numpy()
+    ref = ho.attention(keys, vals, q, sc.numpy(), s >= th[:, None], q2kv)
+    assert rel_err(att, ref) <= (2e-3 if dtype == torch.bfloat16 else 1e-5)
+
+
+def test_update_is_reproducible_and_grows_capacity(gpu_device):
+    from hira_amd.indexer.hip import HIPIndexer
+
+    keys = torch.from_numpy(clustered_keys(2, 600, 64, seed=2))[None]
+    a = HIPIndexer(3, 1, 8).build(keys[:, :, :256])
+    b = HIPIndexer(3, 1, 8, capacity=4096).build(keys[:, :, :256])
+    cap0 = list(a.cap)
+    for lo in range(256, 600, 43):
+        a.update(keys[:, :, lo:lo + 43])
+        b.update(keys[:, :, lo:lo + 43])
+    assert a.cap[0] > cap0[0] and a.size == b.size and a.num_keys == b.num_keys == 600
+    n0 = a.size[0]
+    assert torch.equal(a.perm[:, :n0], b.perm[:, :n0])
+    assert torch.equal(a.keys_buf[:, :n0], b.keys_buf[:, :n0])
+    for l in (1, 2):
+        assert torch.equal(a.radii[l][:, : a.size[l]], b.radii[l][:, : a.size[l]])
+
+
+def test_update_rejects_bad_shapes(gpu_device):
+    """tests/test_cuda_indexer_searcher.py:594-607 of the reference."""
+    from hira_amd.indexer.hip import HIPIndexer
+
+    keys = torch.from_numpy(clustered_keys(2, 128, 32, seed=61))[None]
+    idx = HIPIndexer(3, 2, 8).build(keys)
+    with pytest.raises(ValueError):
+        idx.update(torch.randn(2, 2, 7, 32))          # batch 2 on a batch-1 index
+    with pytest.raises(ValueError):
+        idx.update(torch.randn(1, 2, 7, 16))          # wrong dim
+    with pytest.raises(ValueError):
+        idx.update(torch.randn(1, 2, 7, 32), torch.randn(1, 2, 7, 32))  # built without values
+    with pytest.raises(ValueError):
+        HIPIndexer(3, 2, 8).update(torch.randn(1, 2, 7, 32))            # not built
+
+
+def test_cache_layer_end_to_end(gpu_device):
+    """Prefill builds, decode steps queue and flush into the index, the attention function
+    reads the CacheOutput: output == dense softmax attention when every key is selected."""
+    from hira_amd.attention import hira_attention_forward
+    from hira_amd.cache.hira_cache import HiraCacheLayer
+    from hira_amd.cache.hira_config import DeviceMode, HiraConfig
+
+    cfg = HiraConfig(device_mode=DeviceMode.CUDA_ONLY, update_every=4, num_levels=3,
+                     branching_factor=16, max_iterations=1)
+    layer = HiraCacheLayer(cfg.device_mode, cfg.update_every, cfg.get_indexer_kwargs(),
+                           cfg.get_searcher_kwargs())
+    g = torch.Generator().manual_seed(0)
+    h_kv, h_q, d, n0 = 2, 4, 64, 300
+    dev = "cuda"
+    K = torch.randn((1, h_kv, n0 + 10, d), generator=g).to(torch.bfloat16).to(dev)
+    V = torch.randn((1, h_kv, n0 + 10, d), generator=g).to(torch.bfloat16).to(dev)
+    out, _ = layer.update(K[:, :, :n0], V[:, :, :n0])
+    assert out.prefill_keys is not None
+    for step in range(10):
+        out, _ = layer.update(K[:, :, n0 + step:n0 + step + 1], V[:, :, n0 + step:n0 + step + 1])
+        n = n0 + step + 1
+        assert layer.get_seq_length() == n
+        assert out.queued_keys.shape[-2] == (step + 1) % 4
+        q = torch.randn((1, h_q, 1, d), generator=g).to(torch.bfloat16).to(dev)
+        att, _ = hira_attention_forward(None, q, out, None, scaling=d ** -0.5, hira_threshold=-3e38)
+        assert att.shape == (1, 1, h_q, d)
+        kk = K[:, :, :n].float().repeat_interleave(h_q // h_kv, 1)
+        vv = V[:, :, :n].float().repeat_interleave(h_q // h_kv, 1)
+        ref = torch.nn.functional.scaled_dot_product_attention(q.float(), kk, vv, scale=d ** -0.5)
+        err = (att.float().transpose(1, 2) - ref).abs().max() / ref.abs().max()
+        assert float(err) < 1e-2, float(err)
