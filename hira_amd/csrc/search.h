@@ -32,7 +32,7 @@ struct SearchParams {
     const void* queue_values;
     int32_t queue_len, queue_cap;
     // work split
-    int32_t nodes_per_wave;  // level-1 nodes (or pseudo blocks) per wave
+    int32_t nodes_per_wave;  // level-1 nodes (or pseudo blocks) per wave; MFMA kernel: tiles per workgroup
     int32_t tree_blocks;     // workgroups that walk the tree; the rest scan the queue
     int32_t num_nodes;       // level-1 nodes (or pseudo blocks over the keys when L == 1)
     int32_t num_queue_blocks;
@@ -67,7 +67,8 @@ struct SearchPlan {
 
 // search_mfma.hip
 bool mfma_search_supported(const HiraTree* t, const HiraQueue* queue);
-size_t mfma_search_smem(int threads, int gmax, int dim, int bf);
+constexpr int kMfmaThreads = 512;       // workgroup size of the MFMA kernel (8 waves), at most
+constexpr int kMfmaMaxTilesPerWg = 8;  // tiles of 16 level-1 nodes one workgroup walks
 int launch_search_mfma(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
 
 // Element index of (row, column j) inside one tree's (cap, D) matrix.

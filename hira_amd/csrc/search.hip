@@ -392,6 +392,19 @@ static int round_pow2(int v) {
     return r;
 }
 
+// compute units of the current device (asked once)
+static int compute_units() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        cus = n;
+    }
+    return cus;
+}
+
 static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* queue,
                      const HiraLaunch* launch, SearchPlan* plan) {
     HIRA_CHECK_ARG(t && q, "tree and query must not be NULL");
@@ -452,15 +465,29 @@ static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* que
         // one workgroup per tile of 16 level-1 nodes; heads in passes of 16
         plan->gmax = q->max_group < 16 ? q->max_group : 16;
         plan->head_chunks = (q->max_group + 15) / 16;
-        int threads = launch && launch->block_threads ? launch->block_threads : 512;
-        HIRA_CHECK_ARG(threads >= 64 && threads <= 512 && threads % 64 == 0,
-                       "block_threads %d must be a multiple of 64 up to 512", threads);
+        int threads = launch && launch->block_threads ? launch->block_threads : kMfmaThreads;
+        HIRA_CHECK_ARG(threads >= 64 && threads <= kMfmaThreads && threads % 64 == 0,
+                       "block_threads %d must be a multiple of 64 up to %d", threads, kMfmaThreads);
         plan->threads = threads;
-        plan->nodes_per_wave = 0;
+        // a workgroup walks `tpw` consecutive tiles of 16 level-1 nodes: as few as keep
+        // one workgroup per CU in the launch (the kernel runs one at a time on a CU) and at
+        // most 64 partials per head to fold
+        const int tiles = (t->size[1] + 15) / 16;
+        int tpw = launch ? launch->nodes_per_wave : 0;
+        HIRA_CHECK_ARG(tpw >= 0 && tpw <= kMfmaMaxTilesPerWg,
+                       "MFMA kernel: %d tiles per workgroup (at most %d)", tpw, kMfmaMaxTilesPerWg);
+        if (tpw == 0) {
+            tpw = 1;
+            while (tpw < kMfmaMaxTilesPerWg &&
+                   ((int64_t)tiles * t->num_trees * plan->head_chunks > compute_units() * (int64_t)tpw ||
+                    tiles > 64 * tpw))
+                tpw *= 2;
+        }
+        plan->nodes_per_wave = tpw;
         plan->num_nodes = t->size[1];
-        plan->tree_blocks = (t->size[1] + 15) / 16;
+        plan->tree_blocks = (tiles + tpw - 1) / tpw;
         plan->queue_blocks = 0;
-        plan->smem = mfma_search_smem(threads, plan->gmax, t->dim, t->bf);
+        plan->smem = 0;
         return HIRA_OK;
     }
     plan->gmax = q->max_group <= 1 ? 1 : (q->max_group <= 4 ? 4 : 8);

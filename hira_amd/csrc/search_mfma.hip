@@ -13,12 +13,6 @@ bool mfma_search_supported(const HiraTree* t, const HiraQueue* queue) {
     return true;
 }
 
-size_t mfma_search_smem(int threads, int gmax, int dim, int bf) {
-    const int gs = gmax <= 4 ? 4 : (gmax <= 8 ? 8 : 16);
-    const int mt = bf / 16 <= 1 ? 1 : (bf / 16 == 2 ? 2 : 4);
-    return (size_t)(threads / 64) * mfma_wave_floats(dim, mt, gs) * sizeof(float);
-}
-
 // grid: x = tree, y = tile of 16 level-1 nodes, z = pass of 16 heads
 int launch_search_mfma(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s) {
     switch (p.dim) {

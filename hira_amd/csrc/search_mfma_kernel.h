@@ -1,27 +1,31 @@
 // MFMA search + sparse attention kernel: bf16 keys/centers in the tiled layout
 // (HIRA_TILE16), fan-out a multiple of 16, D = Dv in {64, 128, 256}, at least two levels.
 //
-// One workgroup owns one tile of 16 consecutive level-1 nodes of one tree; workgroup ids
-// run fastest over the trees so that, with 8 L2 slices (XCDs) served round-robin, the
-// workgroups of one tree share a slice.  Every wave
-//   1. issues, before it waits for anything, all the loads the gates need: its heads'
-//      queries, the 16 x D tile of level-1 centres, the tiles that hold the ancestors of
-//      that tile (one node per level >= 2), radii and child counts;
-//   2. gates with v_mfma_f32_16x16x32_bf16: a wave-wide 128-bit load fetches a 16 x 32
-//      operand tile from 1 KiB of contiguous memory (that is what the tiled layout is for),
-//      the B operand holds the (up to 16) query heads of the GQA group, so the D registers
-//      hold score(row, head) with head = lane % 16 and row = 4*(lane/16) + j; a node
-//      survives for a head when score + ||q|| r >= tau;
-//   3. takes every NW-th surviving node, loads the key tiles of its child block (all at
-//      once) and scores them the same way; the leaf filter q.k >= tau is a compare against
-//      the lane's own threshold;
-//   4. softmax, vectorised over heads: every lane keeps (m, l) of ITS head, raises m by the
-//      block's best selected score, turns its selected scores into weights 2^(z - m) and
-//      parks them in a wave-private LDS table (row, head); then the value rows of the
-//      selected keys are fetched, 8 loads in flight, each row once however many heads
-//      selected it, and acc[head][:] += weight(row, head) * v[:] runs branch-free with the
-//      accumulators in registers (lane owns Dv/64 columns of every head).
-// The waves' states are merged through LDS into one partial per head and workgroup.
+// One workgroup (8 waves, the only one on its CU) owns a run of consecutive tiles of 16 level-1 nodes of one tree;
+// workgroup ids run fastest over the trees so that, with 8 L2 slices (XCDs) served
+// round-robin, the workgroups of one tree share a slice.  The work is split by phase, not by
+// node, so that neither the key scan nor the value gather depends on where in the tree the
+// selected keys sit:
+//   gate   wave w gates tile w of the run: it issues, before it waits for anything, every
+//          load it needs (queries, the 16 x D tile of level-1 centres, the tiles holding the
+//          tile's ancestors, radii, child counts) and gates with v_mfma_f32_16x16x32_bf16:
+//          a wave-wide 128-bit load fetches a 16 x 32 operand tile from 1 KiB of contiguous
+//          memory (that is what the tiled layout is for), the B operand holds the (up to 16)
+//          query heads of the GQA group, so the D registers hold score(row, head) with
+//          head = lane % 16 and row = 4*(lane/16) + j; a node survives for a head when
+//          score + ||q|| r >= tau.  Head masks and child counts of the nodes go to LDS.
+//   scan   the surviving nodes of the run are dealt round-robin to the waves; in each round
+//          a wave loads the key tiles of NB nodes at once, scores them the same way (leaf
+//          filter: q.k >= tau against the lane's own threshold) and the workgroup builds,
+//          in LDS, one list of the selected rows: slot and one softmax weight per head.  All
+//          waves share one running maximum per head, so their sums need no rescaling when
+//          they are added up.
+//   gather the rows of the list are dealt round-robin to the waves: up to kVBatch value rows
+//          in flight per wave, each row fetched once however many heads selected it,
+//          acc[head][:] += weight(row, head) * v[:] with the accumulators in registers
+//          (lane owns Dv/64 columns of every head).
+// One partial (m, l, acc) per head and workgroup goes to global memory; the last workgroup
+// of a tree to arrive folds the tree's partials.
 //
 // Register arrays are only ever indexed by compile-time constants: a run-time index would
 // push them to scratch memory.
@@ -34,27 +38,38 @@ namespace hira {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
-constexpr int kHeadsPerPass = 16;  // MFMA N
-constexpr int kMaxTiles = 4;       // key tiles per block: bf <= 64
-constexpr int kVBatch = 8;         // value rows in flight per wave
+constexpr int kHeadsPerPass = 16;   // MFMA N
+constexpr int kMaxTiles = 4;        // key tiles per block: bf <= 64
+constexpr int kMfmaWaves = kMfmaThreads / 64;  // waves per workgroup, at most: one workgroup of 8
+                                                // waves on a CU leaves every wave 256 registers
+#ifndef HIRA_VBATCH
+#define HIRA_VBATCH 32
+#endif
+constexpr int kVBatch = HIRA_VBATCH;         // value rows in flight per wave
 
 __device__ __forceinline__ bf16x8_t as_bf16x8(const uint4& v) {
     return __builtin_bit_cast(bf16x8_t, v);
 }
 
-// chunk pointer of tile `tile` of one tree's tiled matrix (D = 32*KS columns)
+// Tile `tile` of one tree's tiled matrix (D = 32*KS columns): a uniform base address, to
+// which every lane adds its own 16 bytes' offset, so that the loads can take the base from
+// scalar registers.
+struct TilePtr {
+    const char* base;  // uniform
+    unsigned lane_off; // lane * 16
+};
 template <int KS>
-__device__ __forceinline__ const uint4* tile_ptr(const void* base, size_t tree_row0, size_t tile,
-                                                 int lane) {
-    return reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(base) +
-                                          tree_row0 * (size_t)(32 * KS)) +
-           tile * (size_t)(KS * 64) + lane;
+__device__ __forceinline__ TilePtr tile_ptr(const void* base, size_t tree_row0, size_t tile, int lane) {
+    return TilePtr{reinterpret_cast<const char*>(base) +
+                       (tree_row0 * (size_t)(32 * KS) * 2 + tile * (size_t)(KS * 1024)),
+                   (unsigned)lane * 16u};
 }
 
 template <int KS>
-__device__ __forceinline__ void load_tile(const uint4* tp, uint4 (&a)[KS]) {
+__device__ __forceinline__ void load_tile(const TilePtr tp, uint4 (&a)[KS]) {
 #pragma unroll
-    for (int s = 0; s < KS; ++s) a[s] = tp[s * 64];
+    for (int s = 0; s < KS; ++s)
+        a[s] = *reinterpret_cast<const uint4*>(tp.base + (size_t)(tp.lane_off + (unsigned)(s * 1024)));
 }
 
 template <int KS>
@@ -63,6 +78,18 @@ __device__ __forceinline__ f32x4_t tile_scores(const uint4 (&a)[KS], const bf16x
 #pragma unroll
     for (int s = 0; s < KS; ++s)
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[s]), bq[s], acc, 0, 0, 0);
+    return acc;
+}
+
+// the same with the B operand parked in LDS (chunk s of lane l at [s*64 + l]): the scan keeps
+// its registers for keys in flight
+template <int KS>
+__device__ __forceinline__ f32x4_t tile_scores_lds(const uint4 (&a)[KS], const uint4* bq_lds, int lane) {
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[s]), as_bf16x8(bq_lds[s * 64 + lane]),
+                                                      acc, 0, 0, 0);
     return acc;
 }
 
@@ -79,30 +106,105 @@ __device__ __forceinline__ void stat_add(unsigned long long* st, int slot, unsig
     if (v) atomicAdd(&st[slot], (unsigned long long)v);
 }
 
-// floats of wave-private LDS: the weight table (MT*16 rows x 16 heads) during the scan,
-// the wave's state (GS x (D + 2)) afterwards
-__host__ __device__ constexpr int mfma_wave_floats(int D, int MT, int GS) {
-    return (GS * (D + 2) > MT * 256) ? GS * (D + 2) : MT * 256;
+// Compile-time shape of one instantiation.
+template <int KS, int MT, int GS>
+struct MfmaShape {
+    static constexpr int D = 32 * KS;
+    static constexpr int ROWS = MT * 16;  // key slots of one node
+    // nodes whose key tiles one wave keeps in flight: what the budget of 256 registers leaves
+    // after twice the accumulators (GS x D/64) and some seventy registers of everything else,
+    // and what keeps the round's list under 48 KiB of LDS
+    static constexpr int KEY_REGS = 256 - 72 - 2 * GS * (KS / 2);
+    static constexpr int NB_REGS = KEY_REGS / (MT * KS * 4);
+    static constexpr int NB_LDS = (12000 / (GS + 1)) / (kMfmaWaves * ROWS);
+    static constexpr int NB_MIN = NB_REGS < NB_LDS ? NB_REGS : NB_LDS;
+    static constexpr int NB = NB_MIN < 1 ? 1 : (NB_MIN > 4 ? 4 : NB_MIN);
+    static constexpr int LIST = kMfmaWaves * NB * ROWS;  // rows of the list of one round
+    static constexpr int SCAN_WORDS = LIST * (GS + 1) + LIST / 16;  // row list, tile slots, GS scores per row
+    static constexpr int MERGE_WORDS = kMfmaWaves * 4 * D;  // four heads of every wave
+    // two lists (rounds alternate, one barrier a round) where that stays under 40 KiB
+    static constexpr int LIST_WORDS = 2 * SCAN_WORDS * 4 <= 40 * 1024 ? 2 * SCAN_WORDS : SCAN_WORDS;
+    static constexpr int WORDS = LIST_WORDS > MERGE_WORDS ? LIST_WORDS : MERGE_WORDS;
+};
+
+// What a wave needs to gate one tile of 16 level-1 nodes, as it comes from memory.
+template <int KS>
+struct GateLoads {
+    uint4 a1[KS];      // the tile of level-1 centres
+    float4 r4;         // radii of rows 4*kb .. 4*kb+3
+    int4 c4;           // child counts of the same rows
+    uint4 anc[2][KS];  // tiles holding the ancestors at levels min(L-1,3) and the one below
+    float arad[2];
+    size_t aid[2];
+};
+
+template <int KS>
+__device__ __forceinline__ void gate_issue(const SearchParams& p, int tree, int t1, int lane,
+                                           int kb, GateLoads<KS>& g) {
+    const int L = p.num_levels;
+    const size_t row1 = (size_t)tree * p.cap[1];
+    load_tile<KS>(tile_ptr<KS>(p.centers[1], row1, (size_t)t1, lane), g.a1);
+    g.r4 = *reinterpret_cast<const float4*>(p.radii[1] + row1 + (size_t)t1 * 16 + 4 * kb);
+    g.c4 = *reinterpret_cast<const int4*>(p.counts[1] + row1 + (size_t)t1 * 16 + 4 * kb);
+    size_t sp = 1;  // level-1 nodes under one node of level min(L-1, 3)
+    for (int l = 2; l <= min(L - 1, 3); ++l) sp *= (size_t)p.bf;
+    const int n_par = min(max(L - 2, 0), 2);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        g.arad[i] = 0.f;
+        g.aid[i] = 0;
+        if (i < n_par) {
+            const int l = min(L - 1, 3) - i;
+            g.aid[i] = ((size_t)t1 * 16) / sp;
+            load_tile<KS>(tile_ptr<KS>(p.centers[l], (size_t)tree * p.cap[l], g.aid[i] / 16, lane),
+                          g.anc[i]);
+            g.arad[i] = p.radii[l][(size_t)tree * p.cap[l] + g.aid[i]];
+            sp /= (size_t)p.bf;
+        }
+    }
 }
 
-template <int KS, int MT, int GS>
-__global__ __launch_bounds__(512, (KS <= 4 ? 4 : 2)) void search_mfma_kernel(const SearchParams p) {
-    constexpr int D = 32 * KS;
-    constexpr int VPL = KS / 2;  // value elements per lane: Dv = D = 64 * VPL
+// OUT: the launch also wants dense scores or selection lists (kept out of the attention-only
+// instantiation, whose registers are all spoken for).
+template <int KS, int MT, int GS, bool OUT>
+__global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const SearchParams p) {
+    using S = MfmaShape<KS, MT, GS>;
+    constexpr int D = S::D;
+    constexpr int NB = S::NB;
+    constexpr int VPL = KS / 2;        // value elements per lane: Dv = D = 64 * VPL
     constexpr int VW = (VPL + 1) / 2;  // dwords of a value row per lane
-    constexpr int WAVE_FLOATS = mfma_wave_floats(D, MT, GS);
-    extern __shared__ float smem[];
+    __shared__ uint32_t s_words[S::WORDS];  // the round's list; the merge; the fold
+    __shared__ uint32_t s_nmask[kMfmaMaxTilesPerWg * 16];  // heads for which a node survives
+    __shared__ int32_t s_ncnt[kMfmaMaxTilesPerWg * 16];    // its child count
+    __shared__ int32_t s_cntw[2][kMfmaWaves];          // rows a wave selected (by round parity)
+    __shared__ float s_mxw[2][kMfmaWaves * 16];        // its best selected score per head
+    __shared__ float s_lw[kMfmaWaves * 16];
+    __shared__ float s_mh[kHeadsPerPass];
+    __shared__ float s_red[2 * kHeadsPerPass];
+    __shared__ int s_nc[kHeadsPerPass];
+    __shared__ int s_last;
+    __shared__ uint4 s_bq[KS * 64];  // the B operand (queries) of the scan
 
     const int lane = lane_id();
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int nw = blockDim.x >> 6;
     const int col = lane & 15;  // head within the pass
     const int kb = lane >> 4;   // column block of 8 inside each 32-column step
     const int tree = blockIdx.x;
-    const int t1 = blockIdx.y;  // tile of level-1 nodes
     const int L = p.num_levels, bf = p.bf;
     const bool want_attn = p.part_acc != nullptr;
+    const int tile0 = (int)blockIdx.y * p.nodes_per_wave;  // first tile of my run
+    const int ntile = min(p.nodes_per_wave, ((p.size[1] + 15) >> 4) - tile0);
+#ifdef HIRA_TIMELINE  // experiment builds only: p.stats receives 8 time stamps per workgroup
+    unsigned long long* stats = nullptr;
+    unsigned long long* tl =
+        p.stats + (((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 16;
+#define HIRA_TL(k) do { if (threadIdx.x == 0) tl[k] = wall_clock64(); } while (0)
+#else
     unsigned long long* stats = p.stats ? p.stats + (size_t)tree * (HIRA_MAX_LEVELS + 2) : nullptr;
+#define HIRA_TL(k) do { } while (0)
+#endif
+    HIRA_TL(0);
 
     // ---- heads of this pass ----------------------------------------------------------
     int hoff, G;
@@ -113,54 +215,27 @@ __global__ __launch_bounds__(512, (KS <= 4 ? 4 : 2)) void search_mfma_kernel(con
         hoff = p.tree_q_off[tree] + blockIdx.z * kHeadsPerPass;
         G = min(kHeadsPerPass, p.tree_q_off[tree + 1] - hoff);
     }
-    if (G <= 0) return;  // uniform
+    if (G <= 0 || ntile <= 0) return;  // uniform
     G = min(G, GS);
     const bool head_ok = col < G;
     int qh = 0;
     if (head_ok) qh = p.group_size > 0 ? hoff + col : p.tree_q_heads[hoff + col];
 
-    // ---- every load the gates need, issued before the first wait ------------------------
+    // ---- queries and the first tile's gate operands, issued before the first wait --------
+    // (only the waves that gate need the queries in registers: the scan reads them from LDS)
+    int tl_mine = wave;  // tile of the run this wave gates next
     uint4 qraw[KS];
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
         qraw[s] = make_uint4(0, 0, 0, 0);
-        if (head_ok)
+        if (head_ok && tl_mine < ntile)
             qraw[s] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.q) +
                                                       (size_t)qh * D + s * 32 + kb * 8);
     }
     const float tau = head_ok ? p.tau[qh] : INFINITY;
     const float sc = head_ok ? p.scaling[qh] : 0.0f;
-
-    const size_t row1 = (size_t)tree * p.cap[1];
-    uint4 a1[KS];
-    load_tile<KS>(tile_ptr<KS>(p.centers[1], row1, (size_t)t1, lane), a1);
-    const float4 r4 = *reinterpret_cast<const float4*>(p.radii[1] + row1 + (size_t)t1 * 16 + 4 * kb);
-    const int4 c4 = *reinterpret_cast<const int4*>(p.counts[1] + row1 + (size_t)t1 * 16 + 4 * kb);
-
-    // ancestors: levels L-1 .. 2; the two lowest ones (3 and 2) are fetched right away
-    size_t span = 1;  // level-1 nodes under one node of the current level
-    for (int l = 2; l < L; ++l) span *= (size_t)bf;
-    int lcur = L - 1;
-    size_t span_hi = span;
-    for (int l = L - 1; l > 3; --l) span_hi /= (size_t)bf;  // span at level min(L-1, 3)
-    const int n_par = min(max(L - 2, 0), 2);                // ancestor levels fetched in parallel
-    uint4 anc[2][KS];
-    float arad[2] = {0.f, 0.f};
-    size_t aid[2] = {0, 0};
-    {
-        size_t sp = span_hi;
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            if (i < n_par) {
-                const int l = min(L - 1, 3) - i;
-                aid[i] = ((size_t)t1 * 16) / sp;
-                load_tile<KS>(tile_ptr<KS>(p.centers[l], (size_t)tree * p.cap[l], aid[i] / 16, lane),
-                              anc[i]);
-                arad[i] = p.radii[l][(size_t)tree * p.cap[l] + aid[i]];
-                sp /= (size_t)bf;
-            }
-        }
-    }
+    GateLoads<KS> gl;
+    if (tl_mine < ntile) gate_issue<KS>(p, tree, tile0 + tl_mine, lane, kb, gl);
 
     // ---- B operand and ||q|| -----------------------------------------------------------
     bf16x8_t bq[KS];
@@ -176,256 +251,381 @@ __global__ __launch_bounds__(512, (KS <= 4 ? 4 : 2)) void search_mfma_kernel(con
     ss += __shfl_xor(ss, 16, 64);
     ss += __shfl_xor(ss, 32, 64);
     const float qn = sqrtf(ss);
-    const bool count_nodes = stats != nullptr && wave == 0 && lane == 0;
-
-    // ---- ancestor gates, top-down ---------------------------------------------------------
-    bool chain = head_ok;  // this head is still alive above the current level
-    for (; lcur > 3; --lcur) {  // trees deeper than four levels: one level at a time
-        const size_t a = ((size_t)t1 * 16) / span;
-        uint4 t[KS];
-        load_tile<KS>(tile_ptr<KS>(p.centers[lcur], (size_t)tree * p.cap[lcur], a / 16, lane), t);
-        const float rad = p.radii[lcur][(size_t)tree * p.cap[lcur] + a];
-        const bool any_alive = __ballot(chain) != 0ull;
-        if (count_nodes && ((size_t)t1 * 16) % span == 0 && any_alive && rad > -INFINITY)
-            stat_add(stats, lcur, 1u);
-        const float d = row_score(tile_scores<KS>(t, bq), (int)(a % 16), col);
-        chain = chain && (d + qn * rad >= tau);
-        span /= (size_t)bf;
-    }
+    if (wave == 0) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        if (i < n_par) {
+        for (int s = 0; s < KS; ++s) s_bq[s * 64 + lane] = qraw[s];
+    }
+
+    // ---- gate: one tile per wave at a time ------------------------------------------------
+    while (tl_mine < ntile) {  // uniform in the wave
+        const int t1 = tile0 + tl_mine;
+        const bool count_nodes = stats != nullptr && lane == 0;
+        size_t span = 1;  // level-1 nodes under one node of the current level
+        for (int l = 2; l < L; ++l) span *= (size_t)bf;
+        int lcur = L - 1;
+        bool chain = head_ok;  // this head is still alive above the current level
+        for (; lcur > 3; --lcur) {  // trees deeper than four levels: one level at a time
+            const size_t a = ((size_t)t1 * 16) / span;
+            uint4 t[KS];
+            load_tile<KS>(tile_ptr<KS>(p.centers[lcur], (size_t)tree * p.cap[lcur], a / 16, lane), t);
+            const float rad = p.radii[lcur][(size_t)tree * p.cap[lcur] + a];
             const bool any_alive = __ballot(chain) != 0ull;
-            if (count_nodes && ((size_t)t1 * 16) % span == 0 && any_alive && arad[i] > -INFINITY)
+            if (count_nodes && ((size_t)t1 * 16) % span == 0 && any_alive && rad > -INFINITY)
                 stat_add(stats, lcur, 1u);
-            const float d = row_score(tile_scores<KS>(anc[i], bq), (int)(aid[i] % 16), col);
-            chain = chain && (d + qn * arad[i] >= tau);
+            const float d = row_score(tile_scores<KS>(t, bq), (int)(a % 16), col);
+            chain = chain && (d + qn * rad >= tau);
             span /= (size_t)bf;
-            --lcur;
         }
-    }
-    const bool tile_live = __ballot(chain) != 0ull;  // uniform
-
-    // ---- level-1 gates: 16 nodes at once ----------------------------------------------------
-    unsigned alive4 = 0u;
-    const int cc[4] = {c4.x, c4.y, c4.z, c4.w};
-    if (tile_live) {
-        const f32x4_t g1 = tile_scores<KS>(a1, bq);
-        const float rr[4] = {r4.x, r4.y, r4.z, r4.w};
-        unsigned real = 0u;
+        const int n_par = min(max(L - 2, 0), 2);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            if (chain && (g1[j] + qn * rr[j] >= tau)) alive4 |= 1u << j;
-            if (stats) real += (unsigned)__popcll(__ballot(col == 0 && rr[j] > -INFINITY));
+        for (int i = 0; i < 2; ++i) {
+            if (i < n_par) {
+                const bool any_alive = __ballot(chain) != 0ull;
+                if (count_nodes && ((size_t)t1 * 16) % span == 0 && any_alive &&
+                    gl.arad[i] > -INFINITY)
+                    stat_add(stats, lcur, 1u);
+                const float d = row_score(tile_scores<KS>(gl.anc[i], bq), (int)(gl.aid[i] % 16), col);
+                chain = chain && (d + qn * gl.arad[i] >= tau);
+                span /= (size_t)bf;
+                --lcur;
+            }
         }
-        if (count_nodes) stat_add(stats, 1, real);
-    }
-    unsigned long long nb[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) nb[j] = __ballot((alive4 >> j) & 1u);
+        const bool tile_live = __ballot(chain) != 0ull;  // uniform
 
-    // ---- softmax state: (m, l) of this lane's head; acc[g][e] = column lane*VPL + e of head g
-    float* wl = smem + (size_t)wave * WAVE_FLOATS;  // weight table (row, head) during the scan
+        // level-1 gates: 16 nodes at once
+        unsigned alive4 = 0u;
+        const int cc[4] = {gl.c4.x, gl.c4.y, gl.c4.z, gl.c4.w};
+        if (tile_live) {
+            const f32x4_t g1 = tile_scores<KS>(gl.a1, bq);
+            const float rr[4] = {gl.r4.x, gl.r4.y, gl.r4.z, gl.r4.w};
+            unsigned real = 0u;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (chain && (g1[j] + qn * rr[j] >= tau)) alive4 |= 1u << j;
+                if (stats) real += (unsigned)__popcll(__ballot(col == 0 && rr[j] > -INFINITY));
+            }
+            if (count_nodes) stat_add(stats, 1, real);
+        }
+        unsigned long long nb[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) nb[j] = __ballot((alive4 >> j) & 1u);
+        // node n = 4*kb' + j of the tile: its heads are field kb' of nb[j]
+        if (lane < 16) {
+            const int jn = lane & 3;
+            const unsigned long long bits = jn == 0 ? nb[0] : (jn == 1 ? nb[1] : (jn == 2 ? nb[2] : nb[3]));
+            s_nmask[tl_mine * 16 + lane] = (uint32_t)((bits >> (16 * (lane >> 2))) & 0xFFFFull);
+        }
+        if (col == 0) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) s_ncnt[tl_mine * 16 + 4 * kb + j] = cc[j];
+        }
+        tl_mine += nw;
+        if (tl_mine < ntile) gate_issue<KS>(p, tree, tile0 + tl_mine, lane, kb, gl);
+    }
+    HIRA_TL(7);
+    __syncthreads();
+    HIRA_TL(1);
+
+    // ---- the surviving nodes of the run, dealt round-robin to the waves ----------------------
+    unsigned long long my0, my1;  // bit n: node n (n + 64) of the run survives and is mine
+    int rounds;
+    {
+        const int NT = ntile * 16;
+        const bool a0 = lane < NT && s_nmask[lane] != 0u;
+        const bool a1 = lane + 64 < NT && s_nmask[lane + 64] != 0u;
+        const unsigned long long A0 = __ballot(a0), A1 = __ballot(a1);
+        const unsigned long long lt = (1ull << lane) - 1ull;
+        const int r0 = __popcll(A0 & lt), r1 = __popcll(A0) + __popcll(A1 & lt);
+        my0 = __ballot(a0 && (r0 % nw) == wave);
+        my1 = __ballot(a1 && (r1 % nw) == wave);
+        const int alive = __popcll(A0) + __popcll(A1);
+        rounds = ((alive + nw - 1) / nw + NB - 1) / NB;
+    }
+
+    // ---- softmax state: running maximum m of the lane's head (the same in every wave);
+    // per wave: l over the rows it gathered, acc[g][e] = column lane*VPL + e of head g -------
+    constexpr bool DB = S::LIST_WORDS == 2 * S::SCAN_WORDS;  // room for a second list: one barrier a round
     const float sc2 = sc * kLog2e;
     const size_t row0 = (size_t)tree * p.cap[0];
-    float m_h = -INFINITY, l_h = 0.0f;
+    float m_run = -INFINITY;
+    float l_mine = 0.0f;  // this lane's share of l of head lane % GS, over the rows this wave gathered
     float acc[GS][VPL];
 #pragma unroll
     for (int g = 0; g < GS; ++g)
 #pragma unroll
         for (int e = 0; e < VPL; ++e) acc[g][e] = 0.0f;
 
-    // ---- my share of the surviving nodes: every nw-th one --------------------------------
-    unsigned mine16 = 0u;  // bit n: level-1 node n of the tile survives and is mine
-    {
-        int k_alive = 0;
+    for (int r = 0; r < rounds; ++r) {  // uniform in the workgroup
+        const int par = r & 1;
+        // the round's list: row -> key slot and one scaled score per head (-inf: not selected);
+        // every wave fills its own stretch of ROWS * NB rows
+        uint32_t* lst_row = s_words + (DB ? par * S::SCAN_WORDS : 0);  // (LIST) listed row -> table row
+        uint32_t* lst_tslot = lst_row + S::LIST;                       // (LIST/16) table tile -> key slot
+        float* lst_z = reinterpret_cast<float*>(lst_tslot + S::LIST / 16);  // (LIST, GS) the table
+        if (!DB && want_attn && r > 0) __syncthreads();  // the previous list has been gathered
+
+        // ---- scan: key tiles of up to NB nodes in flight -----------------------------------
+        int node[NB], cnt[NB];
+        uint32_t nmask[NB];
+        uint4 a[NB][MT][KS];
 #pragma unroll
-        for (int n = 0; n < 16; ++n) {
-            if (((nb[n & 3] >> (16 * (n >> 2))) & 0xFFFFull) != 0ull) {
-                if (k_alive == wave) mine16 |= 1u << n;
-                if (++k_alive == nw) k_alive = 0;
+        for (int u = 0; u < NB; ++u) {
+            int n = -1;
+            if (my0 != 0ull) {
+                n = __ffsll((long long)my0) - 1;
+                my0 &= my0 - 1ull;
+            } else if (my1 != 0ull) {
+                n = 64 + __ffsll((long long)my1) - 1;
+                my1 &= my1 - 1ull;
             }
+            node[u] = n;
+            cnt[u] = __builtin_amdgcn_readfirstlane(n >= 0 ? s_ncnt[n] : 0);
+            nmask[u] = (uint32_t)__builtin_amdgcn_readfirstlane((int)(n >= 0 ? s_nmask[n] : 0u));
+            const size_t tile_first = ((size_t)(tile0 * 16 + max(n, 0)) * bf) / 16;
+#pragma unroll
+            for (int tt = 0; tt < MT; ++tt)
+                if (tt * 16 < cnt[u])
+                    load_tile<KS>(tile_ptr<KS>(p.keys, row0, tile_first + tt, lane), a[u][tt]);
         }
-    }
 
-    while (mine16 != 0u) {  // uniform
-        const int n = __ffs(mine16) - 1;
-        mine16 &= mine16 - 1u;
-        const int jn = n & 3;
-        const unsigned long long nbits = jn == 0 ? nb[0] : (jn == 1 ? nb[1] : (jn == 2 ? nb[2] : nb[3]));
-        const unsigned node_mask = (unsigned)((nbits >> (16 * (n >> 2))) & 0xFFFFull);
-        const int cnt = __shfl(jn == 0 ? cc[0] : (jn == 1 ? cc[1] : (jn == 2 ? cc[2] : cc[3])),
-                               16 * (n >> 2), 64);
-        const size_t slot0 = (size_t)(t1 * 16 + n) * bf;
-        const bool my_alive = (node_mask >> col) & 1u;
-        if (stats && lane == 0) stat_add(stats, 0, (unsigned)cnt);
+        // all the products first: the operand registers are free before the bookkeeping starts
+        f32x4_t sco_all[NB][MT];
+#pragma unroll
+        for (int u = 0; u < NB; ++u)
+#pragma unroll
+            for (int tt = 0; tt < MT; ++tt)  // (only read where it is written: under this condition)
+                if (tt * 16 < cnt[u]) sco_all[u][tt] = tile_scores_lds<KS>(a[u][tt], s_bq, lane);
 
-        // all key tiles of the block in flight at once
-        uint4 a[MT][KS];
-#pragma unroll
-        for (int tt = 0; tt < MT; ++tt)
-            if (tt * 16 < cnt) load_tile<KS>(tile_ptr<KS>(p.keys, row0, slot0 / 16 + tt, lane), a[tt]);
+        if (r == 0) HIRA_TL(8);
+        // The bookkeeping below derives everything per-lane from this copy, which the compiler
+        // cannot see through: otherwise it computes those values once, ahead of the loop, and
+        // they crowd out the registers that the loads above need.
+        int lane_o = lane;
+        asm volatile("" : "+v"(lane_o));
+        const int col = lane_o & 15, kb = lane_o >> 4;
 
-        f32x4_t sco[MT];
-        unsigned sel4[MT];
-        unsigned long long sb[MT][4];
-        unsigned long long any = 0ull;
+        int nsel = 0;  // rows of my stretch of the list
+        float zmax = -INFINITY;
+        const int zrow0 = wave * (NB * S::ROWS);  // my stretch of the round's rows
 #pragma unroll
-        for (int tt = 0; tt < MT; ++tt) {
-            sel4[tt] = 0u;
-            sco[tt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-            if (tt * 16 < cnt) {
-                sco[tt] = tile_scores<KS>(a[tt], bq);
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    if (my_alive && (tt * 16 + 4 * kb + j) < cnt && sco[tt][j] >= tau) sel4[tt] |= 1u << j;
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                sb[tt][j] = __ballot((sel4[tt] >> j) & 1u);
-                any |= sb[tt][j];
-            }
-        }
-        if (any == 0ull) continue;  // uniform: nothing selected in this block
-
-        // ---- dense scores / compact lists ----------------------------------------------------
-        if (p.dense != nullptr || p.sel_count != nullptr) {
+        for (int u = 0; u < NB; ++u) {
+            // a head for which the node did not survive selects nothing
+            const float tau_u = ((nmask[u] >> col) & 1u) ? tau : INFINITY;
+            const unsigned slot0 = (unsigned)((tile0 * 16 + max(node[u], 0)) * bf);
+            if (stats && lane == 0) stat_add(stats, 0, (unsigned)cnt[u]);
 #pragma unroll
             for (int tt = 0; tt < MT; ++tt) {
-                if ((sb[tt][0] | sb[tt][1] | sb[tt][2] | sb[tt][3]) == 0ull) continue;
-                const unsigned tslot = (unsigned)(slot0 + tt * 16);
-                int base = 0;
-                if (p.sel_count != nullptr) {  // one atomic per head of the tile (lane g, kb = 0)
-                    int mine = 0;
+                if (tt * 16 >= cnt[u]) continue;  // uniform
+                const f32x4_t sco = sco_all[u][tt];
+                const int lim = cnt[u] - tt * 16 - 4 * kb;  // my rows j < lim hold keys
+                unsigned sel4 = 0u;
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        mine += __popcll(sb[tt][j] & (0x0001000100010001ull << col));
-                    int b0 = 0;
-                    if (kb == 0 && mine > 0) b0 = atomicAdd(&p.sel_count[qh], mine);
-                    base = __shfl(b0, col, 64);
+                for (int j = 0; j < 4; ++j)
+                    if (sco[j] >= tau_u && j < lim) sel4 |= 1u << j;
+                if (__ballot(sel4 != 0u) == 0ull) continue;  // uniform
+                // rows selected by some head: OR over the 16 lanes (heads) of my row group by
+                // rotating inside the group, then the four groups side by side
+                unsigned any4 = sel4;
+                any4 |= (unsigned)__builtin_amdgcn_update_dpp(0, (int)any4, 0x121, 0xF, 0xF, false);
+                any4 |= (unsigned)__builtin_amdgcn_update_dpp(0, (int)any4, 0x122, 0xF, 0xF, false);
+                any4 |= (unsigned)__builtin_amdgcn_update_dpp(0, (int)any4, 0x124, 0xF, 0xF, false);
+                any4 |= (unsigned)__builtin_amdgcn_update_dpp(0, (int)any4, 0x128, 0xF, 0xF, false);
+                const unsigned rowmask = (unsigned)__builtin_amdgcn_readlane((int)any4, 0) |
+                                         ((unsigned)__builtin_amdgcn_readlane((int)any4, 16) << 4) |
+                                         ((unsigned)__builtin_amdgcn_readlane((int)any4, 32) << 8) |
+                                         ((unsigned)__builtin_amdgcn_readlane((int)any4, 48) << 12);
+                if (stats) {
+                    const unsigned pairs = (unsigned)__popcll(__ballot(sel4 & 1u)) +
+                                           (unsigned)__popcll(__ballot(sel4 & 2u)) +
+                                           (unsigned)__popcll(__ballot(sel4 & 4u)) +
+                                           (unsigned)__popcll(__ballot(sel4 & 8u));
+                    if (lane == 0) {
+                        stat_add(stats, HIRA_MAX_LEVELS, (unsigned)__popc(rowmask));
+                        stat_add(stats, HIRA_MAX_LEVELS + 1, pairs);
+                    }
                 }
+                const unsigned tslot = slot0 + tt * 16;
+
+                // ---- dense scores / compact lists ------------------------------------------
+                if (OUT && (p.dense != nullptr || p.sel_count != nullptr)) {
+                    unsigned long long sb[4];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    if ((sel4[tt] >> j) & 1u) {
-                        const unsigned slot = tslot + 4 * kb + j;
-                        int idx = (int)slot;
-                        if (p.dense_by_position) idx = p.perm[row0 + slot];
-                        if (p.dense != nullptr)
-                            p.dense[(int64_t)qh * p.dense_stride + idx] = sco[tt][j] * sc;
-                        if (p.sel_count != nullptr) {
-                            // hits of my head ordered before (kb, j): rows j' < j of any kb,
-                            // then row j of lower kb
-                            int before = 0;
+                    for (int j = 0; j < 4; ++j) sb[j] = __ballot((sel4 >> j) & 1u);
+                    int base = 0;
+                    if (p.sel_count != nullptr) {  // one atomic per head of the tile (kb = 0)
+                        int mine = 0;
 #pragma unroll
-                            for (int j2 = 0; j2 < 4; ++j2) {
-                                unsigned long long bits = sb[tt][j2] & (0x0001000100010001ull << col);
-                                if (j2 == j) bits &= (1ull << (16 * kb)) - 1ull;
-                                if (j2 <= j) before += __popcll(bits);
-                            }
-                            const int pos = base + before;
-                            if (pos < p.sel_cap) {
-                                p.sel_index[(int64_t)qh * p.sel_cap + pos] = idx;
-                                p.sel_score[(int64_t)qh * p.sel_cap + pos] = sco[tt][j];
+                        for (int j = 0; j < 4; ++j)
+                            mine += __popcll(sb[j] & (0x0001000100010001ull << col));
+                        int b0 = 0;
+                        if (kb == 0 && mine > 0) b0 = atomicAdd(&p.sel_count[qh], mine);
+                        base = __shfl(b0, col, 64);
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if ((sel4 >> j) & 1u) {
+                            const unsigned slot = tslot + 4 * kb + j;
+                            int idx = (int)slot;
+                            if (p.dense_by_position) idx = p.perm[row0 + slot];
+                            if (p.dense != nullptr)
+                                p.dense[(int64_t)qh * p.dense_stride + idx] = sco[j] * sc;
+                            if (p.sel_count != nullptr) {
+                                // hits of my head ordered before (kb, j): rows j' < j of any
+                                // kb, then row j of lower kb
+                                int before = 0;
+#pragma unroll
+                                for (int j2 = 0; j2 < 4; ++j2) {
+                                    unsigned long long bits = sb[j2] & (0x0001000100010001ull << col);
+                                    if (j2 == j) bits &= (1ull << (16 * kb)) - 1ull;
+                                    if (j2 <= j) before += __popcll(bits);
+                                }
+                                const int pos = base + before;
+                                if (pos < p.sel_cap) {
+                                    p.sel_index[(int64_t)qh * p.sel_cap + pos] = idx;
+                                    p.sel_score[(int64_t)qh * p.sel_cap + pos] = sco[j];
+                                }
                             }
                         }
                     }
                 }
+
+                // ---- the tile's scores go to the table, its selected rows join my list -----------
+                if (want_attn) {
+                    const int trow = zrow0 + (u * MT + tt) * 16;  // the tile's rows in the table
+                    float zs[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        zs[j] = ((sel4 >> j) & 1u) ? sco[j] * sc2 : -INFINITY;
+                        zmax = fmaxf(zmax, zs[j]);
+                    }
+                    if (col < GS) {
+                        float* zp = lst_z + (trow + 4 * kb) * GS + col;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) zp[j * GS] = zs[j];
+                    }
+                    if (lane_o < 16 && ((rowmask >> lane_o) & 1u))
+                        lst_row[zrow0 + nsel + __popc(rowmask & ((1u << lane_o) - 1u))] = (uint32_t)(trow + lane_o);
+                    if (lane_o == 0) lst_tslot[trow >> 4] = tslot;
+                }
+                nsel += __popc(rowmask);
             }
         }
-        if (stats && lane == 0) {
-            unsigned pairs = 0, rows = 0;
-#pragma unroll
-            for (int tt = 0; tt < MT; ++tt)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    pairs += (unsigned)__popcll(sb[tt][j]);
-#pragma unroll
-                    for (int q4 = 0; q4 < 4; ++q4) rows += ((sb[tt][j] >> (16 * q4)) & 0xFFFFull) != 0ull;
-                }
-            stat_add(stats, HIRA_MAX_LEVELS, rows);
-            stat_add(stats, HIRA_MAX_LEVELS + 1, pairs);
-        }
-        if (!want_attn) continue;
+        if (!want_attn) continue;  // uniform in the launch
 
-        // ---- softmax bookkeeping, one head per lane -------------------------------------------
-        float zmax = -INFINITY;
-#pragma unroll
-        for (int tt = 0; tt < MT; ++tt)
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                if ((sel4[tt] >> j) & 1u) zmax = fmaxf(zmax, sco[tt][j] * sc2);
+        // ---- every wave learns all counts and the best scores of the round ---------------------
         zmax = fmaxf(zmax, __shfl_xor(zmax, 16, 64));
         zmax = fmaxf(zmax, __shfl_xor(zmax, 32, 64));
-        const float mnew = fmaxf(m_h, zmax);
-        // rescale factor of what this head has accumulated so far (1 if nothing changes)
-        const float f = (zmax == -INFINITY || m_h == mnew) ? 1.0f : exp2f(m_h - mnew);
-        float lsum = 0.0f;
+        if (r == 0) HIRA_TL(9);
+        if (lane == 0) s_cntw[par][wave] = nsel;
+        if (kb == 0) s_mxw[par][wave * 16 + col] = zmax;
+        __syncthreads();
+        int cw[kMfmaWaves];
+        int tot = 0;
+        float rmax = -INFINITY;
+        {
+            // one read each, then lane by lane: no wait between the waves' entries
+            const int cv = s_cntw[par][lane_o & (kMfmaWaves - 1)];
+            float mv[kMfmaWaves];
 #pragma unroll
-        for (int tt = 0; tt < MT; ++tt)
+            for (int w = 0; w < kMfmaWaves; ++w) mv[w] = s_mxw[par][w * 16 + col];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float w = ((sel4[tt] >> j) & 1u) ? exp2f(sco[tt][j] * sc2 - mnew) : 0.0f;
-                lsum += w;
-                wl[(tt * 16 + 4 * kb + j) * 16 + col] = w;
+            for (int w = 0; w < kMfmaWaves; ++w) {
+                cw[w] = w < nw ? __builtin_amdgcn_readlane(cv, w) : 0;
+                tot += cw[w];
+                if (w < nw) rmax = fmaxf(rmax, mv[w]);
             }
-        lsum += __shfl_xor(lsum, 16, 64);
-        lsum += __shfl_xor(lsum, 32, 64);
-        l_h = l_h * f + lsum;
-        m_h = mnew;
+        }
+#ifdef HIRA_TIMELINE
+        if (r == 0) HIRA_TL(10);
+        if (threadIdx.x == 0 && r == 0) { tl[6] = (unsigned long long)tot; tl[12] = (unsigned long long)rounds; }
+#endif
+        if (tot == 0) continue;  // uniform in the workgroup: nothing selected in this round
+
+        // the new maximum of every head, and what it does to the sums so far; head g lives in
+        // lane g; the weights below are computed with lane = (row, head), head = lane % GS
+        const float mnew = fmaxf(m_run, rmax);
+        const float f = (m_run == mnew) ? 1.0f : exp2f(m_run - mnew);
+        m_run = mnew;
+        // a head without a selected key has m = -inf and only z = -inf: any finite stand-in
+        const float m_lane = __shfl(mnew == -INFINITY ? 0.0f : mnew, lane_o & (GS - 1), 64);
         if (__ballot(f != 1.0f) != 0ull) {  // uniform
+            l_mine *= __shfl(f, lane_o & (GS - 1), 64);
 #pragma unroll
             for (int g = 0; g < GS; ++g) {
-                const float fg = __shfl(f, g, 64);
+                const float fg = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), g));
 #pragma unroll
                 for (int e = 0; e < VPL; ++e) acc[g][e] *= fg;
             }
         }
 
-        // ---- value rows of the selected keys: each row once, kVBatch loads in flight --------
-        unsigned long long rowmask = 0ull;  // bit tt*16 + r
+        // ---- gather: list rows wave, wave + nw, ...; kVBatch value rows in flight --------------
+        constexpr int RP = 64 / GS;          // rows whose weights one pass over the lanes computes
+        constexpr int NPASS = kVBatch / RP;  // GS = 4: 1, GS = 8: 2, GS = 16: 4
+        const char* vtree = reinterpret_cast<const char*>(p.values) + row0 * (size_t)(D * 2);
+        // where the rows of a batch sit (row `le` of the round is row `rem` of the stretch of the
+        // wave it falls in; lane = (row of the pass, head)), and their value rows
+        auto issue = [&](int e0, int (&at_v)[NPASS], uint32_t (&vraw)[kVBatch][VW]) {
 #pragma unroll
-        for (int tt = 0; tt < MT; ++tt)
+            for (int ps = 0; ps < NPASS; ++ps) {
+                const int le = e0 + (ps * RP + lane_o / GS) * nw;
+                int rem = le, at = -1;
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
-                if (((sb[tt][r & 3] >> (16 * (r >> 2))) & 0xFFFFull) != 0ull)
-                    rowmask |= 1ull << (tt * 16 + r);
-        while (rowmask != 0ull) {  // uniform
-            int rows[kVBatch];
-            uint32_t vraw[kVBatch][VW];
+                for (int w = 0; w < kMfmaWaves; ++w) {
+                    if (at < 0 && rem < cw[w]) at = w * (NB * S::ROWS) + rem;
+                    rem -= cw[w];
+                }
+                // -> its row in the score table (-1: past the end)
+                at_v[ps] = (le < tot && at >= 0) ? (int)lst_row[at] : -1;
+            }
+            int slot_v[NPASS];  // the key slots of all the rows of a pass
 #pragma unroll
-            for (int u = 0; u < kVBatch; ++u) {
-                rows[u] = -1;
+            for (int ps = 0; ps < NPASS; ++ps)
+                slot_v[ps] = at_v[ps] >= 0 ? (int)(lst_tslot[at_v[ps] >> 4] + (unsigned)(at_v[ps] & 15)) : 0;
+            // (a batch is always loaded whole, rows past the end as slot 0: straight-line code)
 #pragma unroll
-                for (int e = 0; e < VW; ++e) vraw[u][e] = 0u;
-                if (rowmask != 0ull) {
-                    const int r = __ffsll((long long)rowmask) - 1;
-                    rowmask &= rowmask - 1ull;
-                    rows[u] = r;
-                    const uint16_t* vp = reinterpret_cast<const uint16_t*>(p.values) +
-                                         (row0 + slot0 + r) * (size_t)D + lane * VPL;
+            for (int i = 0; i < kVBatch; ++i) {
+                {
+                    const unsigned slot = (unsigned)__builtin_amdgcn_readlane(slot_v[i / RP], (i % RP) * GS);
+                    const uint16_t* vp =
+                        reinterpret_cast<const uint16_t*>(vtree + (size_t)slot * (D * 2)) + lane_o * VPL;
                     if (VPL == 1) {
-                        vraw[u][0] = *vp;
+                        vraw[i][0] = *vp;
                     } else {
 #pragma unroll
                         for (int e = 0; e < VPL / 2; ++e)
-                            vraw[u][e] = reinterpret_cast<const uint32_t*>(vp)[e];
+                            vraw[i][e] = reinterpret_cast<const uint32_t*>(vp)[e];
                     }
                 }
             }
+        };
+        auto consume = [&](int e0, const int (&at_v)[NPASS], const uint32_t (&vraw)[kVBatch][VW]) {
+            // (nothing of what follows may be scheduled ahead of loads issued before this point)
+            __builtin_amdgcn_sched_barrier(0);
+            // scores -> weights, in place, 64 (row, head) pairs at a time
 #pragma unroll
-            for (int u = 0; u < kVBatch; ++u) {
-                if (rows[u] < 0) break;  // uniform
+            for (int ps = 0; ps < NPASS; ++ps) {
+                if (at_v[ps] >= 0) {
+                    float* zp = lst_z + at_v[ps] * GS + (lane_o & (GS - 1));
+                    const float w = __builtin_amdgcn_exp2f(*zp - m_lane);
+                    l_mine += w;
+                    *zp = w;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < kVBatch; ++i) {
+                if (e0 + i * nw >= tot) break;  // uniform
+                const int at = __builtin_amdgcn_readlane(at_v[i / RP], (i % RP) * GS);
                 float vf[VPL];
                 if (VPL == 1) {
-                    vf[0] = bf16_lo(vraw[u][0]);
+                    vf[0] = bf16_lo(vraw[i][0]);
                 } else {
 #pragma unroll
                     for (int e = 0; e < VPL / 2; ++e) {
-                        vf[2 * e] = bf16_lo(vraw[u][e]);
-                        vf[2 * e + 1] = bf16_hi(vraw[u][e]);
+                        vf[2 * e] = bf16_lo(vraw[i][e]);
+                        vf[2 * e + 1] = bf16_hi(vraw[i][e]);
                     }
                 }
-                const float* wr = wl + rows[u] * 16;  // weights of this row, one per head
+                const float* wr = lst_z + at * GS;  // weights of this row, one per head
 #pragma unroll
                 for (int g = 0; g < GS; ++g) {
                     const float w = wr[g];  // same address in every lane: a broadcast read
@@ -433,50 +633,62 @@ __global__ __launch_bounds__(512, (KS <= 4 ? 4 : 2)) void search_mfma_kernel(con
                     for (int e = 0; e < VPL; ++e) acc[g][e] += w * vf[e];
                 }
             }
+        };
+        for (int e0 = wave; e0 < tot; e0 += nw * kVBatch) {  // uniform in the wave
+            int at_v[NPASS];
+            uint32_t vraw[kVBatch][VW];
+            issue(e0, at_v, vraw);
+            consume(e0, at_v, vraw);
         }
+        if (r == 0) HIRA_TL(11);
     }
     if (!want_attn) return;  // uniform
+    HIRA_TL(2);
 
-    // ---- the wave's state goes to LDS: (GS, D + 2) = acc[D], m, l per head ----------------
-    float* wsm = smem + (size_t)wave * WAVE_FLOATS;
+    // ---- merge the waves: same m everywhere, so l and acc simply add up ------------------------
 #pragma unroll
-    for (int g = 0; g < GS; ++g)
-#pragma unroll
-        for (int e = 0; e < VPL; ++e) wsm[g * (D + 2) + lane * VPL + e] = acc[g][e];
-    if (kb == 0 && col < GS) {
-        wsm[col * (D + 2) + D] = m_h;
-        wsm[col * (D + 2) + D + 1] = l_h;
-    }
-    __syncthreads();
-
-    // ---- merge the waves' states into this workgroup's partial ------------------------------
+    for (int off = GS; off < 64; off <<= 1) l_mine += __shfl_xor(l_mine, off, 64);
+    if (lane < GS) s_lw[wave * 16 + lane] = l_mine;
+    if (wave == 0 && kb == 0) s_mh[col] = m_run;
+    int tid = threadIdx.x;  // (opaque, like lane_o above: nothing of the merge is computed early)
+    asm volatile("" : "+v"(tid));
+    float* macc = reinterpret_cast<float*>(s_words);  // (nw, 4, D): four heads at a time
     const int P = p.num_parts;
-    for (int t = threadIdx.x; t < G * D; t += blockDim.x) {
-        const int g = t / D, e = t % D;
-        float mall = -INFINITY;
-        for (int w = 0; w < nw; ++w) mall = fmaxf(mall, smem[(size_t)w * WAVE_FLOATS + g * (D + 2) + D]);
-        float a_sum = 0.0f, lsum = 0.0f;
-        for (int w = 0; w < nw; ++w) {
-            const float* ws = smem + (size_t)w * WAVE_FLOATS + g * (D + 2);
-            const float mw = ws[D];
-            const float f = (mw == -INFINITY) ? 0.0f : exp2f(mw - mall);
-            a_sum += ws[e] * f;
-            lsum += ws[D + 1] * f;
-        }
-        const int head = p.group_size > 0 ? hoff + g : p.tree_q_heads[hoff + g];
-        const size_t slot = (size_t)head * P + t1;
-        // device-scope stores: written through, so that the workgroup that folds the
-        // partials (maybe on another L2 slice) reads them without cache-wide flushes
-        __hip_atomic_store(&p.part_acc[slot * D + e], a_sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (e == 0) {
-            __hip_atomic_store(&p.part_m[slot], mall, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(&p.part_l[slot], lsum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int c = 0; c < GS / 4; ++c) {
+        if (c * 4 >= G) break;  // uniform
+        __syncthreads();        // the list (or the previous four heads) is not needed any more
+#pragma unroll
+        for (int gi = 0; gi < 4; ++gi)
+#pragma unroll
+            for (int e = 0; e < VPL; ++e) macc[(wave * 4 + gi) * D + (tid & 63) * VPL + e] = acc[c * 4 + gi][e];
+        __syncthreads();
+        if (c == 0) HIRA_TL(3);
+        for (int t = tid; t < 4 * D; t += blockDim.x) {
+            const int gi = t / D, e = t % D, g = c * 4 + gi;
+            if (g >= G) break;
+            float a_sum = 0.0f, lsum = 0.0f;
+            for (int w = 0; w < nw; ++w) {
+                a_sum += macc[(w * 4 + gi) * D + e];
+                lsum += s_lw[w * 16 + g];
+            }
+            const int head = p.group_size > 0 ? hoff + g : p.tree_q_heads[hoff + g];
+            const size_t slot = (size_t)head * P + blockIdx.y;
+            // device-scope stores: written through, so that the workgroup that folds the
+            // partials (maybe on another L2 slice) reads them without cache-wide flushes;
+            // a head without a selected key only says so (m = -inf)
+            if (lsum > 0.0f)
+                __hip_atomic_store(&p.part_acc[slot * D + e], a_sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (e == 0) {
+                __hip_atomic_store(&p.part_m[slot], lsum > 0.0f ? s_mh[g] : -INFINITY, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&p.part_l[slot], lsum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
         }
     }
     if (p.done == nullptr) return;  // the caller folds the partials in a second launch
 
     // ---- the last workgroup of this tree (and pass) to arrive folds the tree's partials ----
-    __shared__ int s_last;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // my stores have completed
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -486,87 +698,103 @@ __global__ __launch_bounds__(512, (KS <= 4 ? 4 : 2)) void search_mfma_kernel(con
         if (s_last) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
+    HIRA_TL(4);
     if (!s_last) return;
 
     auto ld = [](const float* q) {
         return __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     };
-    float* red = smem;                      // (16, 2): M and L of every head
-    float* wts = smem + 2 * kHeadsPerPass;  // (G, P) weights 2^(m_p - M), if they fit
-    const bool wts_fit = (size_t)G * P + 2 * kHeadsPerPass <= (size_t)nw * WAVE_FLOATS;
-    // phase 1: wave w handles heads w, w + nw, ...: M = max m_p, L = sum 2^(m_p - M) l_p
+    // phase 1: wave w handles heads w, w + nw, ...: M = max m_p, L = sum 2^(m_p - M) l_p, and
+    // the list of the partials that hold anything, with their weights 2^(m_p - M)
+    const bool listed = 2 * (size_t)G * P <= (size_t)S::WORDS;
+    int* clist = reinterpret_cast<int*>(s_words);                // (G, P)
+    float* cwt = reinterpret_cast<float*>(s_words) + (size_t)G * P;  // (G, P)
     for (int g = wave; g < G; g += nw) {
         const int head = p.group_size > 0 ? hoff + g : p.tree_q_heads[hoff + g];
         const float* pm = p.part_m + (size_t)head * P;
         const float* pl = p.part_l + (size_t)head * P;
-        float mx = -INFINITY;
-        for (int i = lane; i < P; i += 64) mx = fmaxf(mx, ld(pm + i));
+        const float mp0 = lane < P ? ld(pm + lane) : -INFINITY;
+        const float lp0 = lane < P ? ld(pl + lane) : 0.0f;
+        float mx = mp0;
+        for (int i = lane + 64; i < P; i += 64) mx = fmaxf(mx, ld(pm + i));
         mx = wave_max(mx);
         float ls = 0.0f;
-        for (int i = lane; i < P; i += 64) {
-            const float mp = ld(pm + i);
-            const float lp = ld(pl + i);
+        int nc = 0;
+        for (int i0 = 0; i0 < P; i0 += 64) {  // uniform
+            const int i = i0 + lane;
+            const float mp = i0 == 0 ? mp0 : (i < P ? ld(pm + i) : -INFINITY);
+            const float lp = i0 == 0 ? lp0 : (i < P ? ld(pl + i) : 0.0f);
             const float w = (mp > -INFINITY) ? exp2f(mp - mx) : 0.0f;
             ls += w * lp;
-            if (wts_fit) wts[g * P + i] = w;
+            const bool nz = w > 0.0f && lp > 0.0f;
+            const unsigned long long bal = __ballot(nz);
+            if (listed && nz) {
+                const int k = nc + __popcll(bal & ((1ull << lane) - 1ull));
+                clist[g * P + k] = i;
+                cwt[g * P + k] = w;
+            }
+            nc += __popcll(bal);
         }
 #pragma unroll
         for (int off = 1; off < 64; off <<= 1) ls += __shfl_xor(ls, off, 64);
         if (lane == 0) {
-            red[2 * g] = mx;
-            red[2 * g + 1] = ls;
+            s_red[2 * g] = mx;
+            s_red[2 * g + 1] = ls;
+            s_nc[g] = nc;
         }
     }
     __syncthreads();
-    // phase 2: thread t owns output column e of head g; empty partials are skipped
-    for (int t = threadIdx.x; t < G * D; t += blockDim.x) {
+    // phase 2: thread t owns output column e of head g; only partials that hold something
+    for (int t = tid; t < G * D; t += blockDim.x) {
         const int g = t / D, e = t % D;
         const int head = p.group_size > 0 ? hoff + g : p.tree_q_heads[hoff + g];
-        const float M = red[2 * g], Lg = red[2 * g + 1];
+        const float M = s_red[2 * g], Lg = s_red[2 * g + 1];
         const float* pm = p.part_m + (size_t)head * P;
         const float* pa = p.part_acc + (size_t)head * P * D + e;
-        float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+        float s0 = 0.0f, s1 = 0.0f;
         if (Lg > 0.0f) {
-            int i = 0;
-#pragma unroll 4
-            for (; i + 4 <= P; i += 4) {
-                float w0, w1, w2, w3;
-                if (wts_fit) {
-                    w0 = wts[g * P + i], w1 = wts[g * P + i + 1];
-                    w2 = wts[g * P + i + 2], w3 = wts[g * P + i + 3];
-                } else {
-                    const float m0 = ld(pm + i), m1 = ld(pm + i + 1), m2 = ld(pm + i + 2), m3 = ld(pm + i + 3);
-                    w0 = m0 > -INFINITY ? exp2f(m0 - M) : 0.0f;
-                    w1 = m1 > -INFINITY ? exp2f(m1 - M) : 0.0f;
-                    w2 = m2 > -INFINITY ? exp2f(m2 - M) : 0.0f;
-                    w3 = m3 > -INFINITY ? exp2f(m3 - M) : 0.0f;
+            if (listed) {
+                const int nc = s_nc[g];
+                const int* cl = clist + g * P;
+                const float* cw = cwt + g * P;
+                for (int k = 0; k < nc; k += 8) {  // uniform over the columns of a head
+                    float v[8];
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) v[u] = ld(pa + (size_t)cl[min(k + u, nc - 1)] * D);
+#pragma unroll
+                    for (int u = 0; u < 8; u += 2) {
+                        s0 += (k + u < nc ? cw[k + u] : 0.0f) * v[u];
+                        s1 += (k + u + 1 < nc ? cw[k + u + 1] : 0.0f) * v[u + 1];
+                    }
                 }
-                // weights are uniform over the columns of a head: the skips do not diverge
-                if (w0 > 0.0f) s0 += w0 * ld(pa + (size_t)i * D);
-                if (w1 > 0.0f) s1 += w1 * ld(pa + (size_t)(i + 1) * D);
-                if (w2 > 0.0f) s2 += w2 * ld(pa + (size_t)(i + 2) * D);
-                if (w3 > 0.0f) s3 += w3 * ld(pa + (size_t)(i + 3) * D);
-            }
-            for (; i < P; ++i) {
-                const float mi = ld(pm + i);
-                const float w = wts_fit ? wts[g * P + i] : (mi > -INFINITY ? exp2f(mi - M) : 0.0f);
-                if (w > 0.0f) s0 += w * ld(pa + (size_t)i * D);
+            } else {
+                for (int i = 0; i < P; ++i) {
+                    const float mi = ld(pm + i);
+                    const float w = mi > -INFINITY ? exp2f(mi - M) : 0.0f;
+                    if (w > 0.0f) s0 += w * ld(pa + (size_t)i * D);
+                }
             }
         }
         const float inv = Lg > 0.0f ? 1.0f / Lg : 0.0f;
-        p.attn_out[(size_t)head * D + e] = (s0 + s1 + s2 + s3) * inv;
+        p.attn_out[(size_t)head * D + e] = (s0 + s1) * inv;
     }
+    HIRA_TL(5);
 }
 
 template <int KS, int MT>
 void launch_mfma_gs(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s) {
     const dim3 block(plan.threads);
-    if (plan.gmax <= 4)
-        hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 4>), grid, block, plan.smem, s, p);
-    else if (plan.gmax <= 8)
-        hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 8>), grid, block, plan.smem, s, p);
-    else
-        hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 16>), grid, block, plan.smem, s, p);
+    const bool out = p.dense != nullptr || p.sel_count != nullptr;
+    if (plan.gmax <= 4) {
+        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 4, true>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 4, false>), grid, block, 0, s, p);
+    } else if (plan.gmax <= 8) {
+        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 8, true>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 8, false>), grid, block, 0, s, p);
+    } else {
+        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 16, true>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 16, false>), grid, block, 0, s, p);
+    }
 }
 
 template <int KS>
