@@ -458,7 +458,7 @@ static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* que
     const bool mfma_ok = mfma_search_supported(t, queue);
     HIRA_CHECK_ARG(want != 2 || mfma_ok,
                    "the MFMA kernel needs bf16, tiled layout, >= 2 levels, fan-out 16/32/48/64, "
-                   "dim = vdim in {64,128,256} and no queue");
+                   "dim = vdim in {64,128,256}");
     plan->kernel = (want == 2 || (want == 0 && mfma_ok)) ? 2 : 1;
     plan->lpr = lpr;
     if (plan->kernel == 2) {
@@ -486,7 +486,7 @@ static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* que
         plan->nodes_per_wave = tpw;
         plan->num_nodes = t->size[1];
         plan->tree_blocks = (tiles + tpw - 1) / tpw;
-        plan->queue_blocks = 0;
+        plan->queue_blocks = plan->num_queue_blocks > 0 ? 1 : 0;  // one workgroup takes the whole queue
         plan->smem = 0;
         return HIRA_OK;
     }

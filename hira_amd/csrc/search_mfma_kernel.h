@@ -1,11 +1,11 @@
 // MFMA search + sparse attention kernel: bf16 keys/centers in the tiled layout
 // (HIRA_TILE16), fan-out a multiple of 16, D = Dv in {64, 128, 256}, at least two levels.
 //
-// One workgroup (8 waves, the only one on its CU) owns a run of consecutive tiles of 16 level-1 nodes of one tree;
-// workgroup ids run fastest over the trees so that, with 8 L2 slices (XCDs) served
-// round-robin, the workgroups of one tree share a slice.  The work is split by phase, not by
-// node, so that neither the key scan nor the value gather depends on where in the tree the
-// selected keys sit:
+// One workgroup (8 waves; 256 registers a wave, so the only one on its CU) owns a run of
+// consecutive tiles of 16 level-1 nodes of one tree; workgroup ids run fastest over the trees
+// so that, with 8 L2 slices (XCDs) served round-robin, the workgroups of one tree share a
+// slice.  The work is split by phase, not by node, so that neither the key scan nor the
+// value gather depends on where in the tree the selected keys sit:
 //   gate   wave w gates tile w of the run: it issues, before it waits for anything, every
 //          load it needs (queries, the 16 x D tile of level-1 centres, the tiles holding the
 //          tile's ancestors, radii, child counts) and gates with v_mfma_f32_16x16x32_bf16:
@@ -15,17 +15,20 @@
 //          head = lane % 16 and row = 4*(lane/16) + j; a node survives for a head when
 //          score + ||q|| r >= tau.  Head masks and child counts of the nodes go to LDS.
 //   scan   the surviving nodes of the run are dealt round-robin to the waves; in each round
-//          a wave loads the key tiles of NB nodes at once, scores them the same way (leaf
-//          filter: q.k >= tau against the lane's own threshold) and the workgroup builds,
-//          in LDS, one list of the selected rows: slot and one softmax weight per head.  All
-//          waves share one running maximum per head, so their sums need no rescaling when
-//          they are added up.
-//   gather the rows of the list are dealt round-robin to the waves: up to kVBatch value rows
-//          in flight per wave, each row fetched once however many heads selected it,
+//          a wave loads the key tiles of NB nodes at once (the B operand now comes from
+//          LDS), scores them the same way (leaf filter: q.k >= tau against the lane's own
+//          threshold) and, for a tile with a selected row, writes the scaled scores of its
+//          rows to a table in LDS (-inf: not selected) and appends the selected rows to its
+//          stretch of the round's row list.  The waves agree on one running maximum per head,
+//          so their sums need no rescaling when they are added up.
+//   gather the rows of the list are dealt round-robin to the waves: kVBatch value rows in
+//          flight per wave, each row fetched once however many heads selected it; scores
+//          become weights 2^(z - m) with lane = (row, head), then
 //          acc[head][:] += weight(row, head) * v[:] with the accumulators in registers
 //          (lane owns Dv/64 columns of every head).
-// One partial (m, l, acc) per head and workgroup goes to global memory; the last workgroup
-// of a tree to arrive folds the tree's partials.
+// Keys queued since the tree was last updated (row-major, attended by every head) get one
+// more workgroup per tree.  One partial (m, l, acc) per head and workgroup goes to global
+// memory; the last workgroup of a tree to arrive folds the tree's partials.
 //
 // Register arrays are only ever indexed by compile-time constants: a run-time index would
 // push them to scratch memory.
@@ -195,6 +198,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     const bool want_attn = p.part_acc != nullptr;
     const int tile0 = (int)blockIdx.y * p.nodes_per_wave;  // first tile of my run
     const int ntile = min(p.nodes_per_wave, ((p.size[1] + 15) >> 4) - tile0);
+    const bool is_queue = (int)blockIdx.y >= p.tree_blocks;  // the workgroup after the tree's
 #ifdef HIRA_TIMELINE  // experiment builds only: p.stats receives 8 time stamps per workgroup
     unsigned long long* stats = nullptr;
     unsigned long long* tl =
@@ -215,138 +219,14 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         hoff = p.tree_q_off[tree] + blockIdx.z * kHeadsPerPass;
         G = min(kHeadsPerPass, p.tree_q_off[tree + 1] - hoff);
     }
-    if (G <= 0 || ntile <= 0) return;  // uniform
+    if (G <= 0 || (ntile <= 0 && !is_queue)) return;  // uniform
     G = min(G, GS);
     const bool head_ok = col < G;
     int qh = 0;
     if (head_ok) qh = p.group_size > 0 ? hoff + col : p.tree_q_heads[hoff + col];
 
-    // ---- queries and the first tile's gate operands, issued before the first wait --------
-    // (only the waves that gate need the queries in registers: the scan reads them from LDS)
-    int tl_mine = wave;  // tile of the run this wave gates next
-    uint4 qraw[KS];
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-        qraw[s] = make_uint4(0, 0, 0, 0);
-        if (head_ok && tl_mine < ntile)
-            qraw[s] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.q) +
-                                                      (size_t)qh * D + s * 32 + kb * 8);
-    }
-    const float tau = head_ok ? p.tau[qh] : INFINITY;
-    const float sc = head_ok ? p.scaling[qh] : 0.0f;
-    GateLoads<KS> gl;
-    if (tl_mine < ntile) gate_issue<KS>(p, tree, tile0 + tl_mine, lane, kb, gl);
-
-    // ---- B operand and ||q|| -----------------------------------------------------------
-    bf16x8_t bq[KS];
-    float ss = 0.0f;
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-        bq[s] = as_bf16x8(qraw[s]);
-        float f[8];
-        unpack<bf16_t>(qraw[s], f);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) ss += f[e] * f[e];
-    }
-    ss += __shfl_xor(ss, 16, 64);
-    ss += __shfl_xor(ss, 32, 64);
-    const float qn = sqrtf(ss);
-    if (wave == 0) {
-#pragma unroll
-        for (int s = 0; s < KS; ++s) s_bq[s * 64 + lane] = qraw[s];
-    }
-
-    // ---- gate: one tile per wave at a time ------------------------------------------------
-    while (tl_mine < ntile) {  // uniform in the wave
-        const int t1 = tile0 + tl_mine;
-        const bool count_nodes = stats != nullptr && lane == 0;
-        size_t span = 1;  // level-1 nodes under one node of the current level
-        for (int l = 2; l < L; ++l) span *= (size_t)bf;
-        int lcur = L - 1;
-        bool chain = head_ok;  // this head is still alive above the current level
-        for (; lcur > 3; --lcur) {  // trees deeper than four levels: one level at a time
-            const size_t a = ((size_t)t1 * 16) / span;
-            uint4 t[KS];
-            load_tile<KS>(tile_ptr<KS>(p.centers[lcur], (size_t)tree * p.cap[lcur], a / 16, lane), t);
-            const float rad = p.radii[lcur][(size_t)tree * p.cap[lcur] + a];
-            const bool any_alive = __ballot(chain) != 0ull;
-            if (count_nodes && ((size_t)t1 * 16) % span == 0 && any_alive && rad > -INFINITY)
-                stat_add(stats, lcur, 1u);
-            const float d = row_score(tile_scores<KS>(t, bq), (int)(a % 16), col);
-            chain = chain && (d + qn * rad >= tau);
-            span /= (size_t)bf;
-        }
-        const int n_par = min(max(L - 2, 0), 2);
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            if (i < n_par) {
-                const bool any_alive = __ballot(chain) != 0ull;
-                if (count_nodes && ((size_t)t1 * 16) % span == 0 && any_alive &&
-                    gl.arad[i] > -INFINITY)
-                    stat_add(stats, lcur, 1u);
-                const float d = row_score(tile_scores<KS>(gl.anc[i], bq), (int)(gl.aid[i] % 16), col);
-                chain = chain && (d + qn * gl.arad[i] >= tau);
-                span /= (size_t)bf;
-                --lcur;
-            }
-        }
-        const bool tile_live = __ballot(chain) != 0ull;  // uniform
-
-        // level-1 gates: 16 nodes at once
-        unsigned alive4 = 0u;
-        const int cc[4] = {gl.c4.x, gl.c4.y, gl.c4.z, gl.c4.w};
-        if (tile_live) {
-            const f32x4_t g1 = tile_scores<KS>(gl.a1, bq);
-            const float rr[4] = {gl.r4.x, gl.r4.y, gl.r4.z, gl.r4.w};
-            unsigned real = 0u;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                if (chain && (g1[j] + qn * rr[j] >= tau)) alive4 |= 1u << j;
-                if (stats) real += (unsigned)__popcll(__ballot(col == 0 && rr[j] > -INFINITY));
-            }
-            if (count_nodes) stat_add(stats, 1, real);
-        }
-        unsigned long long nb[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) nb[j] = __ballot((alive4 >> j) & 1u);
-        // node n = 4*kb' + j of the tile: its heads are field kb' of nb[j]
-        if (lane < 16) {
-            const int jn = lane & 3;
-            const unsigned long long bits = jn == 0 ? nb[0] : (jn == 1 ? nb[1] : (jn == 2 ? nb[2] : nb[3]));
-            s_nmask[tl_mine * 16 + lane] = (uint32_t)((bits >> (16 * (lane >> 2))) & 0xFFFFull);
-        }
-        if (col == 0) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) s_ncnt[tl_mine * 16 + 4 * kb + j] = cc[j];
-        }
-        tl_mine += nw;
-        if (tl_mine < ntile) gate_issue<KS>(p, tree, tile0 + tl_mine, lane, kb, gl);
-    }
-    HIRA_TL(7);
-    __syncthreads();
-    HIRA_TL(1);
-
-    // ---- the surviving nodes of the run, dealt round-robin to the waves ----------------------
-    unsigned long long my0, my1;  // bit n: node n (n + 64) of the run survives and is mine
-    int rounds;
-    {
-        const int NT = ntile * 16;
-        const bool a0 = lane < NT && s_nmask[lane] != 0u;
-        const bool a1 = lane + 64 < NT && s_nmask[lane + 64] != 0u;
-        const unsigned long long A0 = __ballot(a0), A1 = __ballot(a1);
-        const unsigned long long lt = (1ull << lane) - 1ull;
-        const int r0 = __popcll(A0 & lt), r1 = __popcll(A0) + __popcll(A1 & lt);
-        my0 = __ballot(a0 && (r0 % nw) == wave);
-        my1 = __ballot(a1 && (r1 % nw) == wave);
-        const int alive = __popcll(A0) + __popcll(A1);
-        rounds = ((alive + nw - 1) / nw + NB - 1) / NB;
-    }
-
     // ---- softmax state: running maximum m of the lane's head (the same in every wave);
     // per wave: l over the rows it gathered, acc[g][e] = column lane*VPL + e of head g -------
-    constexpr bool DB = S::LIST_WORDS == 2 * S::SCAN_WORDS;  // room for a second list: one barrier a round
-    const float sc2 = sc * kLog2e;
-    const size_t row0 = (size_t)tree * p.cap[0];
     float m_run = -INFINITY;
     float l_mine = 0.0f;  // this lane's share of l of head lane % GS, over the rows this wave gathered
     float acc[GS][VPL];
@@ -355,293 +235,491 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
 #pragma unroll
         for (int e = 0; e < VPL; ++e) acc[g][e] = 0.0f;
 
-    for (int r = 0; r < rounds; ++r) {  // uniform in the workgroup
-        const int par = r & 1;
-        // the round's list: row -> key slot and one scaled score per head (-inf: not selected);
-        // every wave fills its own stretch of ROWS * NB rows
-        uint32_t* lst_row = s_words + (DB ? par * S::SCAN_WORDS : 0);  // (LIST) listed row -> table row
-        uint32_t* lst_tslot = lst_row + S::LIST;                       // (LIST/16) table tile -> key slot
-        float* lst_z = reinterpret_cast<float*>(lst_tslot + S::LIST / 16);  // (LIST, GS) the table
-        if (!DB && want_attn && r > 0) __syncthreads();  // the previous list has been gathered
-
-        // ---- scan: key tiles of up to NB nodes in flight -----------------------------------
-        int node[NB], cnt[NB];
-        uint32_t nmask[NB];
-        uint4 a[NB][MT][KS];
+    if (is_queue) {
+        // ---- the queue of keys appended since the last update of the tree: row-major, every
+        // row counts for every head (no threshold).  Lane owns VPL columns; a wave takes rows
+        // wave, wave + nw, ..., eight at a time, and keeps its own (m, l, acc) per head. -------
+        float qf[GS][VPL], sc2g[GS], mq[GS], lq[GS];
 #pragma unroll
-        for (int u = 0; u < NB; ++u) {
-            int n = -1;
-            if (my0 != 0ull) {
-                n = __ffsll((long long)my0) - 1;
-                my0 &= my0 - 1ull;
-            } else if (my1 != 0ull) {
-                n = 64 + __ffsll((long long)my1) - 1;
-                my1 &= my1 - 1ull;
+        for (int g = 0; g < GS; ++g) {
+            mq[g] = -INFINITY;
+            lq[g] = 0.0f;
+            sc2g[g] = 0.0f;
+#pragma unroll
+            for (int e = 0; e < VPL; ++e) qf[g][e] = 0.0f;
+            if (g < G) {  // uniform
+                const int head = p.group_size > 0 ? hoff + g : p.tree_q_heads[hoff + g];
+                sc2g[g] = p.scaling[head] * kLog2e;
+                const uint16_t* qp = reinterpret_cast<const uint16_t*>(p.q) + (size_t)head * D + lane * VPL;
+#pragma unroll
+                for (int e = 0; e < VPL; ++e) qf[g][e] = bf16_lo((uint32_t)qp[e]);
             }
-            node[u] = n;
-            cnt[u] = __builtin_amdgcn_readfirstlane(n >= 0 ? s_ncnt[n] : 0);
-            nmask[u] = (uint32_t)__builtin_amdgcn_readfirstlane((int)(n >= 0 ? s_nmask[n] : 0u));
-            const size_t tile_first = ((size_t)(tile0 * 16 + max(n, 0)) * bf) / 16;
+        }
+        const uint16_t* qk = reinterpret_cast<const uint16_t*>(p.queue_keys) + (size_t)tree * p.queue_cap * D + lane * VPL;
+        const uint16_t* qv = reinterpret_cast<const uint16_t*>(p.queue_values) + (size_t)tree * p.queue_cap * D + lane * VPL;
+        for (int r0 = wave; r0 < p.queue_len; r0 += 8 * nw) {  // uniform in the wave
+            uint16_t kraw[8][VPL], vraw[8][VPL];
 #pragma unroll
-            for (int tt = 0; tt < MT; ++tt)
-                if (tt * 16 < cnt[u])
-                    load_tile<KS>(tile_ptr<KS>(p.keys, row0, tile_first + tt, lane), a[u][tt]);
+            for (int i = 0; i < 8; ++i) {
+                const int row = min(r0 + i * nw, p.queue_len - 1);
+#pragma unroll
+                for (int e = 0; e < VPL; ++e) {
+                    kraw[i][e] = qk[(size_t)row * D + e];
+                    vraw[i][e] = qv[(size_t)row * D + e];
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                if (r0 + i * nw >= p.queue_len) break;  // uniform
+#pragma unroll
+                for (int g = 0; g < GS; ++g) {
+                    if (g >= G) break;  // uniform
+                    float sdot = 0.0f;
+#pragma unroll
+                    for (int e = 0; e < VPL; ++e) sdot += bf16_lo((uint32_t)kraw[i][e]) * qf[g][e];
+#pragma unroll
+                    for (int off = 1; off < 64; off <<= 1) sdot += __shfl_xor(sdot, off, 64);
+                    const float z = sdot * sc2g[g];
+                    const float mnew = fmaxf(mq[g], z);
+                    const float f = exp2f(mq[g] - mnew);  // 0 the first time
+                    const float w = exp2f(z - mnew);
+                    lq[g] = lq[g] * f + w;
+#pragma unroll
+                    for (int e = 0; e < VPL; ++e)
+                        acc[g][e] = acc[g][e] * f + w * bf16_lo((uint32_t)vraw[i][e]);
+                    mq[g] = mnew;
+                }
+            }
+        }
+        // one maximum per head for the whole workgroup, as the merge below expects
+#pragma unroll
+        for (int g = 0; g < GS; ++g)
+            if (lane == g) s_mxw[0][wave * 16 + g] = mq[g];
+        __syncthreads();
+#pragma unroll
+        for (int g = 0; g < GS; ++g) {
+            float mall = -INFINITY;
+            for (int w = 0; w < nw; ++w) mall = fmaxf(mall, s_mxw[0][w * 16 + g]);
+            const float f = mq[g] == -INFINITY ? 0.0f : exp2f(mq[g] - mall);
+#pragma unroll
+            for (int e = 0; e < VPL; ++e) acc[g][e] *= f;
+            if (lane == g) l_mine = lq[g] * f;
+            if (col == g) m_run = mall;
+        }
+    } else {
+        // ---- queries and the first tile's gate operands, issued before the first wait --------
+        // (only the waves that gate need the queries in registers: the scan reads them from LDS)
+        int tl_mine = wave;  // tile of the run this wave gates next
+        uint4 qraw[KS];
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            qraw[s] = make_uint4(0, 0, 0, 0);
+            if (head_ok && tl_mine < ntile)
+                qraw[s] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.q) +
+                                                          (size_t)qh * D + s * 32 + kb * 8);
+        }
+        const float tau = head_ok ? p.tau[qh] : INFINITY;
+        const float sc = head_ok ? p.scaling[qh] : 0.0f;
+        GateLoads<KS> gl;
+        if (tl_mine < ntile) gate_issue<KS>(p, tree, tile0 + tl_mine, lane, kb, gl);
+
+        // ---- B operand and ||q|| -----------------------------------------------------------
+        bf16x8_t bq[KS];
+        float ss = 0.0f;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            bq[s] = as_bf16x8(qraw[s]);
+            float f[8];
+            unpack<bf16_t>(qraw[s], f);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ss += f[e] * f[e];
+        }
+        ss += __shfl_xor(ss, 16, 64);
+        ss += __shfl_xor(ss, 32, 64);
+        const float qn = sqrtf(ss);
+        if (wave == 0) {
+#pragma unroll
+            for (int s = 0; s < KS; ++s) s_bq[s * 64 + lane] = qraw[s];
         }
 
-        // all the products first: the operand registers are free before the bookkeeping starts
-        f32x4_t sco_all[NB][MT];
+        // ---- gate: one tile per wave at a time ------------------------------------------------
+        while (tl_mine < ntile) {  // uniform in the wave
+            const int t1 = tile0 + tl_mine;
+            const bool count_nodes = stats != nullptr && lane == 0;
+            size_t span = 1;  // level-1 nodes under one node of the current level
+            for (int l = 2; l < L; ++l) span *= (size_t)bf;
+            int lcur = L - 1;
+            bool chain = head_ok;  // this head is still alive above the current level
+            for (; lcur > 3; --lcur) {  // trees deeper than four levels: one level at a time
+                const size_t a = ((size_t)t1 * 16) / span;
+                uint4 t[KS];
+                load_tile<KS>(tile_ptr<KS>(p.centers[lcur], (size_t)tree * p.cap[lcur], a / 16, lane), t);
+                const float rad = p.radii[lcur][(size_t)tree * p.cap[lcur] + a];
+                const bool any_alive = __ballot(chain) != 0ull;
+                if (count_nodes && ((size_t)t1 * 16) % span == 0 && any_alive && rad > -INFINITY)
+                    stat_add(stats, lcur, 1u);
+                const float d = row_score(tile_scores<KS>(t, bq), (int)(a % 16), col);
+                chain = chain && (d + qn * rad >= tau);
+                span /= (size_t)bf;
+            }
+            const int n_par = min(max(L - 2, 0), 2);
 #pragma unroll
-        for (int u = 0; u < NB; ++u)
-#pragma unroll
-            for (int tt = 0; tt < MT; ++tt)  // (only read where it is written: under this condition)
-                if (tt * 16 < cnt[u]) sco_all[u][tt] = tile_scores_lds<KS>(a[u][tt], s_bq, lane);
-
-        if (r == 0) HIRA_TL(8);
-        // The bookkeeping below derives everything per-lane from this copy, which the compiler
-        // cannot see through: otherwise it computes those values once, ahead of the loop, and
-        // they crowd out the registers that the loads above need.
-        int lane_o = lane;
-        asm volatile("" : "+v"(lane_o));
-        const int col = lane_o & 15, kb = lane_o >> 4;
-
-        int nsel = 0;  // rows of my stretch of the list
-        float zmax = -INFINITY;
-        const int zrow0 = wave * (NB * S::ROWS);  // my stretch of the round's rows
-#pragma unroll
-        for (int u = 0; u < NB; ++u) {
-            // a head for which the node did not survive selects nothing
-            const float tau_u = ((nmask[u] >> col) & 1u) ? tau : INFINITY;
-            const unsigned slot0 = (unsigned)((tile0 * 16 + max(node[u], 0)) * bf);
-            if (stats && lane == 0) stat_add(stats, 0, (unsigned)cnt[u]);
-#pragma unroll
-            for (int tt = 0; tt < MT; ++tt) {
-                if (tt * 16 >= cnt[u]) continue;  // uniform
-                const f32x4_t sco = sco_all[u][tt];
-                const int lim = cnt[u] - tt * 16 - 4 * kb;  // my rows j < lim hold keys
-                unsigned sel4 = 0u;
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    if (sco[j] >= tau_u && j < lim) sel4 |= 1u << j;
-                if (__ballot(sel4 != 0u) == 0ull) continue;  // uniform
-                // rows selected by some head: OR over the 16 lanes (heads) of my row group by
-                // rotating inside the group, then the four groups side by side
-                unsigned any4 = sel4;
-                any4 |= (unsigned)__builtin_amdgcn_update_dpp(0, (int)any4, 0x121, 0xF, 0xF, false);
-                any4 |= (unsigned)__builtin_amdgcn_update_dpp(0, (int)any4, 0x122, 0xF, 0xF, false);
-                any4 |= (unsigned)__builtin_amdgcn_update_dpp(0, (int)any4, 0x124, 0xF, 0xF, false);
-                any4 |= (unsigned)__builtin_amdgcn_update_dpp(0, (int)any4, 0x128, 0xF, 0xF, false);
-                const unsigned rowmask = (unsigned)__builtin_amdgcn_readlane((int)any4, 0) |
-                                         ((unsigned)__builtin_amdgcn_readlane((int)any4, 16) << 4) |
-                                         ((unsigned)__builtin_amdgcn_readlane((int)any4, 32) << 8) |
-                                         ((unsigned)__builtin_amdgcn_readlane((int)any4, 48) << 12);
-                if (stats) {
-                    const unsigned pairs = (unsigned)__popcll(__ballot(sel4 & 1u)) +
-                                           (unsigned)__popcll(__ballot(sel4 & 2u)) +
-                                           (unsigned)__popcll(__ballot(sel4 & 4u)) +
-                                           (unsigned)__popcll(__ballot(sel4 & 8u));
-                    if (lane == 0) {
-                        stat_add(stats, HIRA_MAX_LEVELS, (unsigned)__popc(rowmask));
-                        stat_add(stats, HIRA_MAX_LEVELS + 1, pairs);
-                    }
+            for (int i = 0; i < 2; ++i) {
+                if (i < n_par) {
+                    const bool any_alive = __ballot(chain) != 0ull;
+                    if (count_nodes && ((size_t)t1 * 16) % span == 0 && any_alive &&
+                        gl.arad[i] > -INFINITY)
+                        stat_add(stats, lcur, 1u);
+                    const float d = row_score(tile_scores<KS>(gl.anc[i], bq), (int)(gl.aid[i] % 16), col);
+                    chain = chain && (d + qn * gl.arad[i] >= tau);
+                    span /= (size_t)bf;
+                    --lcur;
                 }
-                const unsigned tslot = slot0 + tt * 16;
+            }
+            const bool tile_live = __ballot(chain) != 0ull;  // uniform
 
-                // ---- dense scores / compact lists ------------------------------------------
-                if (OUT && (p.dense != nullptr || p.sel_count != nullptr)) {
-                    unsigned long long sb[4];
+            // level-1 gates: 16 nodes at once
+            unsigned alive4 = 0u;
+            const int cc[4] = {gl.c4.x, gl.c4.y, gl.c4.z, gl.c4.w};
+            if (tile_live) {
+                const f32x4_t g1 = tile_scores<KS>(gl.a1, bq);
+                const float rr[4] = {gl.r4.x, gl.r4.y, gl.r4.z, gl.r4.w};
+                unsigned real = 0u;
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) sb[j] = __ballot((sel4 >> j) & 1u);
-                    int base = 0;
-                    if (p.sel_count != nullptr) {  // one atomic per head of the tile (kb = 0)
-                        int mine = 0;
+                for (int j = 0; j < 4; ++j) {
+                    if (chain && (g1[j] + qn * rr[j] >= tau)) alive4 |= 1u << j;
+                    if (stats) real += (unsigned)__popcll(__ballot(col == 0 && rr[j] > -INFINITY));
+                }
+                if (count_nodes) stat_add(stats, 1, real);
+            }
+            unsigned long long nb[4];
 #pragma unroll
-                        for (int j = 0; j < 4; ++j)
-                            mine += __popcll(sb[j] & (0x0001000100010001ull << col));
-                        int b0 = 0;
-                        if (kb == 0 && mine > 0) b0 = atomicAdd(&p.sel_count[qh], mine);
-                        base = __shfl(b0, col, 64);
+            for (int j = 0; j < 4; ++j) nb[j] = __ballot((alive4 >> j) & 1u);
+            // node n = 4*kb' + j of the tile: its heads are field kb' of nb[j]
+            if (lane < 16) {
+                const int jn = lane & 3;
+                const unsigned long long bits = jn == 0 ? nb[0] : (jn == 1 ? nb[1] : (jn == 2 ? nb[2] : nb[3]));
+                s_nmask[tl_mine * 16 + lane] = (uint32_t)((bits >> (16 * (lane >> 2))) & 0xFFFFull);
+            }
+            if (col == 0) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) s_ncnt[tl_mine * 16 + 4 * kb + j] = cc[j];
+            }
+            tl_mine += nw;
+            if (tl_mine < ntile) gate_issue<KS>(p, tree, tile0 + tl_mine, lane, kb, gl);
+        }
+        HIRA_TL(7);
+        __syncthreads();
+        HIRA_TL(1);
+
+        // ---- the surviving nodes of the run, dealt round-robin to the waves ----------------------
+        unsigned long long my0, my1;  // bit n: node n (n + 64) of the run survives and is mine
+        int rounds;
+        {
+            const int NT = ntile * 16;
+            const bool a0 = lane < NT && s_nmask[lane] != 0u;
+            const bool a1 = lane + 64 < NT && s_nmask[lane + 64] != 0u;
+            const unsigned long long A0 = __ballot(a0), A1 = __ballot(a1);
+            const unsigned long long lt = (1ull << lane) - 1ull;
+            const int r0 = __popcll(A0 & lt), r1 = __popcll(A0) + __popcll(A1 & lt);
+            my0 = __ballot(a0 && (r0 % nw) == wave);
+            my1 = __ballot(a1 && (r1 % nw) == wave);
+            const int alive = __popcll(A0) + __popcll(A1);
+            rounds = ((alive + nw - 1) / nw + NB - 1) / NB;
+        }
+
+        constexpr bool DB = S::LIST_WORDS == 2 * S::SCAN_WORDS;  // room for a second list: one barrier a round
+        const float sc2 = sc * kLog2e;
+        const size_t row0 = (size_t)tree * p.cap[0];
+
+        for (int r = 0; r < rounds; ++r) {  // uniform in the workgroup
+            const int par = r & 1;
+            // the round's list: row -> key slot and one scaled score per head (-inf: not selected);
+            // every wave fills its own stretch of ROWS * NB rows
+            uint32_t* lst_row = s_words + (DB ? par * S::SCAN_WORDS : 0);  // (LIST) listed row -> table row
+            uint32_t* lst_tslot = lst_row + S::LIST;                       // (LIST/16) table tile -> key slot
+            float* lst_z = reinterpret_cast<float*>(lst_tslot + S::LIST / 16);  // (LIST, GS) the table
+            if (!DB && want_attn && r > 0) __syncthreads();  // the previous list has been gathered
+
+            // ---- scan: key tiles of up to NB nodes in flight -----------------------------------
+            int node[NB], cnt[NB];
+            uint32_t nmask[NB];
+            uint4 a[NB][MT][KS];
+#pragma unroll
+            for (int u = 0; u < NB; ++u) {
+                int n = -1;
+                if (my0 != 0ull) {
+                    n = __ffsll((long long)my0) - 1;
+                    my0 &= my0 - 1ull;
+                } else if (my1 != 0ull) {
+                    n = 64 + __ffsll((long long)my1) - 1;
+                    my1 &= my1 - 1ull;
+                }
+                node[u] = n;
+                cnt[u] = __builtin_amdgcn_readfirstlane(n >= 0 ? s_ncnt[n] : 0);
+                nmask[u] = (uint32_t)__builtin_amdgcn_readfirstlane((int)(n >= 0 ? s_nmask[n] : 0u));
+                const size_t tile_first = ((size_t)(tile0 * 16 + max(n, 0)) * bf) / 16;
+#pragma unroll
+                for (int tt = 0; tt < MT; ++tt)
+                    if (tt * 16 < cnt[u])
+                        load_tile<KS>(tile_ptr<KS>(p.keys, row0, tile_first + tt, lane), a[u][tt]);
+            }
+
+            // all the products first: the operand registers are free before the bookkeeping starts
+            f32x4_t sco_all[NB][MT];
+#pragma unroll
+            for (int u = 0; u < NB; ++u)
+#pragma unroll
+                for (int tt = 0; tt < MT; ++tt)  // (only read where it is written: under this condition)
+                    if (tt * 16 < cnt[u]) sco_all[u][tt] = tile_scores_lds<KS>(a[u][tt], s_bq, lane);
+
+            if (r == 0) HIRA_TL(8);
+            // The bookkeeping below derives everything per-lane from this copy, which the compiler
+            // cannot see through: otherwise it computes those values once, ahead of the loop, and
+            // they crowd out the registers that the loads above need.
+            int lane_o = lane;
+            asm volatile("" : "+v"(lane_o));
+            const int col = lane_o & 15, kb = lane_o >> 4;
+
+            int nsel = 0;  // rows of my stretch of the list
+            float zmax = -INFINITY;
+            const int zrow0 = wave * (NB * S::ROWS);  // my stretch of the round's rows
+#pragma unroll
+            for (int u = 0; u < NB; ++u) {
+                // a head for which the node did not survive selects nothing
+                const float tau_u = ((nmask[u] >> col) & 1u) ? tau : INFINITY;
+                const unsigned slot0 = (unsigned)((tile0 * 16 + max(node[u], 0)) * bf);
+                if (stats && lane == 0) stat_add(stats, 0, (unsigned)cnt[u]);
+#pragma unroll
+                for (int tt = 0; tt < MT; ++tt) {
+                    if (tt * 16 >= cnt[u]) continue;  // uniform
+                    const f32x4_t sco = sco_all[u][tt];
+                    const int lim = cnt[u] - tt * 16 - 4 * kb;  // my rows j < lim hold keys
+                    unsigned sel4 = 0u;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (sco[j] >= tau_u && j < lim) sel4 |= 1u << j;
+                    if (__ballot(sel4 != 0u) == 0ull) continue;  // uniform
+                    // rows selected by some head: OR over the 16 lanes (heads) of my row group by
+                    // rotating inside the group, then the four groups side by side
+                    unsigned any4 = sel4;
+                    any4 |= (unsigned)__builtin_amdgcn_update_dpp(0, (int)any4, 0x121, 0xF, 0xF, false);
+                    any4 |= (unsigned)__builtin_amdgcn_update_dpp(0, (int)any4, 0x122, 0xF, 0xF, false);
+                    any4 |= (unsigned)__builtin_amdgcn_update_dpp(0, (int)any4, 0x124, 0xF, 0xF, false);
+                    any4 |= (unsigned)__builtin_amdgcn_update_dpp(0, (int)any4, 0x128, 0xF, 0xF, false);
+                    const unsigned rowmask = (unsigned)__builtin_amdgcn_readlane((int)any4, 0) |
+                                             ((unsigned)__builtin_amdgcn_readlane((int)any4, 16) << 4) |
+                                             ((unsigned)__builtin_amdgcn_readlane((int)any4, 32) << 8) |
+                                             ((unsigned)__builtin_amdgcn_readlane((int)any4, 48) << 12);
+                    if (stats) {
+                        const unsigned pairs = (unsigned)__popcll(__ballot(sel4 & 1u)) +
+                                               (unsigned)__popcll(__ballot(sel4 & 2u)) +
+                                               (unsigned)__popcll(__ballot(sel4 & 4u)) +
+                                               (unsigned)__popcll(__ballot(sel4 & 8u));
+                        if (lane == 0) {
+                            stat_add(stats, HIRA_MAX_LEVELS, (unsigned)__popc(rowmask));
+                            stat_add(stats, HIRA_MAX_LEVELS + 1, pairs);
+                        }
                     }
+                    const unsigned tslot = slot0 + tt * 16;
+
+                    // ---- dense scores / compact lists ------------------------------------------
+                    if (OUT && (p.dense != nullptr || p.sel_count != nullptr)) {
+                        unsigned long long sb[4];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        if ((sel4 >> j) & 1u) {
-                            const unsigned slot = tslot + 4 * kb + j;
-                            int idx = (int)slot;
-                            if (p.dense_by_position) idx = p.perm[row0 + slot];
-                            if (p.dense != nullptr)
-                                p.dense[(int64_t)qh * p.dense_stride + idx] = sco[j] * sc;
-                            if (p.sel_count != nullptr) {
-                                // hits of my head ordered before (kb, j): rows j' < j of any
-                                // kb, then row j of lower kb
-                                int before = 0;
+                        for (int j = 0; j < 4; ++j) sb[j] = __ballot((sel4 >> j) & 1u);
+                        int base = 0;
+                        if (p.sel_count != nullptr) {  // one atomic per head of the tile (kb = 0)
+                            int mine = 0;
 #pragma unroll
-                                for (int j2 = 0; j2 < 4; ++j2) {
-                                    unsigned long long bits = sb[j2] & (0x0001000100010001ull << col);
-                                    if (j2 == j) bits &= (1ull << (16 * kb)) - 1ull;
-                                    if (j2 <= j) before += __popcll(bits);
-                                }
-                                const int pos = base + before;
-                                if (pos < p.sel_cap) {
-                                    p.sel_index[(int64_t)qh * p.sel_cap + pos] = idx;
-                                    p.sel_score[(int64_t)qh * p.sel_cap + pos] = sco[j];
+                            for (int j = 0; j < 4; ++j)
+                                mine += __popcll(sb[j] & (0x0001000100010001ull << col));
+                            int b0 = 0;
+                            if (kb == 0 && mine > 0) b0 = atomicAdd(&p.sel_count[qh], mine);
+                            base = __shfl(b0, col, 64);
+                        }
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            if ((sel4 >> j) & 1u) {
+                                const unsigned slot = tslot + 4 * kb + j;
+                                int idx = (int)slot;
+                                if (p.dense_by_position) idx = p.perm[row0 + slot];
+                                if (p.dense != nullptr)
+                                    p.dense[(int64_t)qh * p.dense_stride + idx] = sco[j] * sc;
+                                if (p.sel_count != nullptr) {
+                                    // hits of my head ordered before (kb, j): rows j' < j of any
+                                    // kb, then row j of lower kb
+                                    int before = 0;
+#pragma unroll
+                                    for (int j2 = 0; j2 < 4; ++j2) {
+                                        unsigned long long bits = sb[j2] & (0x0001000100010001ull << col);
+                                        if (j2 == j) bits &= (1ull << (16 * kb)) - 1ull;
+                                        if (j2 <= j) before += __popcll(bits);
+                                    }
+                                    const int pos = base + before;
+                                    if (pos < p.sel_cap) {
+                                        p.sel_index[(int64_t)qh * p.sel_cap + pos] = idx;
+                                        p.sel_score[(int64_t)qh * p.sel_cap + pos] = sco[j];
+                                    }
                                 }
                             }
                         }
                     }
-                }
 
-                // ---- the tile's scores go to the table, its selected rows join my list -----------
-                if (want_attn) {
-                    const int trow = zrow0 + (u * MT + tt) * 16;  // the tile's rows in the table
-                    float zs[4];
+                    // ---- the tile's scores go to the table, its selected rows join my list -----------
+                    if (want_attn) {
+                        const int trow = zrow0 + (u * MT + tt) * 16;  // the tile's rows in the table
+                        float zs[4];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        zs[j] = ((sel4 >> j) & 1u) ? sco[j] * sc2 : -INFINITY;
-                        zmax = fmaxf(zmax, zs[j]);
+                        for (int j = 0; j < 4; ++j) {
+                            zs[j] = ((sel4 >> j) & 1u) ? sco[j] * sc2 : -INFINITY;
+                            zmax = fmaxf(zmax, zs[j]);
+                        }
+                        if (col < GS) {
+                            float* zp = lst_z + (trow + 4 * kb) * GS + col;
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) zp[j * GS] = zs[j];
+                        }
+                        if (lane_o < 16 && ((rowmask >> lane_o) & 1u))
+                            lst_row[zrow0 + nsel + __popc(rowmask & ((1u << lane_o) - 1u))] = (uint32_t)(trow + lane_o);
+                        if (lane_o == 0) lst_tslot[trow >> 4] = tslot;
                     }
-                    if (col < GS) {
-                        float* zp = lst_z + (trow + 4 * kb) * GS + col;
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) zp[j * GS] = zs[j];
-                    }
-                    if (lane_o < 16 && ((rowmask >> lane_o) & 1u))
-                        lst_row[zrow0 + nsel + __popc(rowmask & ((1u << lane_o) - 1u))] = (uint32_t)(trow + lane_o);
-                    if (lane_o == 0) lst_tslot[trow >> 4] = tslot;
+                    nsel += __popc(rowmask);
                 }
-                nsel += __popc(rowmask);
             }
-        }
-        if (!want_attn) continue;  // uniform in the launch
+            if (!want_attn) continue;  // uniform in the launch
 
-        // ---- every wave learns all counts and the best scores of the round ---------------------
-        zmax = fmaxf(zmax, __shfl_xor(zmax, 16, 64));
-        zmax = fmaxf(zmax, __shfl_xor(zmax, 32, 64));
-        if (r == 0) HIRA_TL(9);
-        if (lane == 0) s_cntw[par][wave] = nsel;
-        if (kb == 0) s_mxw[par][wave * 16 + col] = zmax;
-        __syncthreads();
-        int cw[kMfmaWaves];
-        int tot = 0;
-        float rmax = -INFINITY;
-        {
-            // one read each, then lane by lane: no wait between the waves' entries
-            const int cv = s_cntw[par][lane_o & (kMfmaWaves - 1)];
-            float mv[kMfmaWaves];
+            // ---- every wave learns all counts and the best scores of the round ---------------------
+            zmax = fmaxf(zmax, __shfl_xor(zmax, 16, 64));
+            zmax = fmaxf(zmax, __shfl_xor(zmax, 32, 64));
+            if (r == 0) HIRA_TL(9);
+            if (lane == 0) s_cntw[par][wave] = nsel;
+            if (kb == 0) s_mxw[par][wave * 16 + col] = zmax;
+            __syncthreads();
+            int cw[kMfmaWaves];
+            int tot = 0;
+            float rmax = -INFINITY;
+            {
+                // one read each, then lane by lane: no wait between the waves' entries
+                const int cv = s_cntw[par][lane_o & (kMfmaWaves - 1)];
+                float mv[kMfmaWaves];
 #pragma unroll
-            for (int w = 0; w < kMfmaWaves; ++w) mv[w] = s_mxw[par][w * 16 + col];
-#pragma unroll
-            for (int w = 0; w < kMfmaWaves; ++w) {
-                cw[w] = w < nw ? __builtin_amdgcn_readlane(cv, w) : 0;
-                tot += cw[w];
-                if (w < nw) rmax = fmaxf(rmax, mv[w]);
-            }
-        }
-#ifdef HIRA_TIMELINE
-        if (r == 0) HIRA_TL(10);
-        if (threadIdx.x == 0 && r == 0) { tl[6] = (unsigned long long)tot; tl[12] = (unsigned long long)rounds; }
-#endif
-        if (tot == 0) continue;  // uniform in the workgroup: nothing selected in this round
-
-        // the new maximum of every head, and what it does to the sums so far; head g lives in
-        // lane g; the weights below are computed with lane = (row, head), head = lane % GS
-        const float mnew = fmaxf(m_run, rmax);
-        const float f = (m_run == mnew) ? 1.0f : exp2f(m_run - mnew);
-        m_run = mnew;
-        // a head without a selected key has m = -inf and only z = -inf: any finite stand-in
-        const float m_lane = __shfl(mnew == -INFINITY ? 0.0f : mnew, lane_o & (GS - 1), 64);
-        if (__ballot(f != 1.0f) != 0ull) {  // uniform
-            l_mine *= __shfl(f, lane_o & (GS - 1), 64);
-#pragma unroll
-            for (int g = 0; g < GS; ++g) {
-                const float fg = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), g));
-#pragma unroll
-                for (int e = 0; e < VPL; ++e) acc[g][e] *= fg;
-            }
-        }
-
-        // ---- gather: list rows wave, wave + nw, ...; kVBatch value rows in flight --------------
-        constexpr int RP = 64 / GS;          // rows whose weights one pass over the lanes computes
-        constexpr int NPASS = kVBatch / RP;  // GS = 4: 1, GS = 8: 2, GS = 16: 4
-        const char* vtree = reinterpret_cast<const char*>(p.values) + row0 * (size_t)(D * 2);
-        // where the rows of a batch sit (row `le` of the round is row `rem` of the stretch of the
-        // wave it falls in; lane = (row of the pass, head)), and their value rows
-        auto issue = [&](int e0, int (&at_v)[NPASS], uint32_t (&vraw)[kVBatch][VW]) {
-#pragma unroll
-            for (int ps = 0; ps < NPASS; ++ps) {
-                const int le = e0 + (ps * RP + lane_o / GS) * nw;
-                int rem = le, at = -1;
+                for (int w = 0; w < kMfmaWaves; ++w) mv[w] = s_mxw[par][w * 16 + col];
 #pragma unroll
                 for (int w = 0; w < kMfmaWaves; ++w) {
-                    if (at < 0 && rem < cw[w]) at = w * (NB * S::ROWS) + rem;
-                    rem -= cw[w];
-                }
-                // -> its row in the score table (-1: past the end)
-                at_v[ps] = (le < tot && at >= 0) ? (int)lst_row[at] : -1;
-            }
-            int slot_v[NPASS];  // the key slots of all the rows of a pass
-#pragma unroll
-            for (int ps = 0; ps < NPASS; ++ps)
-                slot_v[ps] = at_v[ps] >= 0 ? (int)(lst_tslot[at_v[ps] >> 4] + (unsigned)(at_v[ps] & 15)) : 0;
-            // (a batch is always loaded whole, rows past the end as slot 0: straight-line code)
-#pragma unroll
-            for (int i = 0; i < kVBatch; ++i) {
-                {
-                    const unsigned slot = (unsigned)__builtin_amdgcn_readlane(slot_v[i / RP], (i % RP) * GS);
-                    const uint16_t* vp =
-                        reinterpret_cast<const uint16_t*>(vtree + (size_t)slot * (D * 2)) + lane_o * VPL;
-                    if (VPL == 1) {
-                        vraw[i][0] = *vp;
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < VPL / 2; ++e)
-                            vraw[i][e] = reinterpret_cast<const uint32_t*>(vp)[e];
-                    }
+                    cw[w] = w < nw ? __builtin_amdgcn_readlane(cv, w) : 0;
+                    tot += cw[w];
+                    if (w < nw) rmax = fmaxf(rmax, mv[w]);
                 }
             }
-        };
-        auto consume = [&](int e0, const int (&at_v)[NPASS], const uint32_t (&vraw)[kVBatch][VW]) {
-            // (nothing of what follows may be scheduled ahead of loads issued before this point)
-            __builtin_amdgcn_sched_barrier(0);
-            // scores -> weights, in place, 64 (row, head) pairs at a time
-#pragma unroll
-            for (int ps = 0; ps < NPASS; ++ps) {
-                if (at_v[ps] >= 0) {
-                    float* zp = lst_z + at_v[ps] * GS + (lane_o & (GS - 1));
-                    const float w = __builtin_amdgcn_exp2f(*zp - m_lane);
-                    l_mine += w;
-                    *zp = w;
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < kVBatch; ++i) {
-                if (e0 + i * nw >= tot) break;  // uniform
-                const int at = __builtin_amdgcn_readlane(at_v[i / RP], (i % RP) * GS);
-                float vf[VPL];
-                if (VPL == 1) {
-                    vf[0] = bf16_lo(vraw[i][0]);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < VPL / 2; ++e) {
-                        vf[2 * e] = bf16_lo(vraw[i][e]);
-                        vf[2 * e + 1] = bf16_hi(vraw[i][e]);
-                    }
-                }
-                const float* wr = lst_z + at * GS;  // weights of this row, one per head
+#ifdef HIRA_TIMELINE
+            if (r == 0) HIRA_TL(10);
+            if (threadIdx.x == 0 && r == 0) { tl[6] = (unsigned long long)tot; tl[12] = (unsigned long long)rounds; }
+#endif
+            if (tot == 0) continue;  // uniform in the workgroup: nothing selected in this round
+
+            // the new maximum of every head, and what it does to the sums so far; head g lives in
+            // lane g; the weights below are computed with lane = (row, head), head = lane % GS
+            const float mnew = fmaxf(m_run, rmax);
+            const float f = (m_run == mnew) ? 1.0f : exp2f(m_run - mnew);
+            m_run = mnew;
+            // a head without a selected key has m = -inf and only z = -inf: any finite stand-in
+            const float m_lane = __shfl(mnew == -INFINITY ? 0.0f : mnew, lane_o & (GS - 1), 64);
+            if (__ballot(f != 1.0f) != 0ull) {  // uniform
+                l_mine *= __shfl(f, lane_o & (GS - 1), 64);
 #pragma unroll
                 for (int g = 0; g < GS; ++g) {
-                    const float w = wr[g];  // same address in every lane: a broadcast read
+                    const float fg = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), g));
 #pragma unroll
-                    for (int e = 0; e < VPL; ++e) acc[g][e] += w * vf[e];
+                    for (int e = 0; e < VPL; ++e) acc[g][e] *= fg;
                 }
             }
-        };
-        for (int e0 = wave; e0 < tot; e0 += nw * kVBatch) {  // uniform in the wave
-            int at_v[NPASS];
-            uint32_t vraw[kVBatch][VW];
-            issue(e0, at_v, vraw);
-            consume(e0, at_v, vraw);
+
+            // ---- gather: list rows wave, wave + nw, ...; kVBatch value rows in flight --------------
+            constexpr int RP = 64 / GS;          // rows whose weights one pass over the lanes computes
+            constexpr int NPASS = kVBatch / RP;  // GS = 4: 1, GS = 8: 2, GS = 16: 4
+            const char* vtree = reinterpret_cast<const char*>(p.values) + row0 * (size_t)(D * 2);
+            // where the rows of a batch sit (row `le` of the round is row `rem` of the stretch of the
+            // wave it falls in; lane = (row of the pass, head)), and their value rows
+            auto issue = [&](int e0, int (&at_v)[NPASS], uint32_t (&vraw)[kVBatch][VW]) {
+#pragma unroll
+                for (int ps = 0; ps < NPASS; ++ps) {
+                    const int le = e0 + (ps * RP + lane_o / GS) * nw;
+                    int rem = le, at = -1;
+#pragma unroll
+                    for (int w = 0; w < kMfmaWaves; ++w) {
+                        if (at < 0 && rem < cw[w]) at = w * (NB * S::ROWS) + rem;
+                        rem -= cw[w];
+                    }
+                    // -> its row in the score table (-1: past the end)
+                    at_v[ps] = (le < tot && at >= 0) ? (int)lst_row[at] : -1;
+                }
+                int slot_v[NPASS];  // the key slots of all the rows of a pass
+#pragma unroll
+                for (int ps = 0; ps < NPASS; ++ps)
+                    slot_v[ps] = at_v[ps] >= 0 ? (int)(lst_tslot[at_v[ps] >> 4] + (unsigned)(at_v[ps] & 15)) : 0;
+                // (a batch is always loaded whole, rows past the end as slot 0: straight-line code)
+#pragma unroll
+                for (int i = 0; i < kVBatch; ++i) {
+                    {
+                        const unsigned slot = (unsigned)__builtin_amdgcn_readlane(slot_v[i / RP], (i % RP) * GS);
+                        const uint16_t* vp =
+                            reinterpret_cast<const uint16_t*>(vtree + (size_t)slot * (D * 2)) + lane_o * VPL;
+                        if (VPL == 1) {
+                            vraw[i][0] = *vp;
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < VPL / 2; ++e)
+                                vraw[i][e] = reinterpret_cast<const uint32_t*>(vp)[e];
+                        }
+                    }
+                }
+            };
+            auto consume = [&](int e0, const int (&at_v)[NPASS], const uint32_t (&vraw)[kVBatch][VW]) {
+                // (nothing of what follows may be scheduled ahead of loads issued before this point)
+                __builtin_amdgcn_sched_barrier(0);
+                // scores -> weights, in place, 64 (row, head) pairs at a time
+#pragma unroll
+                for (int ps = 0; ps < NPASS; ++ps) {
+                    if (at_v[ps] >= 0) {
+                        float* zp = lst_z + at_v[ps] * GS + (lane_o & (GS - 1));
+                        const float w = __builtin_amdgcn_exp2f(*zp - m_lane);
+                        l_mine += w;
+                        *zp = w;
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < kVBatch; ++i) {
+                    if (e0 + i * nw >= tot) break;  // uniform
+                    const int at = __builtin_amdgcn_readlane(at_v[i / RP], (i % RP) * GS);
+                    float vf[VPL];
+                    if (VPL == 1) {
+                        vf[0] = bf16_lo(vraw[i][0]);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < VPL / 2; ++e) {
+                            vf[2 * e] = bf16_lo(vraw[i][e]);
+                            vf[2 * e + 1] = bf16_hi(vraw[i][e]);
+                        }
+                    }
+                    const float* wr = lst_z + at * GS;  // weights of this row, one per head
+#pragma unroll
+                    for (int g = 0; g < GS; ++g) {
+                        const float w = wr[g];  // same address in every lane: a broadcast read
+#pragma unroll
+                        for (int e = 0; e < VPL; ++e) acc[g][e] += w * vf[e];
+                    }
+                }
+            };
+            for (int e0 = wave; e0 < tot; e0 += nw * kVBatch) {  // uniform in the wave
+                int at_v[NPASS];
+                uint32_t vraw[kVBatch][VW];
+                issue(e0, at_v, vraw);
+                consume(e0, at_v, vraw);
+            }
+            if (r == 0) HIRA_TL(11);
         }
-        if (r == 0) HIRA_TL(11);
-    }
+    }  // tree or queue
     if (!want_attn) return;  // uniform
     HIRA_TL(2);
 

@@ -265,6 +265,35 @@ def test_attention_with_queue_and_empty_selection(gpu_device):
     assert float(z.abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("h_kv,h_q,m", [(2, 8, 1), (2, 8, 37), (1, 8, 200), (2, 32, 64)])
+def test_mfma_attention_with_queue(h_kv, h_q, m, gpu_device):
+    """bf16 tiled index (MFMA kernel) plus a row-major queue of m keys per tree that every
+    head attends to; both kernels against the fp64 oracle over index rows >= tau + queue."""
+    from hira_amd.searcher.hip import HIPSearcher
+
+    d = 128
+    print(f"case h_kv={h_kv} h_q={h_q} m={m}", flush=True)
+    c = _setup(h_kv, h_q, 2048, d, 32, 3, torch.bfloat16, seed=77 + m, keep=40)
+    assert c["idx"].tiled
+    rng = np.random.default_rng(m)
+    qk = bf16_round(rng.normal(size=(h_kv, m, d)).astype(np.float32) * 0.3)
+    qv = bf16_round(rng.normal(size=(h_kv, m, d)).astype(np.float32))
+    sc = torch.full((h_q,), d ** -0.5)
+    th = c["th"].copy()
+    th[1] = 1e9  # head 1 selects nothing from the index: only the queue remains
+    keys_all = np.concatenate([c["ff"].keys, qk], axis=1)
+    vals_all = np.concatenate([c["vslot"], qv], axis=1)
+    mask = (c["s"] >= th[:, None]) & c["valid"]
+    mask = np.concatenate([mask, np.ones((h_q, m), bool)], axis=1)
+    ref = ho.attention(keys_all, vals_all, c["q"], sc.numpy(), mask, c["q2kv"])
+    for kernel in (2, 1):
+        out = HIPSearcher(kernel=kernel).search_attention(
+            torch.from_numpy(c["q"]), torch.from_numpy(th), c["idx"], scaling=sc,
+            queue_keys=torch.from_numpy(qk).to(torch.bfloat16),
+            queue_values=torch.from_numpy(qv).to(torch.bfloat16)).cpu().numpy()
+        assert rel_err(out, ref) <= 2e-3, (kernel, rel_err(out, ref))
+
+
 def test_bad_inputs_raise_value_error(gpu_device):
     """tests/test_triton_kernels.py:547-601 of the reference."""
     from hira_amd.searcher.hip import HIPSearcher
