@@ -1,0 +1,235 @@
+// Nearest-centroid assignment of the index build on the matrix cores (bf16 rows).
+//
+// Replaces the distance step of the reference's k-means (faiss.Kmeans.train / index.search,
+// indexer/cpu.py:239-250) and of its capacity packing (indexer/cuda.py:247-334):
+//   argmin_k ||x_i - c_k||^2 = argmin_k (||c_k||^2 - 2 x_i.c_k),
+// with X.C^T on v_mfma_f32_16x16x32_bf16 and the argmin fused into the epilogue, so the
+// n x K distance matrix is never written.  Items are bf16 (exact operands).  Centroids are
+// fp32 means: each is split into two bf16 numbers, c = hi + lo (16 bits of mantissa), and
+// both halves are multiplied, so the distances are as good as fp32 ones for choosing the
+// nearest centroid.
+//
+// k_cent_prep   centroids (T, K, D) fp32 -> tiles of 16 centroids, hi and lo halves, in the
+//               operand layout (chunk (s, kb, i) of 16 bytes at s*64 + kb*16 + i), plus
+//               ||hi + lo||^2; a centroid that is full (fill[k] >= bf) or past K gets +inf.
+// k_assign_mfma a workgroup of 4 waves owns 256 items (64 a wave: 4 operand tiles kept in
+//               registers) and walks all centroid tiles; a tile is staged once per workgroup
+//               in LDS (double buffered, one barrier a tile).  Lane (n, kb) of a wave sees
+//               the products of its centroid column n with rows 4*kb + j, keeps the best
+//               (value, index) per row, and the 16 columns are merged at the end
+//               (lowest index on ties).
+#include "common.hip.h"
+
+namespace hira {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 abf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float af32x4_t;
+
+constexpr int kAssignRI = 4;       // operand tiles of 16 items per wave
+constexpr int kAssignThreads = 256;
+
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+    return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
+}
+
+template <int KS>
+__global__ __launch_bounds__(64) void k_cent_prep(const float* cent, int K, const int32_t* fill,
+                                                  int bf, uint4* tiles, float* cn2, int Kt) {
+    constexpr int D = 32 * KS;
+    const int lane = threadIdx.x & 63, i = lane & 15, kb = lane >> 4;
+    const int tile = blockIdx.x, t = blockIdx.y;
+    const int k = tile * 16 + i;
+    uint4* out = tiles + ((size_t)t * Kt + tile) * (size_t)(2 * KS * 64);
+    float ss = 0.0f;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+        float c[8], hi[8], lo[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            c[e] = k < K ? cent[((size_t)t * K + k) * D + s * 32 + kb * 8 + e] : 0.0f;
+            hi[e] = bf16_bits_to_f32(f32_to_bf16_bits(c[e]));
+            lo[e] = bf16_bits_to_f32(f32_to_bf16_bits(c[e] - hi[e]));
+            const float v = hi[e] + lo[e];
+            ss += v * v;
+        }
+        out[s * 64 + kb * 16 + i] = make_uint4(pack_bf16(hi[0], hi[1]), pack_bf16(hi[2], hi[3]),
+                                               pack_bf16(hi[4], hi[5]), pack_bf16(hi[6], hi[7]));
+        out[KS * 64 + s * 64 + kb * 16 + i] =
+            make_uint4(pack_bf16(lo[0], lo[1]), pack_bf16(lo[2], lo[3]), pack_bf16(lo[4], lo[5]),
+                       pack_bf16(lo[6], lo[7]));
+    }
+    ss += __shfl_xor(ss, 16, 64);
+    ss += __shfl_xor(ss, 32, 64);
+    if (kb == 0) {
+        const bool usable = k < K && !(fill != nullptr && fill[(size_t)t * K + k] >= bf);
+        cn2[((size_t)t * Kt + tile) * 16 + i] = usable ? ss : INFINITY;
+    }
+}
+
+template <int KS>
+__global__ __launch_bounds__(kAssignThreads, 2) void k_assign_mfma(
+    const void* x, int n_c, size_t x_tree_stride, const uint4* tiles, const float* cn2, int Kt,
+    const int32_t* list, const int32_t* list_count, size_t list_stride, int32_t* assign,
+    float* dist) {
+    constexpr int D = 32 * KS;
+    constexpr int RI = kAssignRI;
+    constexpr int TILE_CHUNKS = 2 * KS * 64;                 // hi and lo halves of 16 centroids
+    constexpr int CPT = TILE_CHUNKS / kAssignThreads;        // chunks a thread stages per tile
+    static_assert(TILE_CHUNKS % kAssignThreads == 0, "tile does not split over the workgroup");
+    __shared__ uint4 s_c[2][TILE_CHUNKS];
+    __shared__ float s_n2[2][16];
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n = lane & 15, kb = lane >> 4;  // operand row / centroid column, column block
+    const int t = blockIdx.y;
+    const int n_items = list ? list_count[t] : n_c;
+    const int first = (blockIdx.x * (kAssignThreads / 64) + wave) * (RI * 16);
+    if ((int)blockIdx.x * (kAssignThreads / 64) * (RI * 16) >= n_items) return;  // uniform
+
+    // ---- my items: operand tiles in registers, ||x||^2 of row lane % 16 ------------------
+    int item[RI];
+    uint4 a[RI][KS];
+    float x2[RI];
+#pragma unroll
+    for (int ri = 0; ri < RI; ++ri) {
+        const int pos = first + ri * 16 + n;
+        item[ri] = -1;
+        if (pos < n_items) item[ri] = list ? list[(size_t)t * list_stride + pos] : pos;
+        float ss = 0.0f;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            a[ri][s] = make_uint4(0, 0, 0, 0);
+            if (item[ri] >= 0)
+                a[ri][s] = *reinterpret_cast<const uint4*>(
+                    reinterpret_cast<const uint16_t*>(x) +
+                    ((size_t)t * x_tree_stride + item[ri]) * D + s * 32 + kb * 8);
+            float f[8];
+            unpack<bf16_t>(a[ri][s], f);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ss += f[e] * f[e];
+        }
+        ss += __shfl_xor(ss, 16, 64);
+        ss += __shfl_xor(ss, 32, 64);
+        x2[ri] = ss;
+    }
+    float best[RI][4];
+    int arg[RI][4];
+#pragma unroll
+    for (int ri = 0; ri < RI; ++ri)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            best[ri][j] = INFINITY;
+            arg[ri][j] = -1;
+        }
+
+    // ---- all centroid tiles, staged through LDS -------------------------------------------
+    const uint4* tt = tiles + (size_t)t * Kt * TILE_CHUNKS;
+    const float* n2t = cn2 + (size_t)t * Kt * 16;
+    uint4 stage[CPT];
+    float stage_n2 = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CPT; ++c) s_c[0][threadIdx.x + c * kAssignThreads] = tt[threadIdx.x + c * kAssignThreads];
+    if (threadIdx.x < 16) s_n2[0][threadIdx.x] = n2t[threadIdx.x];
+    __syncthreads();
+    for (int tile = 0; tile < Kt; ++tile) {
+        const int cur = tile & 1;
+        if (tile + 1 < Kt) {  // the next tile is on its way while this one is used
+#pragma unroll
+            for (int c = 0; c < CPT; ++c)
+                stage[c] = tt[(size_t)(tile + 1) * TILE_CHUNKS + threadIdx.x + c * kAssignThreads];
+            if (threadIdx.x < 16) stage_n2 = n2t[(tile + 1) * 16 + threadIdx.x];
+        }
+        abf16x8_t bh[KS], bl[KS];
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            bh[s] = __builtin_bit_cast(abf16x8_t, s_c[cur][s * 64 + lane]);
+            bl[s] = __builtin_bit_cast(abf16x8_t, s_c[cur][KS * 64 + s * 64 + lane]);
+        }
+        const float n2 = s_n2[cur][n];
+        const int kcol = tile * 16 + n;
+#pragma unroll
+        for (int ri = 0; ri < RI; ++ri) {
+            af32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+                const abf16x8_t av = __builtin_bit_cast(abf16x8_t, a[ri][s]);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bh[s], acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bl[s], acc, 0, 0, 0);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float v = n2 - 2.0f * acc[j];
+                if (v < best[ri][j]) {  // tiles come in increasing order: ties keep the lower k
+                    best[ri][j] = v;
+                    arg[ri][j] = kcol;
+                }
+            }
+        }
+        if (tile + 1 < Kt) {
+#pragma unroll
+            for (int c = 0; c < CPT; ++c) s_c[cur ^ 1][threadIdx.x + c * kAssignThreads] = stage[c];
+            if (threadIdx.x < 16) s_n2[cur ^ 1][threadIdx.x] = stage_n2;
+        }
+        __syncthreads();
+    }
+
+    // ---- merge the 16 centroid columns of a row group; column 0 writes -----------------------
+#pragma unroll
+    for (int ri = 0; ri < RI; ++ri)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float b = best[ri][j];
+            int g = arg[ri][j];
+#pragma unroll
+            for (int off = 1; off < 16; off <<= 1) {
+                const float ob = __shfl_xor(b, off, 64);
+                const int og = __shfl_xor(g, off, 64);
+                if (og >= 0 && (g < 0 || ob < b || (ob == b && og < g))) {
+                    b = ob;
+                    g = og;
+                }
+            }
+            // row 4*kb + j of the operand tile: its item and ||x||^2 live in lane 4*kb + j
+            const int it = __shfl(item[ri], 4 * kb + j, 64);
+            const float xx = __shfl(x2[ri], 4 * kb + j, 64);
+            if (n == 0 && it >= 0) {
+                assign[(size_t)t * n_c + it] = g;
+                dist[(size_t)t * n_c + it] = fmaxf(b + xx, 0.0f);
+            }
+        }
+}
+
+// hi/lo tiles and norms of the centroids of every tree
+int launch_cent_prep(int dim, const float* cent, int K, int num_trees, const int32_t* fill, int bf,
+                     void* tiles, float* cn2, hipStream_t s) {
+    const int Kt = (K + 15) / 16;
+    const dim3 grid(Kt, num_trees);
+    uint4* tl = reinterpret_cast<uint4*>(tiles);
+    switch (dim) {
+        case 64: hipLaunchKernelGGL((k_cent_prep<2>), grid, dim3(64), 0, s, cent, K, fill, bf, tl, cn2, Kt); break;
+        case 128: hipLaunchKernelGGL((k_cent_prep<4>), grid, dim3(64), 0, s, cent, K, fill, bf, tl, cn2, Kt); break;
+        case 256: hipLaunchKernelGGL((k_cent_prep<8>), grid, dim3(64), 0, s, cent, K, fill, bf, tl, cn2, Kt); break;
+        default: return fail(HIRA_EINVAL, "MFMA assignment: dim %d", dim);
+    }
+    return HIRA_OK;
+}
+
+// nearest usable centroid of every item (or of the items list[0 .. *list_count) of each tree)
+int launch_assign_mfma(int dim, const void* x, int n_c, size_t x_tree_stride, const void* tiles,
+                       const float* cn2, int K, int num_trees, const int32_t* list,
+                       const int32_t* list_count, size_t list_stride, int32_t* assign, float* dist,
+                       hipStream_t s) {
+    const int Kt = (K + 15) / 16;
+    const int per_block = (kAssignThreads / 64) * kAssignRI * 16;
+    const dim3 grid((n_c + per_block - 1) / per_block, num_trees);
+    const uint4* tl = reinterpret_cast<const uint4*>(tiles);
+    switch (dim) {
+        case 64: hipLaunchKernelGGL((k_assign_mfma<2>), grid, dim3(kAssignThreads), 0, s, x, n_c, x_tree_stride, tl, cn2, Kt, list, list_count, list_stride, assign, dist); break;
+        case 128: hipLaunchKernelGGL((k_assign_mfma<4>), grid, dim3(kAssignThreads), 0, s, x, n_c, x_tree_stride, tl, cn2, Kt, list, list_count, list_stride, assign, dist); break;
+        case 256: hipLaunchKernelGGL((k_assign_mfma<8>), grid, dim3(kAssignThreads), 0, s, x, n_c, x_tree_stride, tl, cn2, Kt, list, list_count, list_stride, assign, dist); break;
+        default: return fail(HIRA_EINVAL, "MFMA assignment: dim %d", dim);
+    }
+    return HIRA_OK;
+}
+
+}  // namespace hira

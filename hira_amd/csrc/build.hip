@@ -487,6 +487,8 @@ struct Carver {
 
 struct BuildWs {
     float* cent_f32;
+    void* cent_tiles;  // centroids as bf16 operand tiles (matrix-core assignment), or NULL
+    float* cent_n2;
     int32_t *assign, *placed, *members, *sorted, *list, *list_count;
     float* dist;
     int32_t *counts, *offsets, *cursor, *fill, *scratch;
@@ -497,6 +499,19 @@ struct BuildWs {
 };
 
 static int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// assign_mfma.hip
+int launch_cent_prep(int dim, const float* cent, int K, int num_trees, const int32_t* fill, int bf,
+                     void* tiles, float* cn2, hipStream_t s);
+int launch_assign_mfma(int dim, const void* x, int n_c, size_t x_tree_stride, const void* tiles,
+                       const float* cn2, int K, int num_trees, const int32_t* list,
+                       const int32_t* list_count, size_t list_stride, int32_t* assign, float* dist,
+                       hipStream_t s);
+
+// bf16 rows of 64, 128 or 256 columns are assigned on the matrix cores
+static bool assign_on_mfma(const HiraTree* t) {
+    return t->dtype == HIRA_BF16 && (t->dim == 64 || t->dim == 128 || t->dim == 256);
+}
 
 // cluster counts per level: K[0] = n, K[l] = ceil(K[l-1] / bf)
 static void cluster_counts(int n, int bf, int L, int* K) {
@@ -512,6 +527,13 @@ static void carve(const HiraTree* t, int n, void* ws, BuildWs* b) {
     Carver c{reinterpret_cast<char*>(ws), 0};
     const size_t k1 = L >= 2 ? (size_t)K[1] : 1;
     b->cent_f32 = c.take<float>((size_t)T * k1 * D);
+    b->cent_tiles = nullptr;
+    b->cent_n2 = nullptr;
+    if (assign_on_mfma(t)) {
+        const size_t kpad = (k1 + 15) / 16 * 16;
+        b->cent_tiles = c.take<char>((size_t)T * kpad * D * 4);  // hi and lo halves, 2 bytes each
+        b->cent_n2 = c.take<float>((size_t)T * kpad);
+    }
     b->assign = c.take<int32_t>((size_t)T * n);
     b->placed = c.take<int32_t>((size_t)T * n);
     b->members = c.take<int32_t>((size_t)T * n);
@@ -590,8 +612,16 @@ static int build_impl(const HiraTree* t, const void* keys_in, const void* values
         hipLaunchKernelGGL((k_init_centroids<T>), g_cent, dim3(64), 0, s, x, n_c, xs, Kl, D,
                            seed + 7919ull * (uint64_t)l, w.cent_f32);
         for (int it = 0; it < niter; ++it) {
-            int rc = launch_assign<T>(lpr, g_assign, s, x, n_c, xs, w.cent_f32, Kl, D, nullptr, bf,
+            int rc;
+            if (w.cent_tiles != nullptr) {
+                rc = launch_cent_prep(D, w.cent_f32, Kl, NT, nullptr, bf, w.cent_tiles, w.cent_n2, s);
+                if (rc == HIRA_OK)
+                    rc = launch_assign_mfma(D, x, n_c, xs, w.cent_tiles, w.cent_n2, Kl, NT, nullptr,
+                                            nullptr, 0, w.assign, w.dist, s);
+            } else {
+                rc = launch_assign<T>(lpr, g_assign, s, x, n_c, xs, w.cent_f32, Kl, D, nullptr, bf,
                                       nullptr, nullptr, 0, w.assign, w.dist);
+            }
             if (rc != HIRA_OK) return rc;
             fill_i32(w.counts, (size_t)NT * Kl, 0, s);
             hipLaunchKernelGGL(k_bucket_count, g_items, dim3(256), 0, s, w.assign, n_c, nullptr,
@@ -616,8 +646,16 @@ static int build_impl(const HiraTree* t, const void* keys_in, const void* values
                 hipLaunchKernelGGL(k_collect_unplaced, g_items, dim3(256), 0, s, w.placed, n_c,
                                    w.list, w.list_count);
             }
-            int rc = launch_assign<T>(lpr, g_assign, s, x, n_c, xs, w.cent_f32, Kl, D, w.fill, bf,
+            int rc;
+            if (w.cent_tiles != nullptr) {  // full centroids get an infinite norm: never nearest
+                rc = launch_cent_prep(D, w.cent_f32, Kl, NT, w.fill, bf, w.cent_tiles, w.cent_n2, s);
+                if (rc == HIRA_OK)
+                    rc = launch_assign_mfma(D, x, n_c, xs, w.cent_tiles, w.cent_n2, Kl, NT, list,
+                                            lcnt, (size_t)n_c, w.assign, w.dist, s);
+            } else {
+                rc = launch_assign<T>(lpr, g_assign, s, x, n_c, xs, w.cent_f32, Kl, D, w.fill, bf,
                                       list, lcnt, (size_t)n_c, w.assign, w.dist);
+            }
             if (rc != HIRA_OK) return rc;
             fill_i32(w.counts, (size_t)NT * Kl, 0, s);
             hipLaunchKernelGGL(k_bucket_count, g_items, dim3(256), 0, s, w.assign, n_c, list, lcnt,
