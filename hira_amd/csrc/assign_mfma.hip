@@ -13,8 +13,8 @@
 //               operand layout (chunk (s, kb, i) of 16 bytes at s*64 + kb*16 + i), plus
 //               ||hi + lo||^2; a centroid that is full (fill[k] >= bf) or past K gets +inf.
 // k_assign_mfma a workgroup of 4 waves owns 256 items (64 a wave: 4 operand tiles kept in
-//               registers) and walks all centroid tiles; a tile is staged once per workgroup
-//               in LDS (double buffered, one barrier a tile).  Lane (n, kb) of a wave sees
+//               registers) and walks all centroid tiles; four tiles at a time are staged once
+//               per workgroup in LDS (double buffered, one barrier a stage).  Lane (n, kb) of a wave sees
 //               the products of its centroid column n with rows 4*kb + j, keeps the best
 //               (value, index) per row, and the 16 columns are merged at the end
 //               (lowest index on ties).
@@ -27,6 +27,10 @@ typedef __attribute__((ext_vector_type(4))) float af32x4_t;
 
 constexpr int kAssignRI = 4;       // operand tiles of 16 items per wave
 constexpr int kAssignThreads = 256;
+constexpr int kAssignStage = 4;    // centroid tiles staged together: the time they keep the
+                                   // matrix cores busy covers the latency of fetching the next
+                                   // four (two for D = 256, whose tiles are twice as large)
+constexpr int assign_stage(int KS) { return KS <= 4 ? kAssignStage : kAssignStage / 2; }
 
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
     return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
@@ -35,6 +39,7 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
 template <int KS>
 __global__ __launch_bounds__(64) void k_cent_prep(const float* cent, int K, const int32_t* fill,
                                                   int bf, uint4* tiles, float* cn2, int Kt) {
+    // (Kt counts whole stages of kAssignStage tiles: the tiles past K are zeros with norm +inf)
     constexpr int D = 32 * KS;
     const int lane = threadIdx.x & 63, i = lane & 15, kb = lane >> 4;
     const int tile = blockIdx.x, t = blockIdx.y;
@@ -74,10 +79,14 @@ __global__ __launch_bounds__(kAssignThreads, 2) void k_assign_mfma(
     constexpr int D = 32 * KS;
     constexpr int RI = kAssignRI;
     constexpr int TILE_CHUNKS = 2 * KS * 64;                 // hi and lo halves of 16 centroids
-    constexpr int CPT = TILE_CHUNKS / kAssignThreads;        // chunks a thread stages per tile
-    static_assert(TILE_CHUNKS % kAssignThreads == 0, "tile does not split over the workgroup");
-    __shared__ uint4 s_c[2][TILE_CHUNKS];
-    __shared__ float s_n2[2][16];
+    constexpr int TPS = assign_stage(KS);
+    constexpr int STAGE_CHUNKS = TPS * TILE_CHUNKS;
+    constexpr int CPT = STAGE_CHUNKS / kAssignThreads;       // chunks a thread stages per stage
+    static_assert(STAGE_CHUNKS % kAssignThreads == 0, "stage does not split over the workgroup");
+    extern __shared__ uint4 s_dyn[];                         // two stages of tiles, then their norms
+    uint4* s_c0 = s_dyn;
+    uint4* s_c1 = s_dyn + STAGE_CHUNKS;
+    float* s_n2 = reinterpret_cast<float*>(s_dyn + 2 * STAGE_CHUNKS);  // (2, TPS * 16)
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, kb = lane >> 4;  // operand row / centroid column, column block
@@ -122,54 +131,67 @@ __global__ __launch_bounds__(kAssignThreads, 2) void k_assign_mfma(
             arg[ri][j] = -1;
         }
 
-    // ---- all centroid tiles, staged through LDS -------------------------------------------
-    const uint4* tt = tiles + (size_t)t * Kt * TILE_CHUNKS;
-    const float* n2t = cn2 + (size_t)t * Kt * 16;
+    // ---- all centroid tiles, staged through LDS TPS at a time (the last stage may hold fewer;
+    // the arrays are padded to whole stages, their norms with +inf) ---------------------------
+    const int Ks = (Kt + TPS - 1) / TPS;  // stages
+    const uint4* tt = tiles + (size_t)t * Ks * STAGE_CHUNKS;
+    const float* n2t = cn2 + (size_t)t * Ks * (TPS * 16);
     uint4 stage[CPT];
     float stage_n2 = 0.0f;
 #pragma unroll
-    for (int c = 0; c < CPT; ++c) s_c[0][threadIdx.x + c * kAssignThreads] = tt[threadIdx.x + c * kAssignThreads];
-    if (threadIdx.x < 16) s_n2[0][threadIdx.x] = n2t[threadIdx.x];
+    for (int c = 0; c < CPT; ++c) s_c0[threadIdx.x + c * kAssignThreads] = tt[threadIdx.x + c * kAssignThreads];
+    if (threadIdx.x < TPS * 16) s_n2[threadIdx.x] = n2t[threadIdx.x];
     __syncthreads();
-    for (int tile = 0; tile < Kt; ++tile) {
-        const int cur = tile & 1;
-        if (tile + 1 < Kt) {  // the next tile is on its way while this one is used
+    for (int st = 0; st < Ks; ++st) {
+        const uint4* cbuf = (st & 1) ? s_c1 : s_c0;
+        uint4* nbuf = (st & 1) ? s_c0 : s_c1;
+        const float* n2buf = s_n2 + (st & 1) * (TPS * 16);
+        // the next stage is on its way while this one is used (after the last stage: the last
+        // one again, unused; straight-line code keeps `stage` in registers)
+        const int nst = min(st + 1, Ks - 1);
 #pragma unroll
-            for (int c = 0; c < CPT; ++c)
-                stage[c] = tt[(size_t)(tile + 1) * TILE_CHUNKS + threadIdx.x + c * kAssignThreads];
-            if (threadIdx.x < 16) stage_n2 = n2t[(tile + 1) * 16 + threadIdx.x];
-        }
-        abf16x8_t bh[KS], bl[KS];
+        for (int c = 0; c < CPT; ++c)
+            stage[c] = tt[(size_t)nst * STAGE_CHUNKS + threadIdx.x + c * kAssignThreads];
+        stage_n2 = n2t[nst * (TPS * 16) + (threadIdx.x & (TPS * 16 - 1))];
 #pragma unroll
-        for (int s = 0; s < KS; ++s) {
-            bh[s] = __builtin_bit_cast(abf16x8_t, s_c[cur][s * 64 + lane]);
-            bl[s] = __builtin_bit_cast(abf16x8_t, s_c[cur][KS * 64 + s * 64 + lane]);
-        }
-        const float n2 = s_n2[cur][n];
-        const int kcol = tile * 16 + n;
-#pragma unroll
-        for (int ri = 0; ri < RI; ++ri) {
-            af32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+        for (int ti = 0; ti < TPS; ++ti) {
+            abf16x8_t bh[KS], bl[KS];
 #pragma unroll
             for (int s = 0; s < KS; ++s) {
-                const abf16x8_t av = __builtin_bit_cast(abf16x8_t, a[ri][s]);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bh[s], acc, 0, 0, 0);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bl[s], acc, 0, 0, 0);
+                bh[s] = __builtin_bit_cast(abf16x8_t, cbuf[ti * TILE_CHUNKS + s * 64 + lane]);
+                bl[s] = __builtin_bit_cast(abf16x8_t, cbuf[ti * TILE_CHUNKS + KS * 64 + s * 64 + lane]);
+            }
+            const float n2 = n2buf[ti * 16 + n];
+            const int kcol = (st * TPS + ti) * 16 + n;
+            // four independent accumulator chains: a product never waits for the one before it
+            af32x4_t acc[RI];
+#pragma unroll
+            for (int ri = 0; ri < RI; ++ri) acc[ri] = af32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+#pragma unroll
+                for (int ri = 0; ri < RI; ++ri)
+                    acc[ri] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        __builtin_bit_cast(abf16x8_t, a[ri][s]), bh[s], acc[ri], 0, 0, 0);
+#pragma unroll
+                for (int ri = 0; ri < RI; ++ri)
+                    acc[ri] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                        __builtin_bit_cast(abf16x8_t, a[ri][s]), bl[s], acc[ri], 0, 0, 0);
             }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float v = n2 - 2.0f * acc[j];
-                if (v < best[ri][j]) {  // tiles come in increasing order: ties keep the lower k
-                    best[ri][j] = v;
-                    arg[ri][j] = kcol;
+            for (int ri = 0; ri < RI; ++ri)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float v = n2 - 2.0f * acc[ri][j];
+                    if (v < best[ri][j]) {  // tiles come in increasing order: ties keep the lower k
+                        best[ri][j] = v;
+                        arg[ri][j] = kcol;
+                    }
                 }
-            }
         }
-        if (tile + 1 < Kt) {
 #pragma unroll
-            for (int c = 0; c < CPT; ++c) s_c[cur ^ 1][threadIdx.x + c * kAssignThreads] = stage[c];
-            if (threadIdx.x < 16) s_n2[cur ^ 1][threadIdx.x] = stage_n2;
-        }
+        for (int c = 0; c < CPT; ++c) nbuf[threadIdx.x + c * kAssignThreads] = stage[c];
+        if (threadIdx.x < TPS * 16) s_n2[((st + 1) & 1) * (TPS * 16) + threadIdx.x] = stage_n2;
         __syncthreads();
     }
 
@@ -199,10 +221,16 @@ __global__ __launch_bounds__(kAssignThreads, 2) void k_assign_mfma(
         }
 }
 
+// centroid tiles per tree, in whole stages
+int assign_tiles(int K) {
+    const int kt = (K + 15) / 16;
+    return (kt + kAssignStage - 1) / kAssignStage * kAssignStage;
+}
+
 // hi/lo tiles and norms of the centroids of every tree
 int launch_cent_prep(int dim, const float* cent, int K, int num_trees, const int32_t* fill, int bf,
                      void* tiles, float* cn2, hipStream_t s) {
-    const int Kt = (K + 15) / 16;
+    const int Kt = assign_tiles(K);
     const dim3 grid(Kt, num_trees);
     uint4* tl = reinterpret_cast<uint4*>(tiles);
     switch (dim) {
@@ -219,14 +247,27 @@ int launch_assign_mfma(int dim, const void* x, int n_c, size_t x_tree_stride, co
                        const float* cn2, int K, int num_trees, const int32_t* list,
                        const int32_t* list_count, size_t list_stride, int32_t* assign, float* dist,
                        hipStream_t s) {
-    const int Kt = (K + 15) / 16;
+    const int Kt = assign_tiles(K);
     const int per_block = (kAssignThreads / 64) * kAssignRI * 16;
+    const int tps = assign_stage(dim / 32);
+    const size_t smem = 2 * (size_t)tps * (2 * (dim / 32) * 64) * sizeof(uint4) + 2 * (size_t)tps * 16 * sizeof(float);
     const dim3 grid((n_c + per_block - 1) / per_block, num_trees);
     const uint4* tl = reinterpret_cast<const uint4*>(tiles);
     switch (dim) {
-        case 64: hipLaunchKernelGGL((k_assign_mfma<2>), grid, dim3(kAssignThreads), 0, s, x, n_c, x_tree_stride, tl, cn2, Kt, list, list_count, list_stride, assign, dist); break;
-        case 128: hipLaunchKernelGGL((k_assign_mfma<4>), grid, dim3(kAssignThreads), 0, s, x, n_c, x_tree_stride, tl, cn2, Kt, list, list_count, list_stride, assign, dist); break;
-        case 256: hipLaunchKernelGGL((k_assign_mfma<8>), grid, dim3(kAssignThreads), 0, s, x, n_c, x_tree_stride, tl, cn2, Kt, list, list_count, list_stride, assign, dist); break;
+#define HIRA_ASSIGN_MFMA(KS)                                                                        \
+    {                                                                                               \
+        /* more than 64 KiB of dynamic LDS has to be asked for */                                   \
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_assign_mfma<KS>),                  \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) \
+            return fail(HIRA_ELAUNCH, "MFMA assignment: %zu bytes of LDS refused", smem);              \
+        hipLaunchKernelGGL((k_assign_mfma<KS>), grid, dim3(kAssignThreads), smem, s, x, n_c,        \
+                           x_tree_stride, tl, cn2, Kt, list, list_count, list_stride, assign, dist); \
+    }                                                                                               \
+    break;
+        case 64: HIRA_ASSIGN_MFMA(2)
+        case 128: HIRA_ASSIGN_MFMA(4)
+        case 256: HIRA_ASSIGN_MFMA(8)
+#undef HIRA_ASSIGN_MFMA
         default: return fail(HIRA_EINVAL, "MFMA assignment: dim %d", dim);
     }
     return HIRA_OK;

@@ -501,6 +501,7 @@ struct BuildWs {
 static int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 // assign_mfma.hip
+int assign_tiles(int K);
 int launch_cent_prep(int dim, const float* cent, int K, int num_trees, const int32_t* fill, int bf,
                      void* tiles, float* cn2, hipStream_t s);
 int launch_assign_mfma(int dim, const void* x, int n_c, size_t x_tree_stride, const void* tiles,
@@ -530,7 +531,7 @@ static void carve(const HiraTree* t, int n, void* ws, BuildWs* b) {
     b->cent_tiles = nullptr;
     b->cent_n2 = nullptr;
     if (assign_on_mfma(t)) {
-        const size_t kpad = (k1 + 15) / 16 * 16;
+        const size_t kpad = (size_t)assign_tiles((int)k1) * 16;
         b->cent_tiles = c.take<char>((size_t)T * kpad * D * 4);  // hi and lo halves, 2 bytes each
         b->cent_n2 = c.take<float>((size_t)T * kpad);
     }
