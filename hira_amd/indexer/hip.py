@@ -425,3 +425,73 @@ class HIPIndexer(BaseIndexer):
             self.size = size
         self._tree_struct = None
         return self
+
+    @torch.no_grad()
+    def rebuild_subtree(self, node: int) -> "HIPIndexer":
+        """Re-cluster everything under node `node` of level 2 (its bf level-1 nodes and their
+        keys), in every tree: appends only ever grow radii around centres that never move
+        (indexer/cuda.py:544-701), so a subtree that took many of them is rebuilt from its
+        keys now and then.  The keys stay in the subtree's own slots [node*bf*bf,
+        (node+1)*bf*bf); its level-1 nodes get new centres, radii and counts; the level-2
+        node keeps its centre, gets the radius its new children need, and its ancestors are
+        inflated where that radius grew.  One small build per tree (the trees hold different
+        numbers of keys there)."""
+        if self.keys_buf is None:
+            raise ValueError("Indexer is not built: call build() first.")
+        if self.num_levels < 3:
+            raise ValueError("rebuild_subtree needs at least three levels")
+        bf = self.branching_factor
+        if not 0 <= node < self.size[2]:
+            raise ValueError(f"level-2 node {node} not in 0..{self.size[2] - 1}")
+        s0, n0 = node * bf * bf, node * bf
+        s1, n1 = min(s0 + bf * bf, self.cap[0]), min(n0 + bf, self.cap[1])
+        for t in range(self.num_trees):
+            perm_sub = self.perm[t, s0:s1].clone()
+            live = (perm_sub >= 0).nonzero().squeeze(1)
+            n = int(live.numel())
+            if n == 0:
+                continue
+            rows = self.keys_buf[t:t + 1, s0:s1]
+            rows = (from_tiled(rows) if self.tiled else rows)[0, live]
+            vals = None if self.values_buf is None else self.values_buf[t, s0:s1][live]
+            sub = HIPIndexer(2, self.max_iterations, bf, seed=self.seed + node,
+                             device=str(self.device), pack_rounds=self.pack_rounds,
+                             layout="tiled" if self.tiled else "row_major")
+            sub.build(rows[None, None], None if vals is None else vals[None, None])
+            k, m = sub.size[1], sub.size[0]  # level-1 nodes and key slots the subtree uses now
+            # keys, values, positions: the rebuilt slots first, the rest of the subtree empty
+            self.keys_buf[t, s0:s1] = 0
+            self.keys_buf[t, s0:s0 + m] = sub.keys_buf[0, :m]
+            if vals is not None:
+                self.values_buf[t, s0:s1] = 0
+                self.values_buf[t, s0:s0 + m] = sub.values_buf[0, :m]
+            sub_perm = sub.perm[0, :m].long()
+            self.perm[t, s0:s1] = -1
+            self.perm[t, s0:s0 + m] = torch.where(
+                sub_perm >= 0, perm_sub[live][sub_perm.clamp(min=0)],
+                torch.full_like(sub_perm, -1, dtype=torch.int32))
+            # level 1 (a tile of 16 centres is contiguous, so tiled rows copy as they are)
+            kc = -(-k // 16) * 16 if self.tiled else k
+            self.centers[1][t, n0:n1] = 0
+            self.centers[1][t, n0:n0 + kc] = sub.centers[1][0, :kc]
+            self.radii[1][t, n0:n1] = float("-inf")
+            self.radii[1][t, n0:n0 + k] = sub.radii[1][0, :k]
+            self.counts[1][t, n0:n1] = 0
+            self.counts[1][t, n0:n0 + k] = sub.counts[1][0, :k]
+            # level 2: same centre, the radius its children need; ancestors cover it
+            c1 = sub.centers_rowmajor(1)[0].float()
+            child, c_child, r_child = node, None, None
+            for l in range(2, self.num_levels):
+                tile0 = child // 16 * 16  # (de-tiling needs whole tiles)
+                cl = self.centers[l][t:t + 1, tile0:tile0 + 16]
+                cl = (from_tiled(cl) if self.tiled else cl)[0, child - tile0].float()
+                if l == 2:
+                    r = ((c1 - cl).norm(dim=1) + sub.radii[1][0, :k]).max() * (1 + 1e-6)
+                    self.counts[2][t, child] = k
+                else:
+                    r = torch.maximum(self.radii[l][t, child],
+                                      ((c_child - cl).norm() + r_child) * (1 + 1e-6))
+                self.radii[l][t, child] = r
+                c_child, r_child, child = cl, r, child // bf
+        self._tree_struct = None
+        return self

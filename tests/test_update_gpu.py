@@ -100,6 +100,44 @@ def test_update_keeps_tree_valid_and_search_exact(case, gpu_device):
     assert rel_err(att, ref) <= (2e-3 if dtype == torch.bfloat16 else 1e-5)
 
 
+@pytest.mark.parametrize("dtype,d,bf", [(torch.bfloat16, 128, 16), (torch.float32, 32, 8)])
+def test_rebuild_subtree_after_appends(dtype, d, bf, gpu_device):
+    """Appends loosen the balls of the nodes they land in; rebuilding a level-2 subtree
+    re-clusters its keys in place: the tree stays valid, nothing is lost, search is exact,
+    and the rebuilt level-1 balls are no larger on average than before."""
+    from hira_amd.indexer.hip import HIPIndexer
+    from hira_amd.searcher.hip import HIPSearcher
+
+    t, n0, m = 2, bf * bf * 3, bf * bf // 2
+    n = n0 + m
+    rnd = bf16_round if dtype == torch.bfloat16 else (lambda x: x)
+    keys = rnd(clustered_keys(t, n, d, seed=5, clusters=12))
+    vals = rnd(np.random.default_rng(1).normal(size=(t, n, d)).astype(np.float32))
+    K, V = torch.from_numpy(keys)[None].to(dtype), torch.from_numpy(vals)[None].to(dtype)
+    idx = HIPIndexer(3, 2, bf).build(K[:, :, :n0 - m], V[:, :, :n0 - m])
+    idx.update(K[:, :, n0 - m:], V[:, :, n0 - m:])
+    _check_tree(idx, keys, vals)
+    before = [idx.radii[1][:, : idx.size[1]].clone()]
+    for node in range(idx.size[2]):
+        idx.rebuild_subtree(node)
+    assert idx.num_keys == n
+    _check_tree(idx, keys, vals)
+    r0, r1 = before[0], idx.radii[1][:, : idx.size[1]]
+    assert float(r1[r1 > -1e30].mean()) <= float(r0[r0 > -1e30].mean()) * 1.05
+    q = rnd(random_query(2 * t, d, seed=3))
+    q2kv = ho.default_q2kv(2 * t, t)
+    s = ho.scores(keys, q, q2kv)
+    th = midpoint_threshold(s, n // 20)
+    out = HIPSearcher(index_space="position").search(torch.from_numpy(q), torch.from_numpy(th), idx)
+    assert_same_selection(out.cpu().numpy() != 0, s, th)
+    # and the index keeps taking appends afterwards
+    extra = rnd(clustered_keys(t, 40, d, seed=6, clusters=3))
+    idx.update(torch.from_numpy(extra)[None].to(dtype), torch.from_numpy(extra)[None].to(dtype))
+    _check_tree(idx, np.concatenate([keys, extra], 1), np.concatenate([vals, extra], 1))
+    with pytest.raises(ValueError):
+        idx.rebuild_subtree(idx.size[2])
+
+
 def test_update_is_reproducible_and_grows_capacity(gpu_device):
     from hira_amd.indexer.hip import HIPIndexer
 
