@@ -144,6 +144,56 @@ def cpu_baseline(w, index, queries, taus, scale, budget_s=20.0):
                        f"search = reference v3 C++ kernel, attention = numpy fp32")
 
 
+def streaming(a, w, index, plan, q_d, taus, out, dev):
+    """Decode with a growing index: per step one key/value per tree is appended (one update
+    launch), then one search + attention over the index as it stands; every
+    a.rebuild_every steps one level-2 subtree is re-clustered (round-robin).  Times are GPU
+    times between events; the update also has a host part (it reads the level sizes back)."""
+    import torch
+
+    from hira_amd import synth
+
+    S = a.stream
+    sk, sv = synth.make_stream(w, S)
+    sk, sv = sk.to(dev), sv.to(dev)
+    index._grow(index._needed_caps(S))  # room for all appends: no re-allocation while timed
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(S)]
+    rb = []
+    nq = q_d.shape[0]
+    torch.cuda.synchronize()
+    t_host_upd = 0.0
+    for t in range(S):
+        ev[t][0].record()
+        h0 = time.perf_counter()
+        index.update(sk[:, :, t:t + 1], sv[:, :, t:t + 1])
+        t_host_upd += time.perf_counter() - h0
+        ev[t][1].record()
+        plan.run(q_d[t % nq], taus[t % nq], out)
+        ev[t][2].record()
+        if a.rebuild_every > 0 and (t + 1) % a.rebuild_every == 0 and index.num_levels >= 3:
+            r0, r1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            r0.record()
+            index.rebuild_subtree(((t + 1) // a.rebuild_every - 1) % index.size[2])
+            r1.record()
+            rb.append((r0, r1))
+    torch.cuda.synchronize()
+    upd = [e[0].elapsed_time(e[1]) * 1e3 for e in ev]
+    sea = [e[1].elapsed_time(e[2]) * 1e3 for e in ev]
+    upd.sort()
+    sea.sort()
+    res = {"steps": S, "keys_after": index.num_keys, "level_sizes": index.size,
+           "update_us_per_step": {"mean": round(sum(upd) / S, 2), "median": round(upd[S // 2], 2),
+                                  "p99": round(upd[min(S - 1, int(S * 0.99))], 2)},
+           "update_host_us_per_step": round(t_host_upd * 1e6 / S, 2),
+           "search_attn_us_per_step": {"mean": round(sum(sea) / S, 2),
+                                       "median": round(sea[S // 2], 2),
+                                       "p99": round(sea[min(S - 1, int(S * 0.99))], 2)},
+           "subtree_rebuilds": len(rb),
+           "rebuild_ms_each": [round(x.elapsed_time(y), 2) for x, y in rb]}
+    log(f"[bench] streaming: {res}")
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -161,6 +211,10 @@ def main():
     ap.add_argument("--profile", action="store_true",
                     help="only the warm-up and the timed steps (no counter pass, no dense or "
                          "CPU comparators): every launch a profiler sees is the measured one")
+    ap.add_argument("--stream", type=int, default=0,
+                    help="after the timed steps: append this many keys one per step, a search "
+                         "after each, one level-2 subtree rebuilt every --rebuild-every steps")
+    ap.add_argument("--rebuild-every", type=int, default=512)
     ap.add_argument("--counters", action="store_true",
                     help="run the steps once, untimed, plus a kernel of known traffic "
                          "(for rocprofv3 --pmc runs)")
@@ -351,6 +405,8 @@ def main():
         "counters": {k: round(v, 1) for k, v in counts.items()},
         "index_build_ms": round(build_ms, 1),
     }
+    if a.stream > 0:
+        result["streaming"] = streaming(a, w, index, plan, q_d, taus, scratch, dev)
     if not a.no_cpu:
         try:
             result["cpu_baseline"] = cpu_baseline(w, index, q_d[W:], taus[W:], scale,

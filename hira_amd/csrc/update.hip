@@ -42,27 +42,6 @@ struct UpdateParams {
     int32_t* state;
 };
 
-__device__ __forceinline__ float block_sum(float v, float* red) {
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) v += __shfl_xor(v, off, 64);
-    __syncthreads();
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-    __syncthreads();
-    return red[0] + red[1] + red[2] + red[3];
-}
-
-// ||x - row||_2 with x in LDS (fp32) and row = node `node` of a tree matrix; whole workgroup
-template <typename T>
-__device__ __forceinline__ float block_dist(const float* x, const void* mat, size_t tree_base,
-                                            int layout, int D, size_t node, float* red) {
-    float ss = 0.0f;
-    for (int j = threadIdx.x; j < D; j += kUpdThreads) {
-        const float df = x[j] - load_elem<T>(mat, tree_base + elem_index(layout, D, node, j));
-        ss += df * df;
-    }
-    return sqrtf(block_sum(ss, red));
-}
-
 // a bound must survive the fp32 rounding of the sums that produced it
 __device__ __forceinline__ float pad_up(float r) { return r > 0.0f ? r * (1.0f + 4.0f * 1.1920929e-7f) + 1e-30f : r; }
 
@@ -77,26 +56,32 @@ __device__ int nearest_with_room(const UpdateParams& p, int tree, int l, int use
     const int32_t* cnt = p.counts[l] + base;
     float best = INFINITY;
     int arg = -1;
-    for (int n0 = wave * 64; n0 < used; n0 += 4 * 64) {
-        const int n = n0 + lane;
-        // a node in use with a free slot; count 0 marks a pad slot, which is not a node yet
-        const bool room = n < used && cnt[n] > 0 && cnt[n] < p.bf;
-        unsigned long long bal = __ballot(room);
-        while (bal != 0ull) {  // uniform in the wave
-            const int b = __ffsll((long long)bal) - 1;
-            bal &= bal - 1ull;
-            const int node = n0 + b;
-            float ss = 0.0f;
-            for (int j = lane; j < D; j += 64) {
-                const float df =
-                    x[j] - load_elem<T>(p.centers[l], base * D + elem_index(p.layout, D, (size_t)node, j));
-                ss += df * df;
-            }
+    for (int nb = wave * 64; nb < used; nb += 4 * 4 * 64) {
+        // four reads of child counts in flight (a wave's nodes still come in increasing order)
+        int c4[4];
 #pragma unroll
-            for (int off = 1; off < 64; off <<= 1) ss += __shfl_xor(ss, off, 64);
-            if (ss < best) {  // nodes come in increasing order inside a wave
-                best = ss;
-                arg = node;
+        for (int u = 0; u < 4; ++u) {
+            const int n = nb + u * 4 * 64 + lane;
+            c4[u] = n < used ? cnt[n] : 0;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            // a node in use with a free slot; count 0 marks a pad slot, which is not a node yet
+            unsigned long long bal = __ballot(c4[u] > 0 && c4[u] < p.bf);
+            while (bal != 0ull) {  // uniform in the wave
+                const int node = nb + u * 4 * 64 + __ffsll((long long)bal) - 1;
+                bal &= bal - 1ull;
+                float ss = 0.0f;
+                for (int j = lane; j < D; j += 64) {
+                    const float df = x[j] - load_elem<T>(p.centers[l], base * D + elem_index(p.layout, D, (size_t)node, j));
+                    ss += df * df;
+                }
+#pragma unroll
+                for (int off = 1; off < 64; off <<= 1) ss += __shfl_xor(ss, off, 64);
+                if (ss < best) {
+                    best = ss;
+                    arg = node;
+                }
             }
         }
     }
@@ -128,6 +113,7 @@ __global__ __launch_bounds__(kUpdThreads) void k_update(const UpdateParams p) {
     float* cbuf = sm + p.dim;   // (D) centre of the node being attached upwards
     __shared__ float red_f[4];
     __shared__ int red_i[4];
+    __shared__ float s_dist[HIRA_MAX_LEVELS], s_rad[HIRA_MAX_LEVELS];
     const int tree = blockIdx.x;
     const int t = threadIdx.x;
     const int D = p.dim, Dv = p.vdim, L = p.num_levels, bf = p.bf;
@@ -232,32 +218,41 @@ __global__ __launch_bounds__(kUpdThreads) void k_update(const UpdateParams p) {
                 if (L == 1 && slot + 1 > st[0]) st[0] = (int)(slot + 1);
             }
         }
-        // ---- radii: the leaf parent covers the key, every ancestor covers its child -----
+        // ---- radii: the leaf parent covers the key, every ancestor covers its child.  The
+        // distances of all levels are taken at once (a wave per level), then one thread walks
+        // the chain R_l = max(R_l, d_l + R_{l-1}). ---------------------------------------------
         if (L >= 2) {
-            size_t child = (size_t)node1;
-            const size_t b1 = (size_t)tree * p.cap[1];
-            float r_child = p.radii[1][b1 + child];
-            {
-                const float dk = block_dist<T>(x, p.centers[1], b1 * D, p.layout, D, child, red_f);
-                const float rn = fmaxf(r_child, pad_up(dk));
-                if (t == 0) p.radii[1][b1 + child] = rn;
-                r_child = rn;
-            }
-            for (int l = 2; l < L; ++l) {
-                const size_t anc = child / bf;
+            const int lane = t & 63;
+            for (int l = 1 + (t >> 6); l < L; l += kUpdThreads / 64) {  // uniform in the wave
+                size_t child = (size_t)node1;  // node of level l - 1 on the key's path (l >= 2)
+                for (int i = 2; i < l; ++i) child /= (size_t)bf;
+                const size_t node = l == 1 ? (size_t)node1 : child / (size_t)bf;
                 const size_t bl = (size_t)tree * p.cap[l], bc = (size_t)tree * p.cap[l - 1];
-                // cbuf := centre of the child
-                __syncthreads();
-                for (int j = t; j < D; j += kUpdThreads)
-                    cbuf[j] = load_elem<T>(p.centers[l - 1], bc * D + elem_index(p.layout, D, child, j));
-                __syncthreads();
-                const float dc = block_dist<T>(cbuf, p.centers[l], bl * D, p.layout, D, anc, red_f);
-                const float ra = p.radii[l][bl + anc];
-                const float rn = fmaxf(ra, pad_up(dc + r_child));
-                __syncthreads();
-                if (t == 0) p.radii[l][bl + anc] = rn;
-                r_child = rn;
-                child = anc;
+                float ss = 0.0f;
+                for (int j = lane; j < D; j += 64) {
+                    const float a =
+                        l == 1 ? x[j]
+                               : load_elem<T>(p.centers[l - 1], bc * D + elem_index(p.layout, D, child, j));
+                    const float b = load_elem<T>(p.centers[l], bl * D + elem_index(p.layout, D, node, j));
+                    ss += (a - b) * (a - b);
+                }
+#pragma unroll
+                for (int off = 1; off < 64; off <<= 1) ss += __shfl_xor(ss, off, 64);
+                if (lane == 0) {
+                    s_dist[l] = sqrtf(ss);
+                    s_rad[l] = p.radii[l][bl + node];
+                }
+            }
+            __syncthreads();
+            if (t == 0) {
+                size_t node = (size_t)node1;
+                float r_child = 0.0f;
+                for (int l = 1; l < L; ++l) {
+                    const float rn = fmaxf(s_rad[l], pad_up(s_dist[l] + r_child));
+                    if (rn != s_rad[l]) p.radii[l][(size_t)tree * p.cap[l] + node] = rn;
+                    r_child = rn;
+                    node /= (size_t)bf;
+                }
             }
         }
         __syncthreads();

@@ -94,6 +94,24 @@ def make_kv(w: Workload, n: Optional[int] = None):
     return keys.to(w.dtype), values.to(w.dtype)
 
 
+def make_stream(w: Workload, steps: int):
+    """keys, values (B, H_kv, steps, D) appended one per decode step after the prefill: the
+    same distribution with a slow drift of the mean, mu_t = mu_0 + 1e-4 t g, g ~ N(0, I)
+    fixed per head."""
+    keys = torch.empty((w.batch, w.h_kv, steps, w.d), dtype=torch.float32)
+    values = torch.empty_like(keys)
+    t = torch.arange(steps, dtype=torch.float32)[:, None]
+    for b in range(w.batch):
+        for h in range(w.h_kv):
+            dist = head_dist(w, b, h)
+            g = _gen(w.cfg, b, h, salt=3)
+            drift = torch.randn(w.d, generator=g)
+            z = torch.randn((steps, w.d), generator=g)
+            keys[b, h] = _boost(dist.mu + 1e-4 * t * drift + dist.s * z, dist)
+            values[b, h] = torch.randn((steps, w.d), generator=g)
+    return keys.to(w.dtype), values.to(w.dtype)
+
+
 def make_queries(w: Workload, keys: torch.Tensor, steps: int, seed: int = 0) -> torch.Tensor:
     """(steps, B, H_q, D) fresh queries: q = k_j + 0.5 N(0, I), j uniform.  The massive
     channels are already scaled in k_j; the noise on them is scaled by 20 as well."""
