@@ -10,6 +10,8 @@ bool mfma_search_supported(const HiraTree* t, const HiraQueue* queue) {
     if (!(t->dim == 64 || t->dim == 128 || t->dim == 256)) return false;
     if (t->vdim != 0 && t->vdim != t->dim) return false;
     (void)queue;  // queued rows get a workgroup of their own
+    // the kernel addresses a tree's keys and values with 32-bit offsets
+    if ((uint64_t)t->cap[0] * (uint64_t)t->dim * 2ull >= (1ull << 32)) return false;
     return true;
 }
 

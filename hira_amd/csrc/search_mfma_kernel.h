@@ -72,7 +72,7 @@ template <int KS>
 __device__ __forceinline__ void load_tile(const TilePtr tp, uint4 (&a)[KS]) {
 #pragma unroll
     for (int s = 0; s < KS; ++s)
-        a[s] = *reinterpret_cast<const uint4*>(tp.base + (size_t)(tp.lane_off + (unsigned)(s * 1024)));
+        a[s] = *reinterpret_cast<const uint4*>(tp.base + (size_t)tp.lane_off + s * 1024);
 }
 
 template <int KS>
@@ -82,6 +82,26 @@ __device__ __forceinline__ f32x4_t tile_scores(const uint4 (&a)[KS], const bf16x
     for (int s = 0; s < KS; ++s)
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[s]), bq[s], acc, 0, 0, 0);
     return acc;
+}
+
+// Buffer addressing for the two streams of the scan and the gather (key tiles, value rows): the
+// base sits in a scalar resource descriptor, the part that differs per load in a scalar offset,
+// and every lane adds the same small offset of its own, so that no load needs vector registers
+// for its address.  (One tree's keys or values must stay under 4 GiB.)
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, size_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)(uint32_t)bytes, 0x00020000);
+}
+
+template <int KS>
+__device__ __forceinline__ void load_tile_buf(__amdgpu_buffer_rsrc_t rsrc, unsigned lane_off,
+                                              unsigned tile_off, uint4 (&a)[KS]) {
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+        a[s] = __builtin_bit_cast(
+            uint4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off + (unsigned)(s * 1024), tile_off, 0));
 }
 
 // the same with the B operand parked in LDS (chunk s of lane l at [s*64 + l]): the scan keeps
@@ -94,6 +114,14 @@ __device__ __forceinline__ f32x4_t tile_scores_lds(const uint4 (&a)[KS], const u
         acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[s]), as_bf16x8(bq_lds[s * 64 + lane]),
                                                       acc, 0, 0, 0);
     return acc;
+}
+
+// A workgroup barrier that orders LDS traffic only: global loads issued before it (the next
+// round's key tiles) stay in flight across it.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
 __device__ __forceinline__ float pick4(const f32x4_t& v, int j) {
@@ -432,19 +460,16 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         const float sc2 = sc * kLog2e;
         const size_t row0 = (size_t)tree * p.cap[0];
 
-        for (int r = 0; r < rounds; ++r) {  // uniform in the workgroup
-            const int par = r & 1;
-            // the round's list: row -> key slot and one scaled score per head (-inf: not selected);
-            // every wave fills its own stretch of ROWS * NB rows
-            uint32_t* lst_row = s_words + (DB ? par * S::SCAN_WORDS : 0);  // (LIST) listed row -> table row
-            uint32_t* lst_tslot = lst_row + S::LIST;                       // (LIST/16) table tile -> key slot
-            float* lst_z = reinterpret_cast<float*>(lst_tslot + S::LIST / 16);  // (LIST, GS) the table
-            if (!DB && want_attn && r > 0) __syncthreads();  // the previous list has been gathered
-
-            // ---- scan: key tiles of up to NB nodes in flight -----------------------------------
-            int node[NB], cnt[NB];
-            uint32_t nmask[NB];
-            uint4 a[NB][MT][KS];
+        const __amdgpu_buffer_rsrc_t krsrc = make_rsrc(
+            reinterpret_cast<const uint16_t*>(p.keys) + row0 * (size_t)D, (size_t)p.cap[0] * D * 2);
+        const __amdgpu_buffer_rsrc_t vrsrc = make_rsrc(
+            reinterpret_cast<const uint16_t*>(p.values) + row0 * (size_t)D, (size_t)p.cap[0] * D * 2);
+        // The nodes a wave takes in a round (up to NB of its share), what LDS says about them,
+        // and the loads of their key tiles.
+        int nx_node[NB], nx_cnt[NB];
+        uint32_t nx_mask[NB];
+        uint4 a[NB][MT][KS];
+        auto fetch = [&]() {
 #pragma unroll
             for (int u = 0; u < NB; ++u) {
                 int n = -1;
@@ -455,16 +480,37 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                     n = 64 + __ffsll((long long)my1) - 1;
                     my1 &= my1 - 1ull;
                 }
-                node[u] = n;
-                cnt[u] = __builtin_amdgcn_readfirstlane(n >= 0 ? s_ncnt[n] : 0);
-                nmask[u] = (uint32_t)__builtin_amdgcn_readfirstlane((int)(n >= 0 ? s_nmask[n] : 0u));
-                const size_t tile_first = ((size_t)(tile0 * 16 + max(n, 0)) * bf) / 16;
+                nx_node[u] = n;
+                nx_cnt[u] = __builtin_amdgcn_readfirstlane(n >= 0 ? s_ncnt[n] : 0);
+                nx_mask[u] = (uint32_t)__builtin_amdgcn_readfirstlane((int)(n >= 0 ? s_nmask[n] : 0u));
+                const unsigned tile_first = (unsigned)((tile0 * 16 + max(n, 0)) * bf) / 16u;
 #pragma unroll
                 for (int tt = 0; tt < MT; ++tt)
-                    if (tt * 16 < cnt[u])
-                        load_tile<KS>(tile_ptr<KS>(p.keys, row0, tile_first + tt, lane), a[u][tt]);
+                    if (tt * 16 < nx_cnt[u])
+                        load_tile_buf<KS>(krsrc, (unsigned)lane * 16u,
+                                          (tile_first + tt) * (unsigned)(KS * 1024), a[u][tt]);
             }
+        };
+        if (rounds > 0) fetch();
 
+        for (int r = 0; r < rounds; ++r) {  // uniform in the workgroup
+            const int par = r & 1;
+            // the round's list: row -> key slot and one scaled score per head (-inf: not selected);
+            // every wave fills its own stretch of ROWS * NB rows
+            uint32_t* lst_row = s_words + (DB ? par * S::SCAN_WORDS : 0);  // (LIST) listed row -> table row
+            uint32_t* lst_tslot = lst_row + S::LIST;                       // (LIST/16) table tile -> key slot
+            float* lst_z = reinterpret_cast<float*>(lst_tslot + S::LIST / 16);  // (LIST, GS) the table
+            if (!DB && want_attn && r > 0) lds_barrier();  // the previous list has been gathered
+
+            // ---- scan: the key tiles of this round's nodes were asked for a round ago -----------
+            int node[NB], cnt[NB];
+            uint32_t nmask[NB];
+#pragma unroll
+            for (int u = 0; u < NB; ++u) {
+                node[u] = nx_node[u];
+                cnt[u] = nx_cnt[u];
+                nmask[u] = nx_mask[u];
+            }
             // all the products first: the operand registers are free before the bookkeeping starts
             f32x4_t sco_all[NB][MT];
 #pragma unroll
@@ -472,6 +518,9 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
 #pragma unroll
                 for (int tt = 0; tt < MT; ++tt)  // (only read where it is written: under this condition)
                     if (tt * 16 < cnt[u]) sco_all[u][tt] = tile_scores_lds<KS>(a[u][tt], s_bq, lane);
+            // ... and taken again at once by the next round's keys, which are on their way while
+            // this round's rows are listed and gathered
+            if (r + 1 < rounds) fetch();
 
             if (r == 0) HIRA_TL(8);
             // The bookkeeping below derives everything per-lane from this copy, which the compiler
@@ -595,7 +644,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
             if (r == 0) HIRA_TL(9);
             if (lane == 0) s_cntw[par][wave] = nsel;
             if (kb == 0) s_mxw[par][wave * 16 + col] = zmax;
-            __syncthreads();
+            lds_barrier();
             int cw[kMfmaWaves];
             int tot = 0;
             float rmax = -INFINITY;
@@ -638,7 +687,6 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
             // ---- gather: list rows wave, wave + nw, ...; kVBatch value rows in flight --------------
             constexpr int RP = 64 / GS;          // rows whose weights one pass over the lanes computes
             constexpr int NPASS = kVBatch / RP;  // GS = 4: 1, GS = 8: 2, GS = 16: 4
-            const char* vtree = reinterpret_cast<const char*>(p.values) + row0 * (size_t)(D * 2);
             // where the rows of a batch sit (row `le` of the round is row `rem` of the stretch of the
             // wave it falls in; lane = (row of the pass, head)), and their value rows
             auto issue = [&](int e0, int (&at_v)[NPASS], uint32_t (&vraw)[kVBatch][VW]) {
@@ -663,14 +711,16 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 for (int i = 0; i < kVBatch; ++i) {
                     {
                         const unsigned slot = (unsigned)__builtin_amdgcn_readlane(slot_v[i / RP], (i % RP) * GS);
-                        const uint16_t* vp =
-                            reinterpret_cast<const uint16_t*>(vtree + (size_t)slot * (D * 2)) + lane_o * VPL;
+                        const unsigned voff = (unsigned)lane_o * (unsigned)(VPL * 2);
+                        const unsigned soff = slot * (unsigned)(D * 2);
                         if (VPL == 1) {
-                            vraw[i][0] = *vp;
+                            vraw[i][0] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(vrsrc, voff, soff, 0);
+                        } else if (VPL == 2) {
+                            vraw[i][0] = __builtin_amdgcn_raw_buffer_load_b32(vrsrc, voff, soff, 0);
                         } else {
-#pragma unroll
-                            for (int e = 0; e < VPL / 2; ++e)
-                                vraw[i][e] = reinterpret_cast<const uint32_t*>(vp)[e];
+                            const u32x2_t v2 = __builtin_amdgcn_raw_buffer_load_b64(vrsrc, voff, soff, 0);
+                            vraw[i][0] = v2.x;
+                            vraw[i][VW - 1] = v2.y;
                         }
                     }
                 }
