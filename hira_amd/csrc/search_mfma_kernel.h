@@ -1,12 +1,12 @@
 // MFMA search + sparse attention kernel: bf16 keys/centers in the tiled layout
 // (HIRA_TILE16), fan-out a multiple of 16, D = Dv in {64, 128, 256}, at least two levels.
 //
-// One workgroup (8 waves; 256 registers a wave, so the only one on its CU) owns a run of
-// consecutive tiles of 16 level-1 nodes of one tree; workgroup ids run fastest over the trees
+// One workgroup (8 waves; 256 registers a wave, so the only one on its CU) owns a few
+// tiles of 16 level-1 nodes of one tree, a stride apart; workgroup ids run fastest over the trees
 // so that, with 8 L2 slices (XCDs) served round-robin, the workgroups of one tree share a
 // slice.  The work is split by phase, not by node, so that neither the key scan nor the
 // value gather depends on where in the tree the selected keys sit:
-//   gate   wave w gates tile w of the run: it issues, before it waits for anything, every
+//   gate   wave w gates the workgroup's tile w: it issues, before it waits for anything, every
 //          load it needs (queries, the 16 x D tile of level-1 centres, the tiles holding the
 //          tile's ancestors, radii, child counts) and gates with v_mfma_f32_16x16x32_bf16:
 //          a wave-wide 128-bit load fetches a 16 x 32 operand tile from 1 KiB of contiguous
@@ -14,7 +14,7 @@
 //          query heads of the GQA group, so the D registers hold score(row, head) with
 //          head = lane % 16 and row = 4*(lane/16) + j; a node survives for a head when
 //          score + ||q|| r >= tau.  Head masks and child counts of the nodes go to LDS.
-//   scan   the surviving nodes of the run are dealt round-robin to the waves; in each round
+//   scan   the surviving nodes of these tiles are dealt round-robin to the waves; in each round
 //          a wave loads the key tiles of NB nodes at once (the B operand now comes from
 //          LDS), scores them the same way (leaf filter: q.k >= tau against the lane's own
 //          threshold) and, for a tile with a selected row, writes the scaled scores of its
@@ -224,8 +224,16 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     const int tree = blockIdx.x;
     const int L = p.num_levels, bf = p.bf;
     const bool want_attn = p.part_acc != nullptr;
-    const int tile0 = (int)blockIdx.y * p.nodes_per_wave;  // first tile of my run
-    const int ntile = min(p.nodes_per_wave, ((p.size[1] + 15) >> 4) - tile0);
+    // my tiles: blockIdx.y, blockIdx.y + (tree workgroups), ...  Neighbouring tiles hold
+    // sibling nodes, which tend to survive (and be selected from) together: striding deals
+    // the busy stretches of the tree out over the workgroups.
+    const int wg_tiles = (p.size[1] + 15) >> 4, wg_stride = p.tree_blocks;
+    const int ntile = (int)blockIdx.y < wg_stride
+                          ? min(p.nodes_per_wave, (wg_tiles - (int)blockIdx.y + wg_stride - 1) / wg_stride)
+                          : 0;
+    auto tile_of = [&](int tl) { return (int)blockIdx.y + tl * wg_stride; };
+    // level-1 node behind entry n (tile n / 16 of mine, node n % 16 of the tile)
+    auto node_of = [&](int n) { return tile_of(n >> 4) * 16 + (n & 15); };
     const bool is_queue = (int)blockIdx.y >= p.tree_blocks;  // the workgroup after the tree's
 #ifdef HIRA_TIMELINE  // experiment builds only: p.stats receives 8 time stamps per workgroup
     unsigned long long* stats = nullptr;
@@ -337,7 +345,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     } else {
         // ---- queries and the first tile's gate operands, issued before the first wait --------
         // (only the waves that gate need the queries in registers: the scan reads them from LDS)
-        int tl_mine = wave;  // tile of the run this wave gates next
+        int tl_mine = wave;  // of my tiles, the one this wave gates next
         uint4 qraw[KS];
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
@@ -349,7 +357,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         const float tau = head_ok ? p.tau[qh] : INFINITY;
         const float sc = head_ok ? p.scaling[qh] : 0.0f;
         GateLoads<KS> gl;
-        if (tl_mine < ntile) gate_issue<KS>(p, tree, tile0 + tl_mine, lane, kb, gl);
+        if (tl_mine < ntile) gate_issue<KS>(p, tree, tile_of(tl_mine), lane, kb, gl);
 
         // ---- B operand and ||q|| -----------------------------------------------------------
         bf16x8_t bq[KS];
@@ -372,7 +380,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
 
         // ---- gate: one tile per wave at a time ------------------------------------------------
         while (tl_mine < ntile) {  // uniform in the wave
-            const int t1 = tile0 + tl_mine;
+            const int t1 = tile_of(tl_mine);
             const bool count_nodes = stats != nullptr && lane == 0;
             size_t span = 1;  // level-1 nodes under one node of the current level
             for (int l = 2; l < L; ++l) span *= (size_t)bf;
@@ -434,14 +442,14 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 for (int j = 0; j < 4; ++j) s_ncnt[tl_mine * 16 + 4 * kb + j] = cc[j];
             }
             tl_mine += nw;
-            if (tl_mine < ntile) gate_issue<KS>(p, tree, tile0 + tl_mine, lane, kb, gl);
+            if (tl_mine < ntile) gate_issue<KS>(p, tree, tile_of(tl_mine), lane, kb, gl);
         }
         HIRA_TL(7);
         __syncthreads();
         HIRA_TL(1);
 
-        // ---- the surviving nodes of the run, dealt round-robin to the waves ----------------------
-        unsigned long long my0, my1;  // bit n: node n (n + 64) of the run survives and is mine
+        // ---- the surviving nodes of my tiles, dealt round-robin to the waves ----------------------
+        unsigned long long my0, my1;  // bit n: node n (n + 64) of my tiles survives and is mine
         int rounds;
         {
             const int NT = ntile * 16;
@@ -483,7 +491,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 nx_node[u] = n;
                 nx_cnt[u] = __builtin_amdgcn_readfirstlane(n >= 0 ? s_ncnt[n] : 0);
                 nx_mask[u] = (uint32_t)__builtin_amdgcn_readfirstlane((int)(n >= 0 ? s_nmask[n] : 0u));
-                const unsigned tile_first = (unsigned)((tile0 * 16 + max(n, 0)) * bf) / 16u;
+                const unsigned tile_first = (unsigned)(node_of(max(n, 0)) * bf) / 16u;
 #pragma unroll
                 for (int tt = 0; tt < MT; ++tt)
                     if (tt * 16 < nx_cnt[u])
@@ -537,7 +545,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
             for (int u = 0; u < NB; ++u) {
                 // a head for which the node did not survive selects nothing
                 const float tau_u = ((nmask[u] >> col) & 1u) ? tau : INFINITY;
-                const unsigned slot0 = (unsigned)((tile0 * 16 + max(node[u], 0)) * bf);
+                const unsigned slot0 = (unsigned)(node_of(max(node[u], 0)) * bf);
                 if (stats && lane == 0) stat_add(stats, 0, (unsigned)cnt[u]);
 #pragma unroll
                 for (int tt = 0; tt < MT; ++tt) {
