@@ -68,7 +68,7 @@ struct SearchPlan {
 // search_mfma.hip
 bool mfma_search_supported(const HiraTree* t, const HiraQueue* queue);
 constexpr int kMfmaThreads = 512;       // workgroup size of the MFMA kernel (8 waves), at most
-constexpr int kMfmaMaxTilesPerWg = 8;  // tiles of 16 level-1 nodes one workgroup walks
+constexpr int kMfmaMaxTilesPerWg = 16;  // tiles of 16 level-1 nodes one workgroup walks, at most
 int launch_search_mfma(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
 
 // Element index of (row, column j) inside one tree's (cap, D) matrix.

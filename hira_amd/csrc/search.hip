@@ -469,7 +469,7 @@ static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* que
         HIRA_CHECK_ARG(threads >= 64 && threads <= kMfmaThreads && threads % 64 == 0,
                        "block_threads %d must be a multiple of 64 up to %d", threads, kMfmaThreads);
         plan->threads = threads;
-        // a workgroup walks `tpw` consecutive tiles of 16 level-1 nodes: as few as keep
+        // a workgroup walks `tpw` tiles of 16 level-1 nodes (a stride apart): as few as keep
         // one workgroup per CU in the launch (the kernel runs one at a time on a CU) and at
         // most 64 partials per head to fold
         const int tiles = (t->size[1] + 15) / 16;
@@ -477,11 +477,13 @@ static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* que
         HIRA_CHECK_ARG(tpw >= 0 && tpw <= kMfmaMaxTilesPerWg,
                        "MFMA kernel: %d tiles per workgroup (at most %d)", tpw, kMfmaMaxTilesPerWg);
         if (tpw == 0) {
-            tpw = 1;
-            while (tpw < kMfmaMaxTilesPerWg &&
-                   ((int64_t)tiles * t->num_trees * plan->head_chunks > compute_units() * (int64_t)tpw ||
-                    tiles > 64 * tpw))
-                tpw *= 2;
+            const int64_t all = (int64_t)tiles * t->num_trees * plan->head_chunks;
+            const int cus = compute_units();
+            tpw = (int)((all + cus - 1) / cus);
+            if (tpw * 64 < tiles) tpw = (tiles + 63) / 64;
+            if (tpw < 1) tpw = 1;
+            // more work than one workgroup per CU can take: several rounds of smaller ones
+            if (tpw > kMfmaMaxTilesPerWg) tpw = kMfmaMaxTilesPerWg / 2;
         }
         plan->nodes_per_wave = tpw;
         plan->num_nodes = t->size[1];

@@ -449,19 +449,22 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         HIRA_TL(1);
 
         // ---- the surviving nodes of my tiles, dealt round-robin to the waves ----------------------
-        unsigned long long my0, my1;  // bit n: node n (n + 64) of my tiles survives and is mine
+        constexpr int NW64 = kMfmaMaxTilesPerWg * 16 / 64;  // 64-bit words of a node set
+        unsigned long long mine[NW64];  // bit n of word i: node 64 i + n of my tiles survives and is mine
         int rounds;
         {
             const int NT = ntile * 16;
-            const bool a0 = lane < NT && s_nmask[lane] != 0u;
-            const bool a1 = lane + 64 < NT && s_nmask[lane + 64] != 0u;
-            const unsigned long long A0 = __ballot(a0), A1 = __ballot(a1);
             const unsigned long long lt = (1ull << lane) - 1ull;
-            const int r0 = __popcll(A0 & lt), r1 = __popcll(A0) + __popcll(A1 & lt);
-            my0 = __ballot(a0 && (r0 % nw) == wave);
-            my1 = __ballot(a1 && (r1 % nw) == wave);
-            const int alive = __popcll(A0) + __popcll(A1);
-            rounds = ((alive + nw - 1) / nw + NB - 1) / NB;
+            int before = 0;  // survivors in the words before
+#pragma unroll
+            for (int i = 0; i < NW64; ++i) {
+                const bool alive = 64 * i + lane < NT && s_nmask[64 * i + lane] != 0u;
+                const unsigned long long all = __ballot(alive);
+                const int rank = before + __popcll(all & lt);
+                mine[i] = __ballot(alive && (rank % nw) == wave);
+                before += __popcll(all);
+            }
+            rounds = ((before + nw - 1) / nw + NB - 1) / NB;
         }
 
         constexpr bool DB = S::LIST_WORDS == 2 * S::SCAN_WORDS;  // room for a second list: one barrier a round
@@ -480,13 +483,13 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         auto fetch = [&]() {
 #pragma unroll
             for (int u = 0; u < NB; ++u) {
-                int n = -1;
-                if (my0 != 0ull) {
-                    n = __ffsll((long long)my0) - 1;
-                    my0 &= my0 - 1ull;
-                } else if (my1 != 0ull) {
-                    n = 64 + __ffsll((long long)my1) - 1;
-                    my1 &= my1 - 1ull;
+                int n = -1;  // my next node: the lowest bit of the first word that has one
+#pragma unroll
+                for (int i = 0; i < NW64; ++i) {
+                    if (n < 0 && mine[i] != 0ull) {
+                        n = 64 * i + __ffsll((long long)mine[i]) - 1;
+                        mine[i] &= mine[i] - 1ull;
+                    }
                 }
                 nx_node[u] = n;
                 nx_cnt[u] = __builtin_amdgcn_readfirstlane(n >= 0 ? s_ncnt[n] : 0);
