@@ -205,8 +205,11 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     constexpr int VPL = KS / 2;        // value elements per lane: Dv = D = 64 * VPL
     constexpr int VW = (VPL + 1) / 2;  // dwords of a value row per lane
     __shared__ uint32_t s_words[S::WORDS];  // the round's list; the merge; the fold
-    __shared__ uint32_t s_nmask[kMfmaMaxTilesPerWg * 16];  // heads for which a node survives
-    __shared__ int32_t s_ncnt[kMfmaMaxTilesPerWg * 16];    // its child count
+    // a node of my tiles: heads for which it survives (16 bits) | child count << 16
+    __shared__ uint32_t s_ninfo[kMfmaMaxTilesPerWg * 16];
+    // the surviving ones in order, a copy per wave (each wave makes its own: no barrier):
+    // node | child count << 8 | heads << 16
+    __shared__ uint32_t s_order[kMfmaWaves][kMfmaMaxTilesPerWg * 16];
     __shared__ int32_t s_cntw[2][kMfmaWaves];          // rows a wave selected (by round parity)
     __shared__ float s_mxw[2][kMfmaWaves * 16];        // its best selected score per head
     __shared__ float s_lw[kMfmaWaves * 16];
@@ -432,14 +435,18 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
 #pragma unroll
             for (int j = 0; j < 4; ++j) nb[j] = __ballot((alive4 >> j) & 1u);
             // node n = 4*kb' + j of the tile: its heads are field kb' of nb[j]
+            // (its child count sits in lane 16*kb', element j, of cc)
+            int cnt_n = 0;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int c = __shfl(cc[j], 16 * ((lane >> 2) & 3), 64);
+                if ((lane & 3) == j) cnt_n = c;
+            }
             if (lane < 16) {
                 const int jn = lane & 3;
                 const unsigned long long bits = jn == 0 ? nb[0] : (jn == 1 ? nb[1] : (jn == 2 ? nb[2] : nb[3]));
-                s_nmask[tl_mine * 16 + lane] = (uint32_t)((bits >> (16 * (lane >> 2))) & 0xFFFFull);
-            }
-            if (col == 0) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) s_ncnt[tl_mine * 16 + 4 * kb + j] = cc[j];
+                s_ninfo[tl_mine * 16 + lane] =
+                    (uint32_t)((bits >> (16 * (lane >> 2))) & 0xFFFFull) | ((uint32_t)cnt_n << 16);
             }
             tl_mine += nw;
             if (tl_mine < ntile) gate_issue<KS>(p, tree, tile_of(tl_mine), lane, kb, gl);
@@ -449,22 +456,22 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         HIRA_TL(1);
 
         // ---- the surviving nodes of my tiles, dealt round-robin to the waves ----------------------
-        constexpr int NW64 = kMfmaMaxTilesPerWg * 16 / 64;  // 64-bit words of a node set
-        unsigned long long mine[NW64];  // bit n of word i: node 64 i + n of my tiles survives and is mine
-        int rounds;
+        int rounds, alive = 0;
         {
             const int NT = ntile * 16;
             const unsigned long long lt = (1ull << lane) - 1ull;
-            int before = 0;  // survivors in the words before
 #pragma unroll
-            for (int i = 0; i < NW64; ++i) {
-                const bool alive = 64 * i + lane < NT && s_nmask[64 * i + lane] != 0u;
-                const unsigned long long all = __ballot(alive);
-                const int rank = before + __popcll(all & lt);
-                mine[i] = __ballot(alive && (rank % nw) == wave);
-                before += __popcll(all);
+            for (int i = 0; i < kMfmaMaxTilesPerWg * 16 / 64; ++i) {
+                if (64 * i >= NT) break;  // uniform
+                const uint32_t info = 64 * i + lane < NT ? s_ninfo[64 * i + lane] : 0u;
+                const bool live = (info & 0xFFFFu) != 0u;
+                const unsigned long long all = __ballot(live);
+                if (live)
+                    s_order[wave][alive + __popcll(all & lt)] =
+                        (uint32_t)(64 * i + lane) | ((info >> 16) << 8) | (info << 16);
+                alive += __popcll(all);
             }
-            rounds = ((before + nw - 1) / nw + NB - 1) / NB;
+            rounds = ((alive + nw - 1) / nw + NB - 1) / NB;
         }
 
         constexpr bool DB = S::LIST_WORDS == 2 * S::SCAN_WORDS;  // room for a second list: one barrier a round
@@ -480,20 +487,21 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         int nx_node[NB], nx_cnt[NB];
         uint32_t nx_mask[NB];
         uint4 a[NB][MT][KS];
-        auto fetch = [&]() {
+        auto fetch = [&](int round) {
+            // my nodes of the round: entries (round*NB + u) * nw + wave of the survivors
+            uint32_t ent[NB];
 #pragma unroll
             for (int u = 0; u < NB; ++u) {
-                int n = -1;  // my next node: the lowest bit of the first word that has one
+                const int k = (round * NB + u) * nw + wave;
+                ent[u] = k < alive ? s_order[wave][k] : 0xFFu;
+            }
 #pragma unroll
-                for (int i = 0; i < NW64; ++i) {
-                    if (n < 0 && mine[i] != 0ull) {
-                        n = 64 * i + __ffsll((long long)mine[i]) - 1;
-                        mine[i] &= mine[i] - 1ull;
-                    }
-                }
+            for (int u = 0; u < NB; ++u) {
+                const uint32_t e = (uint32_t)__builtin_amdgcn_readfirstlane((int)ent[u]);
+                const int n = (e >> 16) != 0u ? (int)(e & 0xFFu) : -1;
                 nx_node[u] = n;
-                nx_cnt[u] = __builtin_amdgcn_readfirstlane(n >= 0 ? s_ncnt[n] : 0);
-                nx_mask[u] = (uint32_t)__builtin_amdgcn_readfirstlane((int)(n >= 0 ? s_nmask[n] : 0u));
+                nx_cnt[u] = (int)((e >> 8) & 0xFFu);
+                nx_mask[u] = e >> 16;
                 const unsigned tile_first = (unsigned)(node_of(max(n, 0)) * bf) / 16u;
 #pragma unroll
                 for (int tt = 0; tt < MT; ++tt)
@@ -502,7 +510,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                                           (tile_first + tt) * (unsigned)(KS * 1024), a[u][tt]);
             }
         };
-        if (rounds > 0) fetch();
+        if (rounds > 0) fetch(0);
 
         for (int r = 0; r < rounds; ++r) {  // uniform in the workgroup
             const int par = r & 1;
@@ -531,7 +539,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                     if (tt * 16 < cnt[u]) sco_all[u][tt] = tile_scores_lds<KS>(a[u][tt], s_bq, lane);
             // ... and taken again at once by the next round's keys, which are on their way while
             // this round's rows are listed and gathered
-            if (r + 1 < rounds) fetch();
+            if (r + 1 < rounds) fetch(r + 1);
 
             if (r == 0) HIRA_TL(8);
             // The bookkeeping below derives everything per-lane from this copy, which the compiler
