@@ -125,8 +125,11 @@ typedef struct HiraSearchOut {
 } HiraSearchOut;
 
 typedef struct HiraLaunch {
-    int32_t block_threads;  /* 64, 128 or 256; 0 = default */
-    int32_t nodes_per_wave; /* level-1 nodes one wavefront walks; 0 = default */
+    int32_t block_threads;  /* vector-ALU kernel: 64, 128 or 256; MFMA kernel: a multiple of 64
+                               up to 512; 0 = default */
+    int32_t nodes_per_wave; /* vector-ALU kernel: level-1 nodes one wavefront walks; MFMA kernel:
+                               tiles of 16 level-1 nodes one workgroup walks (at most 16);
+                               0 = chosen from the tree and the device */
     int32_t kernel;         /* 0 = auto, 1 = vector-ALU kernel, 2 = MFMA kernel (bf16) */
     int32_t separate_merge; /* != 0: fold the attention partials in a second launch even
                                where the search kernel could do it itself */
