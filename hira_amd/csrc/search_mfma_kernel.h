@@ -14,18 +14,21 @@
 //          query heads of the GQA group, so the D registers hold score(row, head) with
 //          head = lane % 16 and row = 4*(lane/16) + j; a node survives for a head when
 //          score + ||q|| r >= tau.  Head masks and child counts of the nodes go to LDS.
-//   scan   the surviving nodes of these tiles are dealt round-robin to the waves; in each round
-//          a wave loads the key tiles of NB nodes at once (the B operand now comes from
-//          LDS), scores them the same way (leaf filter: q.k >= tau against the lane's own
-//          threshold) and, for a tile with a selected row, writes the scaled scores of its
-//          rows to a table in LDS (-inf: not selected) and appends the selected rows to its
-//          stretch of the round's row list.  The waves agree on one running maximum per head,
-//          so their sums need no rescaling when they are added up.
-//   gather the rows of the list are dealt round-robin to the waves: kVBatch value rows in
-//          flight per wave, each row fetched once however many heads selected it; scores
-//          become weights 2^(z - m) with lane = (row, head), then
+//   scan   the surviving nodes of these tiles are dealt round-robin to the waves; from here to
+//          the merge a wave works on its own (no barrier).  In each round it takes NB of its
+//          nodes: their key tiles were requested a round earlier (buffer loads: scalar base and
+//          tile offset, no address registers), the B operand now comes from LDS; all products
+//          first, then the next round's tiles are requested, then the leaf filter (q.k >= tau
+//          against the lane's own threshold).  A tile with a selected row writes the scaled
+//          scores of its rows to the wave's stretch of a table in LDS (-inf: not selected) and
+//          appends the selected rows to the wave's row list.
+//   gather the wave raises its running maximum per head, turns the listed scores into weights
+//          2^(z - m) with lane = (row, head), and fetches the value rows of its list, kVBatch
+//          in flight, each row once however many heads selected it:
 //          acc[head][:] += weight(row, head) * v[:] with the accumulators in registers
 //          (lane owns Dv/64 columns of every head).
+//   merge  the waves agree on one maximum per head, rescale their sums to it and add them up
+//          through LDS.
 // Keys queued since the tree was last updated (row-major, attended by every head) get one
 // more workgroup per tree.  One partial (m, l, acc) per head and workgroup goes to global
 // memory; the last workgroup of a tree to arrive folds the tree's partials.
@@ -116,14 +119,6 @@ __device__ __forceinline__ f32x4_t tile_scores_lds(const uint4 (&a)[KS], const u
     return acc;
 }
 
-// A workgroup barrier that orders LDS traffic only: global loads issued before it (the next
-// round's key tiles) stay in flight across it.
-__device__ __forceinline__ void lds_barrier() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
 __device__ __forceinline__ float pick4(const f32x4_t& v, int j) {
     return j == 0 ? v[0] : (j == 1 ? v[1] : (j == 2 ? v[2] : v[3]));
 }
@@ -153,9 +148,7 @@ struct MfmaShape {
     static constexpr int LIST = kMfmaWaves * NB * ROWS;  // rows of the list of one round
     static constexpr int SCAN_WORDS = LIST * (GS + 1) + LIST / 16;  // row list, tile slots, GS scores per row
     static constexpr int MERGE_WORDS = kMfmaWaves * 4 * D;  // four heads of every wave
-    // two lists (rounds alternate, one barrier a round) where that stays under 40 KiB
-    static constexpr int LIST_WORDS = 2 * SCAN_WORDS * 4 <= 40 * 1024 ? 2 * SCAN_WORDS : SCAN_WORDS;
-    static constexpr int WORDS = LIST_WORDS > MERGE_WORDS ? LIST_WORDS : MERGE_WORDS;
+    static constexpr int WORDS = SCAN_WORDS > MERGE_WORDS ? SCAN_WORDS : MERGE_WORDS;
 };
 
 // What a wave needs to gate one tile of 16 level-1 nodes, as it comes from memory.
@@ -210,8 +203,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     // the surviving ones in order, a copy per wave (each wave makes its own: no barrier):
     // node | child count << 8 | heads << 16
     __shared__ uint32_t s_order[kMfmaWaves][kMfmaMaxTilesPerWg * 16];
-    __shared__ int32_t s_cntw[2][kMfmaWaves];          // rows a wave selected (by round parity)
-    __shared__ float s_mxw[2][kMfmaWaves * 16];        // its best selected score per head
+    __shared__ float s_mxw[kMfmaWaves * 16];           // a wave's running maximum per head
     __shared__ float s_lw[kMfmaWaves * 16];
     __shared__ float s_mh[kHeadsPerPass];
     __shared__ float s_red[2 * kHeadsPerPass];
@@ -330,20 +322,11 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 }
             }
         }
-        // one maximum per head for the whole workgroup, as the merge below expects
-#pragma unroll
-        for (int g = 0; g < GS; ++g)
-            if (lane == g) s_mxw[0][wave * 16 + g] = mq[g];
-        __syncthreads();
+        // hand the wave's state over in the form the merge below expects
 #pragma unroll
         for (int g = 0; g < GS; ++g) {
-            float mall = -INFINITY;
-            for (int w = 0; w < nw; ++w) mall = fmaxf(mall, s_mxw[0][w * 16 + g]);
-            const float f = mq[g] == -INFINITY ? 0.0f : exp2f(mq[g] - mall);
-#pragma unroll
-            for (int e = 0; e < VPL; ++e) acc[g][e] *= f;
-            if (lane == g) l_mine = lq[g] * f;
-            if (col == g) m_run = mall;
+            if (lane == g) l_mine = lq[g];
+            if (col == g) m_run = mq[g];
         }
     } else {
         // ---- queries and the first tile's gate operands, issued before the first wait --------
@@ -474,7 +457,6 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
             rounds = ((alive + nw - 1) / nw + NB - 1) / NB;
         }
 
-        constexpr bool DB = S::LIST_WORDS == 2 * S::SCAN_WORDS;  // room for a second list: one barrier a round
         const float sc2 = sc * kLog2e;
         const size_t row0 = (size_t)tree * p.cap[0];
 
@@ -513,13 +495,11 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         if (rounds > 0) fetch(0);
 
         for (int r = 0; r < rounds; ++r) {  // uniform in the workgroup
-            const int par = r & 1;
-            // the round's list: row -> key slot and one scaled score per head (-inf: not selected);
-            // every wave fills its own stretch of ROWS * NB rows
-            uint32_t* lst_row = s_words + (DB ? par * S::SCAN_WORDS : 0);  // (LIST) listed row -> table row
-            uint32_t* lst_tslot = lst_row + S::LIST;                       // (LIST/16) table tile -> key slot
+            // the round's score table and row list; every wave has a stretch of ROWS * NB rows of
+            // its own and nobody else looks at it: no barrier inside the rounds
+            uint32_t* lst_row = s_words;                                        // (LIST) listed row -> table row
+            uint32_t* lst_tslot = lst_row + S::LIST;                            // (LIST/16) table tile -> key slot
             float* lst_z = reinterpret_cast<float*>(lst_tslot + S::LIST / 16);  // (LIST, GS) the table
-            if (!DB && want_attn && r > 0) lds_barrier();  // the previous list has been gathered
 
             // ---- scan: the key tiles of this round's nodes were asked for a round ago -----------
             int node[NB], cnt[NB];
@@ -657,34 +637,16 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
             }
             if (!want_attn) continue;  // uniform in the launch
 
-            // ---- every wave learns all counts and the best scores of the round ---------------------
+            // ---- the best selected score of every head in my rows of this round --------------------
             zmax = fmaxf(zmax, __shfl_xor(zmax, 16, 64));
             zmax = fmaxf(zmax, __shfl_xor(zmax, 32, 64));
-            if (r == 0) HIRA_TL(9);
-            if (lane == 0) s_cntw[par][wave] = nsel;
-            if (kb == 0) s_mxw[par][wave * 16 + col] = zmax;
-            lds_barrier();
-            int cw[kMfmaWaves];
-            int tot = 0;
-            float rmax = -INFINITY;
-            {
-                // one read each, then lane by lane: no wait between the waves' entries
-                const int cv = s_cntw[par][lane_o & (kMfmaWaves - 1)];
-                float mv[kMfmaWaves];
-#pragma unroll
-                for (int w = 0; w < kMfmaWaves; ++w) mv[w] = s_mxw[par][w * 16 + col];
-#pragma unroll
-                for (int w = 0; w < kMfmaWaves; ++w) {
-                    cw[w] = w < nw ? __builtin_amdgcn_readlane(cv, w) : 0;
-                    tot += cw[w];
-                    if (w < nw) rmax = fmaxf(rmax, mv[w]);
-                }
-            }
+            const float rmax = zmax;
+            const int tot = nsel;
 #ifdef HIRA_TIMELINE
-            if (r == 0) HIRA_TL(10);
+            if (r == 0) HIRA_TL(9);
             if (threadIdx.x == 0 && r == 0) { tl[6] = (unsigned long long)tot; tl[12] = (unsigned long long)rounds; }
 #endif
-            if (tot == 0) continue;  // uniform in the workgroup: nothing selected in this round
+            if (tot == 0) continue;  // uniform in the wave: nothing selected in my rows
 
             // the new maximum of every head, and what it does to the sums so far; head g lives in
             // lane g; the weights below are computed with lane = (row, head), head = lane % GS
@@ -703,23 +665,16 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 }
             }
 
-            // ---- gather: list rows wave, wave + nw, ...; kVBatch value rows in flight --------------
+            // ---- gather my listed rows: kVBatch value rows in flight -------------------------------
             constexpr int RP = 64 / GS;          // rows whose weights one pass over the lanes computes
-            constexpr int NPASS = kVBatch / RP;  // GS = 4: 1, GS = 8: 2, GS = 16: 4
-            // where the rows of a batch sit (row `le` of the round is row `rem` of the stretch of the
-            // wave it falls in; lane = (row of the pass, head)), and their value rows
+            constexpr int NPASS = kVBatch / RP;  // GS = 4: 2, GS = 8: 4, GS = 16: 8
+            // the rows of a batch in the score table (lane = (row of the pass, head)), their key
+            // slots, and the loads of their value rows
             auto issue = [&](int e0, int (&at_v)[NPASS], uint32_t (&vraw)[kVBatch][VW]) {
 #pragma unroll
                 for (int ps = 0; ps < NPASS; ++ps) {
-                    const int le = e0 + (ps * RP + lane_o / GS) * nw;
-                    int rem = le, at = -1;
-#pragma unroll
-                    for (int w = 0; w < kMfmaWaves; ++w) {
-                        if (at < 0 && rem < cw[w]) at = w * (NB * S::ROWS) + rem;
-                        rem -= cw[w];
-                    }
-                    // -> its row in the score table (-1: past the end)
-                    at_v[ps] = (le < tot && at >= 0) ? (int)lst_row[at] : -1;
+                    const int le = e0 + ps * RP + lane_o / GS;
+                    at_v[ps] = le < tot ? (int)lst_row[zrow0 + le] : -1;  // (-1: past the end)
                 }
                 int slot_v[NPASS];  // the key slots of all the rows of a pass
 #pragma unroll
@@ -759,7 +714,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 }
 #pragma unroll
                 for (int i = 0; i < kVBatch; ++i) {
-                    if (e0 + i * nw >= tot) break;  // uniform
+                    if (e0 + i >= tot) break;  // uniform
                     const int at = __builtin_amdgcn_readlane(at_v[i / RP], (i % RP) * GS);
                     float vf[VPL];
                     if (VPL == 1) {
@@ -780,7 +735,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                     }
                 }
             };
-            for (int e0 = wave; e0 < tot; e0 += nw * kVBatch) {  // uniform in the wave
+            for (int e0 = 0; e0 < tot; e0 += kVBatch) {  // uniform in the wave
                 int at_v[NPASS];
                 uint32_t vraw[kVBatch][VW];
                 issue(e0, at_v, vraw);
@@ -792,7 +747,23 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     if (!want_attn) return;  // uniform
     HIRA_TL(2);
 
-    // ---- merge the waves: same m everywhere, so l and acc simply add up ------------------------
+    // ---- merge the waves: first one maximum per head for the workgroup, to which every wave
+    // brings its sums (m_run: lane = head col; l_mine: head lane % GS); then l and acc add up ---
+    if (kb == 0) s_mxw[wave * 16 + col] = m_run;
+    __syncthreads();
+    {
+        float m_all = -INFINITY;
+        for (int w = 0; w < nw; ++w) m_all = fmaxf(m_all, s_mxw[w * 16 + col]);
+        const float fw = m_run == -INFINITY ? 0.0f : exp2f(m_run - m_all);
+        l_mine *= __shfl(fw, lane & (GS - 1), 64);
+#pragma unroll
+        for (int g = 0; g < GS; ++g) {
+            const float fg = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fw), g));
+#pragma unroll
+            for (int e = 0; e < VPL; ++e) acc[g][e] *= fg;
+        }
+        m_run = m_all;
+    }
 #pragma unroll
     for (int off = GS; off < 64; off <<= 1) l_mine += __shfl_xor(l_mine, off, 64);
     if (lane < GS) s_lw[wave * 16 + lane] = l_mine;
