@@ -304,7 +304,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 if (r0 + i * nw >= p.queue_len) break;  // uniform
 #pragma unroll
                 for (int g = 0; g < GS; ++g) {
-                    if (g >= G) break;  // uniform
+                    if (g >= G) continue;  // uniform (no break: the loop has to unroll)
                     float sdot = 0.0f;
 #pragma unroll
                     for (int e = 0; e < VPL; ++e) sdot += bf16_lo((uint32_t)kraw[i][e]) * qf[g][e];
@@ -774,8 +774,8 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     const int P = p.num_parts;
 #pragma unroll
     for (int c = 0; c < GS / 4; ++c) {
-        if (c * 4 >= G) break;  // uniform
-        __syncthreads();        // the list (or the previous four heads) is not needed any more
+        if (c * 4 >= G) continue;  // uniform (no break: the loop has to unroll)
+        __syncthreads();           // the list (or the previous four heads) is not needed any more
 #pragma unroll
         for (int gi = 0; gi < 4; ++gi)
 #pragma unroll
