@@ -469,16 +469,18 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         int nx_node[NB], nx_cnt[NB];
         uint32_t nx_mask[NB];
         uint4 a[NB][MT][KS];
-        auto fetch = [&](int round) {
+        auto fetch = [&](int round, int u_only) {  // u_only < 0: all NB nodes of the round
             // my nodes of the round: entries (round*NB + u) * nw + wave of the survivors
             uint32_t ent[NB];
 #pragma unroll
             for (int u = 0; u < NB; ++u) {
+                if (u_only >= 0 && u != u_only) continue;
                 const int k = (round * NB + u) * nw + wave;
                 ent[u] = k < alive ? s_order[wave][k] : 0xFFu;
             }
 #pragma unroll
             for (int u = 0; u < NB; ++u) {
+                if (u_only >= 0 && u != u_only) continue;
                 const uint32_t e = (uint32_t)__builtin_amdgcn_readfirstlane((int)ent[u]);
                 const int n = (e >> 16) != 0u ? (int)(e & 0xFFu) : -1;
                 nx_node[u] = n;
@@ -492,7 +494,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                                           (tile_first + tt) * (unsigned)(KS * 1024), a[u][tt]);
             }
         };
-        if (rounds > 0) fetch(0);
+        if (rounds > 0) fetch(0, -1);
 
         for (int r = 0; r < rounds; ++r) {  // uniform in the workgroup
             // the round's score table and row list; every wave has a stretch of ROWS * NB rows of
@@ -501,26 +503,9 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
             uint32_t* lst_tslot = lst_row + S::LIST;                            // (LIST/16) table tile -> key slot
             float* lst_z = reinterpret_cast<float*>(lst_tslot + S::LIST / 16);  // (LIST, GS) the table
 
-            // ---- scan: the key tiles of this round's nodes were asked for a round ago -----------
-            int node[NB], cnt[NB];
-            uint32_t nmask[NB];
-#pragma unroll
-            for (int u = 0; u < NB; ++u) {
-                node[u] = nx_node[u];
-                cnt[u] = nx_cnt[u];
-                nmask[u] = nx_mask[u];
-            }
-            // all the products first: the operand registers are free before the bookkeeping starts
-            f32x4_t sco_all[NB][MT];
-#pragma unroll
-            for (int u = 0; u < NB; ++u)
-#pragma unroll
-                for (int tt = 0; tt < MT; ++tt)  // (only read where it is written: under this condition)
-                    if (tt * 16 < cnt[u]) sco_all[u][tt] = tile_scores_lds<KS>(a[u][tt], s_bq, lane);
-            // ... and taken again at once by the next round's keys, which are on their way while
-            // this round's rows are listed and gathered
-            if (r + 1 < rounds) fetch(r + 1);
-
+            // ---- scan: the key tiles of this round's nodes were asked for a round ago; node by
+            // node: the products, at once the request for the node that takes its place in the
+            // next round, then the node's bookkeeping while the other tiles arrive -------------------
             if (r == 0) HIRA_TL(8);
             // The bookkeeping below derives everything per-lane from this copy, which the compiler
             // cannot see through: otherwise it computes those values once, ahead of the loop, and
@@ -532,8 +517,18 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
             int nsel = 0;  // rows of my stretch of the list
             float zmax = -INFINITY;
             const int zrow0 = wave * (NB * S::ROWS);  // my stretch of the round's rows
+            int node[NB], cnt[NB];
+            uint32_t nmask[NB];
 #pragma unroll
             for (int u = 0; u < NB; ++u) {
+                node[u] = nx_node[u];
+                cnt[u] = nx_cnt[u];
+                nmask[u] = nx_mask[u];
+                f32x4_t sco_u[MT];
+#pragma unroll
+                for (int tt = 0; tt < MT; ++tt)  // (only read where it is written: under this condition)
+                    if (tt * 16 < cnt[u]) sco_u[tt] = tile_scores_lds<KS>(a[u][tt], s_bq, lane);
+                if (r + 1 < rounds) fetch(r + 1, u);
                 // a head for which the node did not survive selects nothing
                 const float tau_u = ((nmask[u] >> col) & 1u) ? tau : INFINITY;
                 const unsigned slot0 = (unsigned)(node_of(max(node[u], 0)) * bf);
@@ -541,7 +536,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
 #pragma unroll
                 for (int tt = 0; tt < MT; ++tt) {
                     if (tt * 16 >= cnt[u]) continue;  // uniform
-                    const f32x4_t sco = sco_all[u][tt];
+                    const f32x4_t sco = sco_u[tt];
                     const int lim = cnt[u] - tt * 16 - 4 * kb;  // my rows j < lim hold keys
                     unsigned sel4 = 0u;
 #pragma unroll
