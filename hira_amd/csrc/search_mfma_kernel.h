@@ -4,8 +4,8 @@
 // One workgroup (8 waves; 256 registers a wave, so the only one on its CU) owns a few
 // tiles of 16 level-1 nodes of one tree, a stride apart; workgroup ids run fastest over the trees
 // so that, with 8 L2 slices (XCDs) served round-robin, the workgroups of one tree share a
-// slice.  The work is split by phase, not by node, so that neither the key scan nor the
-// value gather depends on where in the tree the selected keys sit:
+// slice.  After a common gate every wave scans and gathers on its own; the waves meet again
+// for the merge:
 //   gate   wave w gates the workgroup's tile w: it issues, before it waits for anything, every
 //          load it needs (queries, the 16 x D tile of level-1 centres, the tiles holding the
 //          tile's ancestors, radii, child counts) and gates with v_mfma_f32_16x16x32_bf16:
