@@ -79,12 +79,27 @@ def hira_attention_forward(module, query, key, value, attention_mask=None, dropo
     if hira_threshold is None:
         topk = hira_topk or getattr(module, "hira_topk", None) or max(1, indexer.num_keys // 100)
         hira_threshold = index_thresholds(indexer, query, topk)
-    scale = torch.full((b * h_q,), float(scaling), dtype=torch.float32, device=query.device)
+    # one plan per (index, head count, scale): a decode step is then a single library call
+    plans = searcher.__dict__.setdefault("_decode_plans", {})
+    key_ = (id(indexer), b * h_q, float(scaling))
+    plan = plans.get(key_)
+    if plan is None or plan.indexer is not indexer:
+        scale = torch.full((b * h_q,), float(scaling), dtype=torch.float32, device=indexer.device)
+        plan = plans[key_] = searcher.plan_attention(indexer, b * h_q, scaling=scale)
+    q2 = query.reshape(b * h_q, d).to(device=indexer.device, dtype=indexer.dtype).contiguous()
+    th = torch.as_tensor(hira_threshold, dtype=torch.float32, device=indexer.device)
+    if th.ndim == 0:
+        th = th.expand(b * h_q)
+    th = th.reshape(b * h_q).contiguous()
+    out = torch.empty((b * h_q, indexer.vdim), dtype=torch.float32, device=indexer.device)
     qk, qv = cache.queued_keys, cache.queued_values
-    out = searcher.search_attention(
-        query, hira_threshold, indexer, scaling=scale,
-        queue_keys=qk if qk is not None and qk.shape[-2] > 0 else None,
-        queue_values=qv if qv is not None and qv.shape[-2] > 0 else None)
+    if qk is not None and qk.shape[-2] > 0:
+        m = qk.shape[-2]
+        qk = qk.to(device=indexer.device, dtype=indexer.dtype).reshape(indexer.num_trees, m, d).contiguous()
+        qv = qv.to(device=indexer.device, dtype=indexer.dtype).reshape(indexer.num_trees, m, -1).contiguous()
+        plan.run(q2, th, out, queue_keys=qk, queue_values=qv)
+    else:
+        plan.run(q2, th, out)
     return out.reshape(b, 1, h_q, -1).to(query.dtype), None
 
 

@@ -458,7 +458,7 @@ static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* que
     const bool mfma_ok = mfma_search_supported(t, queue);
     HIRA_CHECK_ARG(want != 2 || mfma_ok,
                    "the MFMA kernel needs bf16, tiled layout, >= 2 levels, fan-out 16/32/48/64, "
-                   "dim = vdim in {64,128,256}");
+                   "dim = vdim in {64,128,256}, under 4 GiB of key slots per tree");
     plan->kernel = (want == 2 || (want == 0 && mfma_ok)) ? 2 : 1;
     plan->lpr = lpr;
     if (plan->kernel == 2) {
@@ -548,10 +548,14 @@ static int dispatch_lpr(const SearchPlan& plan, const SearchParams& p, dim3 grid
 using namespace hira;
 
 // partials (acc, m, l) followed by the arrival counters of the fused fold
+// bytes of the arrival counters, which come first: their place does not depend on the
+// number of partials, so a workspace stays usable when the tree grows or a queue comes and goes
+static size_t counter_bytes(int trees, int passes) {
+    return (((size_t)trees * passes * sizeof(int32_t)) + 255) & ~(size_t)255;
+}
+
 static size_t workspace_need(int h_q, size_t P, int vdim, int trees, int passes) {
-    size_t b = (size_t)h_q * P * (size_t)(vdim + 2) * sizeof(float);
-    b = (b + 255) & ~(size_t)255;
-    return b + (size_t)trees * passes * sizeof(int32_t);
+    return counter_bytes(trees, passes) + (size_t)h_q * P * (size_t)(vdim + 2) * sizeof(float);
 }
 
 extern "C" size_t hira_search_workspace_bytes(const HiraTree* tree, const HiraQuery* query,
@@ -639,7 +643,8 @@ extern "C" int hira_search(const HiraTree* tree, const HiraQuery* query, const H
                                            tree->num_trees, plan.head_chunks);
         if (workspace == nullptr || workspace_bytes < need)
             return fail(HIRA_EWORKSPACE, "workspace %zu bytes, need %zu", workspace_bytes, need);
-        float* w = reinterpret_cast<float*>(workspace);
+        float* w = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) +
+                                            counter_bytes(tree->num_trees, plan.head_chunks));
         p.part_acc = w;
         p.part_m = w + (size_t)query->num_q_heads * P * tree->vdim;
         p.part_l = p.part_m + (size_t)query->num_q_heads * P;
@@ -647,9 +652,7 @@ extern "C" int hira_search(const HiraTree* tree, const HiraQuery* query, const H
         // the MFMA kernel folds the partials itself (the last workgroup of a tree to arrive
         // does it) unless the caller asks for the second launch
         if (plan.kernel == 2 && !(launch && launch->separate_merge))
-            p.done = reinterpret_cast<int32_t*>(
-                reinterpret_cast<char*>(workspace) + need -
-                (size_t)tree->num_trees * plan.head_chunks * sizeof(int32_t));
+            p.done = reinterpret_cast<int32_t*>(workspace);
     }
     p.group_size = query->group_size > 0 ? query->group_size : 0;
     if (p.group_size > 0)

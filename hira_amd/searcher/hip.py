@@ -263,20 +263,27 @@ class DecodePlan:
         self.out.stats = None if stats is None else stats.data_ptr()
         self.launch = searcher.launch
         self.tree = indexer.tree_struct()
-        fake_q = _lib.HiraQuery(num_q_heads, 1, 1, 1, 1, 1, gmax, group)  # sizes only
-        self.ws_bytes = self.lib.hira_search_workspace_bytes(
-            C.byref(self.tree), C.byref(fake_q), None, C.byref(self.launch))
+        self.queue = _lib.HiraQueue(1, 1, 1, 1)  # sizes only: room for a queue's partials
+        self.ws_bytes = self._workspace_need()
         self.ws = torch.zeros(max(self.ws_bytes, 1), dtype=torch.uint8, device=dev)
         self._refs = (C.byref(self.tree), C.byref(self.query), C.byref(self.out),
                       C.byref(self.launch))
 
+    def _workspace_need(self) -> int:
+        fake_q = _lib.HiraQuery(self.query.num_q_heads, 1, 1, 1, 1, 1, self.query.max_group,
+                                self.query.group_size)  # sizes only
+        return self.lib.hira_search_workspace_bytes(
+            C.byref(self.tree), C.byref(fake_q), C.byref(self.queue), C.byref(self.launch))
+
     def run(self, query: torch.Tensor, threshold: torch.Tensor, out: torch.Tensor,
-            stream: Optional[int] = None) -> None:
+            stream: Optional[int] = None, queue_keys: Optional[torch.Tensor] = None,
+            queue_values: Optional[torch.Tensor] = None) -> None:
+        """queue_keys / queue_values: (T, m, D) / (T, m, Dv) contiguous, tree dtype: keys not in
+        the index yet, attended by every head of their tree."""
         if self.indexer.tree_struct() is not self.tree:  # the index grew since the plan was made
             self.tree = self.indexer.tree_struct()
-            need = self.lib.hira_search_workspace_bytes(
-                C.byref(self.tree), C.byref(self.query), None, C.byref(self.launch))
-            if need > self.ws_bytes:
+            need = self._workspace_need()
+            if need > self.ws.numel():
                 self.ws = torch.zeros(need, dtype=torch.uint8, device=self.indexer.device)
             self.ws_bytes = need
             self._refs = (C.byref(self.tree), C.byref(self.query), C.byref(self.out),
@@ -287,6 +294,11 @@ class DecodePlan:
         if stream is None:
             stream = torch.cuda.current_stream(self.indexer.device).cuda_stream
         t, q, o, l = self._refs
-        rc = self.lib.hira_search(t, q, None, o, l, self.ws.data_ptr(), self.ws_bytes, stream)
+        qu = None
+        if queue_keys is not None and queue_keys.shape[-2] > 0:
+            m = int(queue_keys.shape[-2])
+            self.queue = _lib.HiraQueue(queue_keys.data_ptr(), queue_values.data_ptr(), m, m)
+            qu = C.byref(self.queue)
+        rc = self.lib.hira_search(t, q, qu, o, l, self.ws.data_ptr(), self.ws_bytes, stream)
         if rc:
             _lib.check(rc)

@@ -138,9 +138,12 @@ typedef struct HiraLaunch {
 int hira_abi_version(void);
 const char* hira_last_error(void);
 
-/* Bytes of workspace hira_search needs for this tree/query (attention partials + arrival
- * counters).  The workspace must be ZERO before its first use; every completed call leaves
- * the counters zero again, so it can be reused without clearing.  Two calls that may run
+/* Bytes of workspace hira_search needs for this tree/query (arrival counters, one per tree
+ * and head pass, at the start; attention partials after them).  The workspace must be ZERO
+ * before its first use; every completed call leaves the counters zero again, and they sit
+ * at an offset that depends only on the number of trees and head passes, so a workspace can
+ * be reused without clearing by any later call with the same trees and heads that needs no
+ * more bytes (a tree that grew, a queue that came or went).  Two calls that may run
  * concurrently need separate workspaces. */
 size_t hira_search_workspace_bytes(const HiraTree* tree, const HiraQuery* query,
                                    const HiraQueue* queue, const HiraLaunch* launch);

@@ -203,3 +203,36 @@ def test_cache_layer_end_to_end(gpu_device):
         ref = torch.nn.functional.scaled_dot_product_attention(q.float(), kk, vv, scale=d ** -0.5)
         err = (att.float().transpose(1, 2) - ref).abs().max() / ref.abs().max()
         assert float(err) < 1e-2, float(err)
+
+
+def test_decode_plan_survives_updates_and_queue_changes(gpu_device):
+    """One DecodePlan (one workspace) reused while the tree grows and a queue comes and goes
+    gives the same output as a fresh call with a fresh workspace each time."""
+    from hira_amd.indexer.hip import HIPIndexer
+    from hira_amd.searcher.hip import HIPSearcher
+
+    t, h_q, d, bf, n0 = 2, 8, 128, 32, 3000
+    keys = bf16_round(clustered_keys(t, n0 + 2200, d, seed=9, clusters=40))
+    K = torch.from_numpy(keys)[None].to(torch.bfloat16)
+    idx = HIPIndexer(3, 1, bf).build(K[:, :, :n0], K[:, :, :n0])
+    searcher = HIPSearcher()
+    scale = torch.full((h_q,), d ** -0.5)
+    plan = searcher.plan_attention(idx, h_q, scaling=scale)
+    q2kv = ho.default_q2kv(h_q, t)
+    at = n0
+    out = torch.empty((h_q, d), dtype=torch.float32, device="cuda")
+    # appends of 1..1100 keys change the number of level-1 tiles (and so the partials per head);
+    # queues of 0..3 keys add or drop the queue's partial
+    for step, (m, qlen) in enumerate([(0, 0), (1, 2), (0, 0), (1100, 3), (0, 1), (1000, 0), (5, 2), (0, 0)]):
+        print(f"step {step} append {m} queue {qlen}", flush=True)
+        if m:
+            idx.update(K[:, :, at:at + m], K[:, :, at:at + m])
+            at += m
+        q = bf16_round(random_query(h_q, d, seed=100 + step))
+        s = ho.scores(keys[:, :at], q, q2kv)
+        th = torch.from_numpy(midpoint_threshold(s, max(1, at // 30))).cuda()
+        qd = torch.from_numpy(q).to(torch.bfloat16).cuda()
+        qk = K[0, :, at:at + qlen].contiguous().cuda() if qlen else None
+        plan.run(qd, th, out, queue_keys=qk, queue_values=qk)
+        ref = searcher.search_attention(qd, th, idx, scaling=scale, queue_keys=qk, queue_values=qk)
+        assert rel_err(out.cpu().numpy(), ref.cpu().numpy()) <= 1e-6, step
