@@ -329,6 +329,31 @@ def main():
         e1.record(stream)
         stream.synchronize()
         eager_ms = e0.elapsed_time(e1)
+
+        # the same loop with an event after every step: the spread of single steps
+        # (event to event, so a step's figure includes its launch gap and the marker)
+        evs = [torch.cuda.Event(enable_timing=True) for _ in range(K + 1)]
+        evs[0].record(stream)
+        for i in range(W, total):
+            plan.run(q_d[i], taus[i], outs[i], stream=stream.cuda_stream)
+            evs[i - W + 1].record(stream)
+        stream.synchronize()
+        per_step = np.array([evs[i].elapsed_time(evs[i + 1]) * 1e3 for i in range(K)])
+
+        # what a plain streaming kernel reaches on this GPU: torch's elementwise add over
+        # 1 GiB in, 1 GiB out
+        src = torch.empty(256 * 1024 * 1024, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(2):
+            torch.add(src, 1.0, out=dst)
+        b0, b1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        b0.record(stream)
+        for _ in range(8):
+            torch.add(src, 1.0, out=dst)
+        b1.record(stream)
+        stream.synchronize()
+        stream_gbs = 8 * 2.0 * src.numel() * 4 / (b0.elapsed_time(b1) * 1e-3) / 1e9
+        del src, dst
     us_per_step = wall_ms * 1e3 / K
     kernel_us = graph_ms * 1e3 / K
 
@@ -399,6 +424,10 @@ def main():
         "algorithmic_bytes_per_step": round(alg_bytes),
         "gpu_us_per_step_events": round(kernel_us, 3),
         "eager_us_per_step": round(eager_ms * 1e3 / K, 3),
+        "eager_step_us": {"mean": round(float(per_step.mean()), 2),
+                          "median": round(float(np.median(per_step)), 2),
+                          "p99": round(float(np.percentile(per_step, 99)), 2)},
+        "streaming_add_GBps": round(stream_gbs, 1),
         "dense_attention_us": {k: round(v, 2) for k, v in dense_us.items()},
         "dense_attention_bytes": dense_bytes,
         "frac_of_dense_time": round(kernel_us / dense_best, 4),
