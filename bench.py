@@ -397,6 +397,28 @@ def main():
     d1.record()
     torch.cuda.synchronize()
     dense_us["ours_all_selected"] = d0.elapsed_time(d1) * 1e3 / 16
+
+    # thresholds from a key sample (1000 keys per tree, mean of the 10 best): the launch a
+    # deployment puts ahead of every search; K of them in one graph
+    from hira_amd.cache.threshold_finder import device_thresholds
+    pick = torch.randperm(w.n, generator=torch.Generator().manual_seed(12345))[:1000].to(dev)
+    samples = keys_d[:, :, pick].reshape(w.batch * w.h_kv, 1000, w.d).contiguous()
+    tau_s = torch.empty((h_all,), dtype=torch.float32, device=dev)
+    device_thresholds(samples, q_d[0], "sample_mean_topk", 10, out=tau_s)
+    g2 = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(g2, stream=stream):
+            for i in range(W, total):
+                device_thresholds(samples, q_d[i], "sample_mean_topk", 10, out=tau_s,
+                                  stream=stream.cuda_stream)
+        g2.replay()
+        stream.synchronize()
+        t0e, t1e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0e.record(stream)
+        g2.replay()
+        t1e.record(stream)
+        stream.synchronize()
+    thr_us = t0e.elapsed_time(t1e) * 1e3 / K
     dense_best = min(dense_us.values())
 
     e = 2 if w.dtype == torch.bfloat16 else 4
@@ -428,6 +450,7 @@ def main():
                           "median": round(float(np.median(per_step)), 2),
                           "p99": round(float(np.percentile(per_step, 99)), 2)},
         "streaming_add_GBps": round(stream_gbs, 1),
+        "sample_threshold_us": round(thr_us, 2),
         "dense_attention_us": {k: round(v, 2) for k, v in dense_us.items()},
         "dense_attention_bytes": dense_bytes,
         "frac_of_dense_time": round(kernel_us / dense_best, 4),

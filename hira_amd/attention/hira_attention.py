@@ -13,8 +13,10 @@ Calling convention of transformers' attention functions:
 * decode (L_q == 1): out[h] = softmax over {indexed keys with q_h.k >= tau_h} + {queued
   keys} of scaling * q_h.k, times V -- one fused search + sparse-attention launch.
 
-The threshold comes from ``hira_threshold`` (tensor (B*H_q,) or scalar) or from
-``hira_topk`` (int: select exactly the k best indexed keys per head).
+The threshold comes from ``hira_threshold`` (tensor (B*H_q,) or scalar), from ``hira_topk``
+(int: select exactly the k best indexed keys per head; scans every key, for tests), or, with
+neither given, from the cache layer's key sample by its configured rule (HiraConfig
+``threshold_method`` / ``sample_size``).
 """
 from __future__ import annotations
 
@@ -23,7 +25,6 @@ from typing import Optional
 import torch
 import torch.nn.functional as F
 
-from hira_amd.cache.threshold_finder import exact_topk
 
 
 def _repeat_kv(x: torch.Tensor, n_rep: int) -> torch.Tensor:
@@ -76,9 +77,13 @@ def hira_attention_forward(module, query, key, value, attention_mask=None, dropo
     b, h_q = query.shape[0], query.shape[1]
     if hira_threshold is None:
         hira_threshold = getattr(module, "hira_threshold", None)
-    if hira_threshold is None:
-        topk = hira_topk or getattr(module, "hira_topk", None) or max(1, indexer.num_keys // 100)
-        hira_threshold = index_thresholds(indexer, query, topk)
+    if hira_topk is None:
+        hira_topk = getattr(module, "hira_topk", None)
+    # with neither given: the cache layer's configured rule on its key sample, one small launch
+    # ahead of the search
+    sampled = hira_threshold is None and hira_topk is None and getattr(cache, "samples", None) is not None
+    if hira_threshold is None and not sampled:
+        hira_threshold = index_thresholds(indexer, query, hira_topk or max(1, indexer.num_keys // 100))
     # one plan per (index, head count, scale): a decode step is then a single library call
     plans = searcher.__dict__.setdefault("_decode_plans", {})
     key_ = (id(indexer), b * h_q, float(scaling))
@@ -87,19 +92,23 @@ def hira_attention_forward(module, query, key, value, attention_mask=None, dropo
         scale = torch.full((b * h_q,), float(scaling), dtype=torch.float32, device=indexer.device)
         plan = plans[key_] = searcher.plan_attention(indexer, b * h_q, scaling=scale)
     q2 = query.reshape(b * h_q, d).to(device=indexer.device, dtype=indexer.dtype).contiguous()
-    th = torch.as_tensor(hira_threshold, dtype=torch.float32, device=indexer.device)
-    if th.ndim == 0:
-        th = th.expand(b * h_q)
-    th = th.reshape(b * h_q).contiguous()
     out = torch.empty((b * h_q, indexer.vdim), dtype=torch.float32, device=indexer.device)
     qk, qv = cache.queued_keys, cache.queued_values
     if qk is not None and qk.shape[-2] > 0:
         m = qk.shape[-2]
         qk = qk.to(device=indexer.device, dtype=indexer.dtype).reshape(indexer.num_trees, m, d).contiguous()
         qv = qv.to(device=indexer.device, dtype=indexer.dtype).reshape(indexer.num_trees, m, -1).contiguous()
-        plan.run(q2, th, out, queue_keys=qk, queue_values=qv)
     else:
-        plan.run(q2, th, out)
+        qk = qv = None
+    if sampled:
+        plan.run_sampled(q2, cache.samples, cache.threshold_method, cache.threshold_topk, out,
+                         queue_keys=qk, queue_values=qv)
+    else:
+        th = torch.as_tensor(hira_threshold, dtype=torch.float32, device=indexer.device)
+        if th.ndim == 0:
+            th = th.expand(b * h_q)
+        th = th.reshape(b * h_q).contiguous()
+        plan.run(q2, th, out, queue_keys=qk, queue_values=qv)
     return out.reshape(b, 1, h_q, -1).to(query.dtype), None
 
 

@@ -35,6 +35,11 @@ class CacheOutput:
     prefill_values: torch.Tensor | None
     indexer: Any
     searcher: Any
+    # beyond the reference's fields: the layer's key sample (B*H_kv, S, D) and the rule that
+    # turns it into per-head thresholds (cache/hira_config.py:20-22 of the reference)
+    samples: torch.Tensor | None = None
+    threshold_method: str | None = None
+    threshold_topk: int = 1
 
 
 class HiraCacheLayer(CacheLayerMixin):
@@ -46,8 +51,11 @@ class HiraCacheLayer(CacheLayerMixin):
         update_every: int,
         indexer_kwargs: dict[str, Any],
         searcher_kwargs: dict[str, Any],
+        threshold_kwargs: dict[str, Any] | None = None,
     ):
         super().__init__()
+        self.threshold_kwargs = threshold_kwargs or {}
+        self.samples = None
         self.device_mode = device_mode
         self.update_every = update_every
         self.indexer_kwargs = indexer_kwargs
@@ -92,32 +100,40 @@ class HiraCacheLayer(CacheLayerMixin):
             self.lazy_initialization(key_states, value_states)
             self.indexer.build(key_states, value_states)
             self.indexed_len = key_states.shape[-2]
-            return (
-                CacheOutput(
-                    queued_keys=self.queued_keys,
-                    queued_values=self.queued_values,
-                    prefill_keys=key_states,
-                    prefill_values=value_states,
-                    indexer=self.indexer,
-                    searcher=self.searcher,
-                ),
-                None,
-            )
+            self._take_samples(key_states)
+            return self._output(key_states, value_states), None
         self.queued_keys = torch.cat([self.queued_keys, key_states], dim=-2)
         self.queued_values = torch.cat([self.queued_values, value_states], dim=-2)
         self.queued_len += key_states.shape[-2]
         if self.queued_len >= self.update_every:
             self.update_index()
-        return (
-            CacheOutput(
-                queued_keys=self.queued_keys,
-                queued_values=self.queued_values,
-                prefill_keys=None,
-                prefill_values=None,
-                indexer=self.indexer,
-                searcher=self.searcher,
-            ),
-            None,
+        return self._output(), None
+
+    def _take_samples(self, key_states):
+        """A seeded random sample of the prompt's keys per KV head, for the sample-based
+        threshold rules; none when the configured rule does not use one."""
+        kw = self.threshold_kwargs
+        if kw.get("method") not in ("sample_max", "sample_mean_topk") or kw.get("sample_size", 0) <= 0:
+            return
+        n = key_states.shape[-2]
+        s = min(int(kw["sample_size"]), n, 4096)
+        pick = torch.randperm(n, generator=torch.Generator().manual_seed(12345))[:s].sort().values
+        k4 = key_states if key_states.ndim == 4 else key_states[None]
+        self.samples = k4[:, :, pick.to(k4.device)].reshape(-1, s, self.dim).contiguous()
+
+    def _output(self, prefill_keys=None, prefill_values=None):
+        kw = self.threshold_kwargs
+        return CacheOutput(
+            queued_keys=self.queued_keys,
+            queued_values=self.queued_values,
+            prefill_keys=prefill_keys,
+            prefill_values=prefill_values,
+            indexer=self.indexer,
+            searcher=self.searcher,
+            samples=self.samples,
+            threshold_method=kw.get("method") if self.samples is not None else None,
+            threshold_topk=max(1, min(int(kw.get("topk", 1)),
+                                      self.samples.shape[1] if self.samples is not None else 1)),
         )
 
     def update_index(self):
@@ -151,6 +167,7 @@ class HiraCacheLayer(CacheLayerMixin):
             self.queued_values = self._empty_queue()
             self.queued_len = 0
             self.indexed_len = 0
+            self.samples = None
             self.is_initialized = False
         if hasattr(self, "cumulative_length"):
             self.cumulative_length = 0
@@ -179,6 +196,7 @@ class HiraCache(Cache):
                 update_every=self.update_every,
                 indexer_kwargs=hira_config.get_indexer_kwargs(),
                 searcher_kwargs=hira_config.get_searcher_kwargs(),
+                threshold_kwargs=hira_config.get_threshold_kwargs(),
             )
             for _ in layer_types
         ]

@@ -24,6 +24,7 @@ class HiraConfig:
     # threshold
     threshold_method: str = "sample_mean_topk"  # "sample_max" | "sample_mean_topk" | "exact_topk"
     sample_size: int = 1000
+    threshold_topk: int = 10  # k of "sample_mean_topk" (the reference passes k at the call)
     # searcher
     chunk_size = 8 * 1024
 
@@ -51,6 +52,11 @@ class HiraConfig:
             "max_iterations": self.max_iterations,
             "branching_factor": self.branching_factor,
         }
+
+    def get_threshold_kwargs(self) -> dict:
+        """What the cache layer needs to keep a key sample and turn it into thresholds."""
+        return {"method": self.threshold_method, "sample_size": self.sample_size,
+                "topk": self.threshold_topk}
 
     def get_searcher_kwargs(self) -> dict:
         if self.device_mode == DeviceMode.CUDA_ONLY:

@@ -1,0 +1,254 @@
+// hira_threshold: per-head thresholds from a sample of a tree's keys, one launch.
+//   tau[h] = max_s q_h . x_s                      (HIRA_TAU_SAMPLE_MAX)
+//   tau[h] = mean of the k largest q_h . x_s      (HIRA_TAU_SAMPLE_MEAN_TOPK)
+// One workgroup of sixteen waves per query head.  Scores: 16 lanes share a sample row (16 bytes
+// each per step), eight rows per lane group in flight.  Then either a maximum, or a bitonic sort
+// by the first four waves with the scores in registers (entry e*256 + thread of the padded
+// array lives in register e of that thread: partners 256 or more apart are a register swap,
+// partners inside a wave a cross-lane move, only the two distances in between go through LDS)
+// and a sum over the first k.
+#include "common.hip.h"
+
+namespace hira {
+
+constexpr int kTauThreads = 1024;
+constexpr int kTauWaves = kTauThreads / 64;
+constexpr int kTauMaxSamples = 4096;
+constexpr int kTauRows = 8;  // sample rows a lane group has in flight
+
+__device__ __forceinline__ float tau_block_reduce(float v, bool is_max, float* s_red) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const float o = __shfl_xor(v, off, 64);
+        v = is_max ? fmaxf(v, o) : v + o;
+    }
+    if (lane == 0) s_red[wave] = v;
+    __syncthreads();
+    float r = s_red[0];
+#pragma unroll
+    for (int w = 1; w < kTauWaves; ++w) r = is_max ? fmaxf(r, s_red[w]) : r + s_red[w];
+    return r;
+}
+
+constexpr int kTauSorters = 256;  // threads that hold the scores during the sort
+
+// One step of the bitonic sort (largest first) of 256 * EE entries, entry e*256 + tid in v[e]
+// of thread tid < 256: entry i meets entry i ^ J; in a stretch that ends up descending
+// ((i & LEN) == 0) the lower index keeps the larger value.  Every thread of the workgroup
+// calls it (the steps through LDS hold a barrier); only the sorters hold data.
+template <int EE, int LEN, int J>
+__device__ __forceinline__ void tau_sort_step(float (&v)[EE], float* s0, float* s1, int& buf,
+                                              int tid, bool sorter, bool rot4_first) {
+    constexpr int ST = kTauSorters;
+    if constexpr (J >= ST) {  // partner in another register of this thread
+        constexpr int JE = J / ST;
+        if (!sorter) return;
+#pragma unroll
+        for (int e = 0; e < EE; ++e) {
+            if ((e & JE) == 0 && (e | JE) < EE) {
+                const bool down = (((e * ST) & LEN) == 0);
+                const float lo = v[e], hi = v[e | JE];
+                const bool swap = down ? lo < hi : lo > hi;
+                v[e] = swap ? hi : lo;
+                v[e | JE] = swap ? lo : hi;
+            }
+        }
+    } else {
+        auto meet = [&](int e, float o) {
+            const int i = e * ST + tid;
+            const bool down = (i & LEN) == 0, lower = (i & J) == 0;
+            v[e] = (down == lower) ? fmaxf(v[e], o) : fminf(v[e], o);
+        };
+        if constexpr (J >= 64) {  // partner in another wave
+            float* sb = buf ? s1 : s0;
+            if (sorter) {
+#pragma unroll
+                for (int e = 0; e < EE; ++e) sb[e * ST + tid] = v[e];
+            }
+            __syncthreads();
+            if (sorter) {
+#pragma unroll
+                for (int e = 0; e < EE; ++e) meet(e, sb[e * ST + (tid ^ J)]);
+            }
+            buf ^= 1;  // the next exchange writes the other half: one barrier per step
+        } else if (!sorter) {
+            // (whole waves: the steps inside a wave are not theirs to spend issue slots on)
+        } else if constexpr (J >= 16) {
+#pragma unroll
+            for (int e = 0; e < EE; ++e) meet(e, __shfl_xor(v[e], J, 64));
+        } else if constexpr (J == 8) {
+#pragma unroll
+            for (int e = 0; e < EE; ++e) meet(e, dpp_move<0x128>(v[e]));  // row rotate by 8
+        } else if constexpr (J == 4) {
+#pragma unroll
+            for (int e = 0; e < EE; ++e) {
+                const float a = dpp_move<0x124>(v[e]), b = dpp_move<0x12C>(v[e]);  // by 4, by 12
+                meet(e, rot4_first ? a : b);
+            }
+        } else if constexpr (J == 2) {
+#pragma unroll
+            for (int e = 0; e < EE; ++e) meet(e, dpp_move<0x4E>(v[e]));  // quad [2,3,0,1]
+        } else {
+#pragma unroll
+            for (int e = 0; e < EE; ++e) meet(e, dpp_move<0xB1>(v[e]));  // quad [1,0,3,2]
+        }
+    }
+}
+
+// All steps from (LEN = 2^LL, J = 2^JJ) on, in order.
+template <int EE, int LOGN, int LL, int JJ>
+struct TauSortFrom {
+    static __device__ __forceinline__ void run(float (&v)[EE], float* s0, float* s1, int& buf,
+                                               int tid, bool sorter, bool rot4_first) {
+        tau_sort_step<EE, (1 << LL), (1 << JJ)>(v, s0, s1, buf, tid, sorter, rot4_first);
+        if constexpr (JJ > 0)
+            TauSortFrom<EE, LOGN, LL, JJ - 1>::run(v, s0, s1, buf, tid, sorter, rot4_first);
+        else if constexpr (LL < LOGN)
+            TauSortFrom<EE, LOGN, LL + 1, LL>::run(v, s0, s1, buf, tid, sorter, rot4_first);
+    }
+};
+
+// E = registers per thread of the sort: the padded array has 1024 * E entries
+template <typename T, int E>
+__global__ __launch_bounds__(kTauThreads) void k_threshold(
+    const T* __restrict__ samples, int S, int D, const T* __restrict__ q,
+    const int32_t* __restrict__ tree_q_off, const int32_t* __restrict__ tree_q_heads,
+    int group_size, int num_trees, int method, int k, float* __restrict__ tau) {
+    constexpr int EPL = Elem<T>::kPerChunk;
+    constexpr int NPAD = kTauThreads * E;
+    __shared__ float s_sc[2][NPAD];  // the scores; the two sides of an exchange through LDS
+    __shared__ float s_red[kTauWaves];
+    const int tid = threadIdx.x;
+
+    // the head of this workgroup and its tree
+    const int pos = blockIdx.x;
+    int head, tree;
+    if (group_size > 0) {
+        head = pos;
+        tree = pos / group_size;
+    } else {
+        tree = 0;
+        while (tree + 1 < num_trees && tree_q_off[tree + 1] <= pos) ++tree;  // uniform
+        head = tree_q_heads[pos];
+    }
+
+    // ---- scores: 16 lanes per sample row, 64 rows per pass, kTauRows passes at a time --------
+    const int sub = tid & 15, grp = tid >> 4;
+    const int chunks = D / EPL;
+    const T* xs = samples + (size_t)tree * S * D;
+    const T* qh = q + (size_t)head * D;
+    constexpr int PASS = kTauThreads / 16;
+    for (int r0 = 0; r0 < S; r0 += PASS * kTauRows) {  // uniform
+        float dot[kTauRows];
+        int row[kTauRows];
+#pragma unroll
+        for (int u = 0; u < kTauRows; ++u) {
+            dot[u] = 0.0f;
+            row[u] = min(r0 + u * PASS + grp, S - 1);
+        }
+        for (int c = sub; c < chunks; c += 16) {
+            uint4 raw[kTauRows];
+#pragma unroll
+            for (int u = 0; u < kTauRows; ++u) raw[u] = load_chunk<T>(xs, (size_t)row[u] * D, c);
+            float b[EPL];
+            unpack<T>(load_chunk<T>(qh, 0, c), b);
+#pragma unroll
+            for (int u = 0; u < kTauRows; ++u) {
+                float a[EPL];
+                unpack<T>(raw[u], a);
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) dot[u] += a[e] * b[e];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kTauRows; ++u) {
+            const float d = group_sum<16>(dot[u]);
+            if (sub == 0 && r0 + u * PASS + grp < S) s_sc[0][r0 + u * PASS + grp] = d;
+        }
+    }
+    __syncthreads();
+    // ---- from here on only the first four waves hold data; the others keep the barriers company
+    constexpr int ST = kTauSorters;
+    constexpr int EE = NPAD / ST;     // entries per sorting thread
+    constexpr int LOGN = E == 1 ? 10 : (E == 2 ? 11 : 12);
+    const bool sorter = tid < ST;
+    float v[EE];
+#pragma unroll
+    for (int e = 0; e < EE; ++e)
+        v[e] = (sorter && e * ST + tid < S) ? s_sc[0][e * ST + tid] : -INFINITY;
+
+    if (method == HIRA_TAU_SAMPLE_MAX) {
+        float m = v[0];
+#pragma unroll
+        for (int e = 1; e < EE; ++e) m = fmaxf(m, v[e]);
+        m = tau_block_reduce(m, true, s_red);
+        if (tid == 0) tau[head] = m;
+        return;
+    }
+
+    // ---- bitonic sort, largest first ---------------------------------------------------------
+    // Which of the two rotations by 4 inside a row of 16 lanes brings lane ^ 4: asked of the
+    // lane numbers themselves.
+    const int lane = tid & 63;
+    const bool rot4_first =
+        __builtin_amdgcn_update_dpp(0, lane, 0x124, 0xF, 0xF, true) == (lane ^ 4);
+    int buf = 1;
+    TauSortFrom<EE, LOGN, 1, 0>::run(v, s_sc[0], s_sc[1], buf, tid, sorter, rot4_first);
+    float sum = 0.0f;
+#pragma unroll
+    for (int e = 0; e < EE; ++e)
+        if (sorter && e * ST + tid < k) sum += v[e];
+    sum = tau_block_reduce(sum, false, s_red);
+    if (tid == 0) tau[head] = sum / (float)k;
+}
+
+template <typename T>
+static void launch_threshold(int e, dim3 grid, hipStream_t s, const void* samples, int S, int D,
+                             const HiraQuery* qu, int num_trees, int method, int k, float* tau) {
+    const T* x = static_cast<const T*>(samples);
+    const T* q = static_cast<const T*>(qu->q);
+    const dim3 block(kTauThreads);
+#define HIRA_TAU_LAUNCH(E)                                                                        \
+    hipLaunchKernelGGL((k_threshold<T, E>), grid, block, 0, s, x, S, D, q, qu->tree_q_off,        \
+                       qu->tree_q_heads, qu->group_size, num_trees, method, k, tau)
+    if (e == 1) HIRA_TAU_LAUNCH(1);
+    else if (e == 2) HIRA_TAU_LAUNCH(2);
+    else HIRA_TAU_LAUNCH(4);
+#undef HIRA_TAU_LAUNCH
+}
+
+}  // namespace hira
+
+extern "C" int hira_threshold(const void* samples, int32_t dtype, int32_t num_trees,
+                              int32_t num_samples, int32_t dim, const HiraQuery* query,
+                              int32_t method, int32_t k, float* tau_out, void* stream) {
+    using namespace hira;
+    HIRA_CHECK_ARG(samples && query && tau_out, "hira_threshold: null argument");
+    HIRA_CHECK_ARG(dtype == HIRA_F32 || dtype == HIRA_BF16, "hira_threshold: dtype %d", dtype);
+    HIRA_CHECK_ARG(num_trees >= 1 && dim >= 1, "hira_threshold: num_trees %d, dim %d", num_trees, dim);
+    const int epl = dtype == HIRA_F32 ? 4 : 8;
+    HIRA_CHECK_ARG(dim % epl == 0, "hira_threshold: dim %d must be a multiple of %d (16-byte chunks)", dim, epl);
+    HIRA_CHECK_ARG(num_samples >= 1 && num_samples <= kTauMaxSamples,
+                   "hira_threshold: %d samples per tree (1..%d)", num_samples, kTauMaxSamples);
+    HIRA_CHECK_ARG(method == HIRA_TAU_SAMPLE_MAX || method == HIRA_TAU_SAMPLE_MEAN_TOPK,
+                   "hira_threshold: method %d", method);
+    HIRA_CHECK_ARG(method == HIRA_TAU_SAMPLE_MAX || (k >= 1 && k <= num_samples),
+                   "hira_threshold: k = %d with %d samples", k, num_samples);
+    HIRA_CHECK_ARG(query->q && query->num_q_heads >= 1, "hira_threshold: query missing");
+    if (query->group_size > 0)
+        HIRA_CHECK_ARG(query->num_q_heads == num_trees * query->group_size,
+                       "hira_threshold: %d heads != %d trees x group of %d", query->num_q_heads,
+                       num_trees, query->group_size);
+    else
+        HIRA_CHECK_ARG(query->tree_q_off && query->tree_q_heads, "hira_threshold: head map missing");
+    const int e = num_samples <= kTauThreads ? 1 : (num_samples <= 2 * kTauThreads ? 2 : 4);
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const dim3 grid(query->num_q_heads);
+    if (dtype == HIRA_F32)
+        launch_threshold<float>(e, grid, s, samples, num_samples, dim, query, num_trees, method, k, tau_out);
+    else
+        launch_threshold<bf16_t>(e, grid, s, samples, num_samples, dim, query, num_trees, method, k, tau_out);
+    HIRA_CHECK_LAUNCH("hira_threshold");
+    return HIRA_OK;
+}

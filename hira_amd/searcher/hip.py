@@ -302,3 +302,30 @@ class DecodePlan:
         rc = self.lib.hira_search(t, q, qu, o, l, self.ws.data_ptr(), self.ws_bytes, stream)
         if rc:
             _lib.check(rc)
+
+    def run_sampled(self, query: torch.Tensor, samples: torch.Tensor, method: str, k: int,
+                    out: torch.Tensor, stream: Optional[int] = None,
+                    queue_keys: Optional[torch.Tensor] = None,
+                    queue_values: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """A decode step whose thresholds come from a key sample (T, S, D), tree dtype,
+        contiguous: ``hira_threshold`` ("sample_max" or "sample_mean_topk" with k) writes them
+        into a buffer of the plan, ``run`` follows on the same stream.  Returns that buffer."""
+        if getattr(self, "tau_buf", None) is None:
+            self.tau_buf = torch.empty((self.query.num_q_heads,), dtype=torch.float32,
+                                       device=self.indexer.device)
+        if samples.ndim != 3 or samples.shape[0] != self.tree.num_trees or \
+                samples.shape[2] != self.tree.dim or samples.dtype != self.indexer.dtype or \
+                not samples.is_contiguous():
+            raise ValueError(f"samples {tuple(samples.shape)} {samples.dtype}: expected contiguous "
+                             f"({self.tree.num_trees}, S, {self.tree.dim}) {self.indexer.dtype}")
+        if stream is None:
+            stream = torch.cuda.current_stream(self.indexer.device).cuda_stream
+        self.query.q = query.data_ptr()
+        rc = self.lib.hira_threshold(
+            samples.data_ptr(), self.tree.dtype, self.tree.num_trees, int(samples.shape[1]),
+            self.tree.dim, self._refs[1], 0 if method == "sample_max" else 1, int(k),
+            self.tau_buf.data_ptr(), stream)
+        if rc:
+            _lib.check(rc)
+        self.run(query, self.tau_buf, out, stream, queue_keys, queue_values)
+        return self.tau_buf

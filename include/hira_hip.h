@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define HIRA_ABI_VERSION 1
+#define HIRA_ABI_VERSION 2
 #define HIRA_MAX_LEVELS 8
 
 enum { HIRA_F32 = 0, HIRA_BF16 = 1 };
@@ -202,6 +202,22 @@ int hira_build(const HiraTree* tree, const void* keys_in, const void* values_in,
  */
 int hira_update(const HiraTree* tree, const void* new_keys, const void* new_values, int32_t m,
                 int32_t* state, void* stream);
+
+/*
+ * Per-head thresholds from a sample of each tree's keys, in one launch ahead of hira_search
+ * on the same stream.  The reference names the two rules and leaves them unwritten
+ * (cache/threshold_finder.py:1-14: sample_max and sample_mean_topk raise NotImplementedError;
+ * cache/hira_config.py:20-22 holds their settings threshold_method and sample_size):
+ *   HIRA_TAU_SAMPLE_MAX        tau[h] = max over the samples x of head h's tree of q_h.x
+ *   HIRA_TAU_SAMPLE_MEAN_TOPK  tau[h] = mean of the k largest q_h.x  (1 <= k <= num_samples)
+ *   samples    (num_trees, num_samples, dim) row-major in `dtype`, num_samples <= 4096
+ *   query      q, num_q_heads and the head map are read (tau and scaling are not)
+ *   tau_out    (H_q) fp32; scores are accumulated in fp32
+ */
+enum { HIRA_TAU_SAMPLE_MAX = 0, HIRA_TAU_SAMPLE_MEAN_TOPK = 1 };
+int hira_threshold(const void* samples, int32_t dtype, int32_t num_trees, int32_t num_samples,
+                   int32_t dim, const HiraQuery* query, int32_t method, int32_t k,
+                   float* tau_out, void* stream);
 
 #ifdef __cplusplus
 }

@@ -80,6 +80,21 @@ def scores(keys, query, q2kv=None, fast: bool = False) -> np.ndarray:
     return out
 
 
+def sample_thresholds(samples, query, method: str, k: int = 1, q2kv=None) -> np.ndarray:
+    """The two threshold rules the reference names and leaves unwritten
+    (cache/threshold_finder.py:1-14; settings in cache/hira_config.py:20-22): per query head,
+    the largest score q.x over its tree's samples ("sample_max") or the mean of the k largest
+    ("sample_mean_topk").  Scores and the mean in float64."""
+    x, q = np.asarray(samples, np.float64), np.asarray(query, np.float64)
+    h_q = q.shape[0]
+    q2kv = default_q2kv(h_q, x.shape[0]) if q2kv is None else np.asarray(q2kv)
+    s = np.einsum("hsd,hd->hs", x[q2kv], q)
+    if method == "sample_max":
+        return s.max(1).astype(np.float32)
+    assert method == "sample_mean_topk" and 1 <= k <= s.shape[1]
+    return (-np.sort(-s, axis=1))[:, :k].mean(1).astype(np.float32)
+
+
 def brute_force(keys, query, th, sc=None, q2kv=None) -> np.ndarray:
     keys, query, th = _f32(keys), _f32(query), _f32(th)
     h_kv, n, d = keys.shape
