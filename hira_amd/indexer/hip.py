@@ -296,6 +296,92 @@ class HIPIndexer(BaseIndexer):
         self.num_keys = int(num_keys if num_keys is not None else (perm[0] >= 0).sum().item())
         return self
 
+    # ------------------------------------------------------------------ persistence
+    def save(self, path: str) -> None:
+        """Write the index to one safetensors file: every level array as it is stored on the
+        device (keys and centres in their storage layout, rows beyond the slots in use cut
+        off), the update bookkeeping, and the constructor settings in the file's metadata.
+        ``HIPIndexer.load`` restores it bit for bit.  (The reference has no persistence; its
+        config loaders and example configs point at one: cache/hira_config.py:27-33.)"""
+        import json
+
+        from safetensors.torch import save_file
+
+        if self.keys_buf is None:
+            raise ValueError("Indexer is not built: nothing to save.")
+        rows = [(-(-s // 16) * 16 if self.tiled else s) for s in self.size]
+        tensors = {"keys": self.keys_buf[:, : rows[0]], "perm": self.perm[:, : rows[0]]}
+        if self.values_buf is not None:
+            tensors["values"] = self.values_buf[:, : rows[0]]
+        for l in range(1, self.num_levels):
+            tensors[f"centers.{l}"] = self.centers[l][:, : rows[l]]
+            tensors[f"radii.{l}"] = self.radii[l][:, : rows[l]]
+            tensors[f"counts.{l}"] = self.counts[l][:, : rows[l]]
+        if self._state is not None:
+            tensors["update_state"] = self._state
+        meta = {
+            "format": "hira_amd.index.v1", "num_levels": self.num_levels,
+            "branching_factor": self.branching_factor, "max_iterations": self.max_iterations,
+            "pack_rounds": self.pack_rounds, "seed": self.seed, "pad_value": self.pad_value,
+            "layout_request": self.layout_request, "tiled": self.tiled, "batch": self.batch,
+            "num_heads": self.num_heads, "dim": self.dim, "vdim": self.vdim,
+            "dtype": "bfloat16" if self.dtype == torch.bfloat16 else "float32",
+            "size": list(self.size), "rows": rows, "num_keys": self.num_keys,
+        }
+        save_file({k: v.detach().cpu().contiguous() for k, v in tensors.items()}, path,
+                  metadata={"hira": json.dumps(meta)})
+
+    @classmethod
+    def load(cls, path: str, device: str = "cuda", capacity: Optional[int] = None) -> "HIPIndexer":
+        """Restore an index written by ``save`` (safetensors: nothing from the file is
+        executed).  ``capacity`` reserves key slots per tree for later appends."""
+        import json
+
+        from safetensors import safe_open
+
+        with safe_open(path, framework="pt", device="cpu") as f:
+            raw = (f.metadata() or {}).get("hira")
+            if raw is None:
+                raise ValueError(f"{path}: not an index file (no 'hira' metadata)")
+            meta = json.loads(raw)
+            if meta.get("format") != "hira_amd.index.v1":
+                raise ValueError(f"{path}: unknown index format {meta.get('format')!r}")
+            tensors = {k: f.get_tensor(k) for k in f.keys()}
+        self = cls(meta["num_levels"], meta["max_iterations"], meta["branching_factor"],
+                   pad_value=meta["pad_value"], seed=meta["seed"], pack_rounds=meta["pack_rounds"],
+                   layout=meta["layout_request"], capacity=capacity, device=device)
+        dtype = torch.bfloat16 if meta["dtype"] == "bfloat16" else torch.float32
+        size, rows = list(meta["size"]), list(meta["rows"])
+        # room for what the file holds (and for `capacity`), then the saved sizes
+        self._allocate(meta["batch"], meta["num_heads"], max(rows[0], 1), meta["dim"],
+                       meta["vdim"], dtype)
+        if self.tiled != bool(meta["tiled"]):
+            raise ValueError(f"{path}: stored layout does not match what this build would choose")
+        self.size = list(rows)
+        self._grow(rows)
+        self.size = size
+
+        def put(dst, name):
+            src = tensors[name]
+            if tuple(src.shape[2:]) != tuple(dst.shape[2:]) or src.shape[0] != dst.shape[0] \
+                    or src.shape[1] > dst.shape[1] or src.dtype != dst.dtype:
+                raise ValueError(f"{path}: tensor {name} {tuple(src.shape)} {src.dtype} does not fit")
+            dst[:, : src.shape[1]] = src.to(self.device)
+
+        put(self.keys_buf, "keys")
+        put(self.perm, "perm")
+        if self.values_buf is not None:
+            put(self.values_buf, "values")
+        for l in range(1, self.num_levels):
+            put(self.centers[l], f"centers.{l}")
+            put(self.radii[l], f"radii.{l}")
+            put(self.counts[l], f"counts.{l}")
+        if "update_state" in tensors:
+            self._state = tensors["update_state"].to(self.device)
+        self.num_keys = int(meta["num_keys"])
+        self._tree_struct = None
+        return self
+
     # ------------------------------------------------------------------ build / update
     @torch.no_grad()
     def build(self, keys: torch.Tensor, values: Optional[torch.Tensor] = None):

@@ -124,6 +124,19 @@ def test_threshold_rules():
     s2 = torch.einsum("hnd,hd->hn", keys[m], q)
     assert torch.allclose(threshold_finder.sample_max(keys, q, m), s2.max(1).values)
     assert set(threshold_finder.THRESHOLD_METHODS) >= {"sample_max", "sample_mean_topk"}
+    # the float64 restatement the GPU tests check hira_threshold against: same rules via
+    # numpy's sort, against torch's topk here; k = 1 is the maximum, k = all the mean score
+    from oracle import hira_oracle as ho
+    kn, qn = keys.numpy(), q.numpy()
+    assert np.allclose(ho.sample_thresholds(kn, qn, "sample_max"), s.max(1).values.numpy(), rtol=1e-6)
+    assert np.allclose(ho.sample_thresholds(kn, qn, "sample_mean_topk", 10),
+                       s.topk(10, dim=1).values.mean(1).numpy(), rtol=1e-5, atol=1e-6)
+    assert np.array_equal(ho.sample_thresholds(kn, qn, "sample_mean_topk", 1),
+                          ho.sample_thresholds(kn, qn, "sample_max"))
+    assert np.allclose(ho.sample_thresholds(kn, qn, "sample_mean_topk", 500), s.mean(1).numpy(),
+                       rtol=1e-4, atol=1e-5)
+    assert np.allclose(ho.sample_thresholds(kn, qn, "sample_max", q2kv=m.numpy()),
+                       s2.max(1).values.numpy(), rtol=1e-6)
 
 
 def test_synthetic_workloads_are_seeded_and_shaped():

@@ -236,3 +236,58 @@ def test_decode_plan_survives_updates_and_queue_changes(gpu_device):
         plan.run(qd, th, out, queue_keys=qk, queue_values=qk)
         ref = searcher.search_attention(qd, th, idx, scaling=scale, queue_keys=qk, queue_values=qk)
         assert rel_err(out.cpu().numpy(), ref.cpu().numpy()) <= 1e-6, step
+
+
+@pytest.mark.parametrize("dtype,d,bf,nl", [(torch.bfloat16, 128, 32, 3), (torch.float32, 32, 8, 4),
+                                           (torch.float32, 16, 4, 1)])
+def test_save_load_roundtrip(dtype, d, bf, nl, gpu_device, tmp_path):
+    """An index that took appends, written to a file and read back: every array equal, the
+    same search result, and the same tree after further appends as the index that never
+    left the device."""
+    from hira_amd.indexer.hip import HIPIndexer
+    from hira_amd.searcher.hip import HIPSearcher
+
+    t, n0, m1, m2 = 2, 700, 150, 90
+    n = n0 + m1 + m2
+    rnd = bf16_round if dtype == torch.bfloat16 else (lambda x: x)
+    keys = rnd(clustered_keys(t, n, d, seed=21, clusters=14))
+    K = torch.from_numpy(keys)[None].to(dtype)
+    a = HIPIndexer(nl, 1, bf).build(K[:, :, :n0], K[:, :, :n0])
+    a.update(K[:, :, n0:n0 + m1], K[:, :, n0:n0 + m1])
+    path = str(tmp_path / "index.safetensors")
+    a.save(path)
+    b = HIPIndexer.load(path)
+    assert (b.size, b.num_keys, b.tiled, b.dtype) == (a.size, a.num_keys, a.tiled, a.dtype)
+
+    def same(x, y):
+        s0 = a.size[0]
+        assert torch.equal(x.perm[:, :s0], y.perm[:, :s0])
+        assert torch.equal(x.keys_rowmajor()[:, :s0], y.keys_rowmajor()[:, :s0])
+        assert torch.equal(x.values_buf[:, :s0], y.values_buf[:, :s0])
+        for l in range(1, nl):
+            k = x.size[l]
+            assert torch.equal(x.centers_rowmajor(l)[:, :k], y.centers_rowmajor(l)[:, :k])
+            assert torch.equal(x.radii[l][:, :k], y.radii[l][:, :k])
+            assert torch.equal(x.counts[l][:, :k], y.counts[l][:, :k])
+
+    same(a, b)
+    q = rnd(random_query(2 * t, d, seed=3))
+    q2kv = ho.default_q2kv(2 * t, t)
+    s = ho.scores(keys[:, :n0 + m1], q, q2kv)
+    th = midpoint_threshold(s, 40)
+    se = HIPSearcher(index_space="position")
+    out_a = se.search(torch.from_numpy(q), torch.from_numpy(th), a).clone()
+    out_b = se.search(torch.from_numpy(q), torch.from_numpy(th), b)
+    assert torch.equal(out_a, out_b)
+    assert_same_selection(out_b.cpu().numpy() != 0, s, th)
+    a.update(K[:, :, n0 + m1:], K[:, :, n0 + m1:])
+    b.update(K[:, :, n0 + m1:], K[:, :, n0 + m1:])
+    assert a.size == b.size and a.num_keys == b.num_keys == n
+    same(a, b)
+    _check_tree(b, keys, keys)
+    with pytest.raises(ValueError):
+        HIPIndexer(3, 1, 8).save(path)          # not built
+    from safetensors.torch import save_file
+    save_file({"x": torch.zeros(1)}, str(tmp_path / "other.safetensors"))
+    with pytest.raises(ValueError):
+        HIPIndexer.load(str(tmp_path / "other.safetensors"))
