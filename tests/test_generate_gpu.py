@@ -35,9 +35,10 @@ def _set(model, **attrs):
                 setattr(m, k, v)
 
 
-@pytest.mark.parametrize("dtype,head_dim,bf,tol", [(torch.float32, 32, 8, 1e-4),
-                                                  (torch.bfloat16, 64, 16, 6e-2)])
-def test_llama_decode_matches_dense_when_every_key_is_selected(dtype, head_dim, bf, tol, gpu_device):
+@pytest.mark.parametrize("dtype,head_dim,bf,tol,batch", [(torch.float32, 32, 8, 1e-4, 1),
+                                                        (torch.float32, 32, 8, 1e-4, 3),  # the reference: B = 1 only
+                                                        (torch.bfloat16, 64, 16, 6e-2, 2)])
+def test_llama_decode_matches_dense_when_every_key_is_selected(dtype, head_dim, bf, tol, batch, gpu_device):
     from hira_amd.cache.hira_cache import HiraCache
     from hira_amd.cache.hira_config import DeviceMode, HiraConfig
 
@@ -46,7 +47,7 @@ def test_llama_decode_matches_dense_when_every_key_is_selected(dtype, head_dim, 
     hc = HiraConfig(device_mode=DeviceMode.CUDA_ONLY, update_every=4, num_levels=3,
                     branching_factor=bf, threshold_method="none")
     cache = HiraCache(cfg, hc)
-    ids = torch.randint(0, 512, (1, 300), device="cuda", generator=torch.Generator("cuda").manual_seed(1))
+    ids = torch.randint(0, 512, (batch, 300), device="cuda", generator=torch.Generator("cuda").manual_seed(1))
     with torch.no_grad():
         o_ref = ref(ids, use_cache=True)
         o = model(ids, past_key_values=cache, use_cache=True)
