@@ -130,3 +130,46 @@ def test_cache_layer_uses_its_sample_rule(gpu_device):
         assert rel_err(att.float().cpu().numpy().reshape(h_q, d), ref) <= 1e-2, step
         assert 0 < mask[:, : layer.indexed_len].mean() < 0.5
     assert compared >= 3
+
+
+def test_decode_step_in_a_hip_graph(gpu_device):
+    """Thresholds + search + attention captured once and replayed with new queries, with eager
+    work and synchronisation between the replays: every replay equals the eager result."""
+    from hira_amd.indexer.hip import HIPIndexer
+    from hira_amd.searcher.hip import HIPSearcher
+
+    t, n, d, h = 4, 5000, 128, 16
+    keys = bf16_round(clustered_keys(t, n, d, seed=14, clusters=50))
+    K = torch.from_numpy(keys)[None].to(torch.bfloat16).cuda()
+    idx = HIPIndexer(3, 1, 32).build(K, K)
+    pick = torch.randperm(n, generator=torch.Generator().manual_seed(1))[:500].cuda()
+    samples = K[0][:, pick].contiguous()
+    queue = K[0][:, :3].contiguous()
+    se = HIPSearcher()
+    scale = torch.full((h,), d ** -0.5)
+    plan = se.plan_attention(idx, h, scaling=scale)
+    q_in = torch.zeros((h, d), dtype=torch.bfloat16, device="cuda")
+    out = torch.zeros((h, d), dtype=torch.float32, device="cuda")
+    plan.run_sampled(q_in, samples, "sample_mean_topk", 8, out, queue_keys=queue, queue_values=queue)
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            plan.run_sampled(q_in, samples, "sample_mean_topk", 8, out, stream=stream.cuda_stream,
+                             queue_keys=queue, queue_values=queue)
+    eager_plan = se.plan_attention(idx, h, scaling=scale)
+    for rep in range(4):
+        q = torch.from_numpy(bf16_round(random_query(h, d, seed=70 + rep))).to(torch.bfloat16).cuda()
+        q_in.copy_(q)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        want = torch.empty_like(out)
+        tau = eager_plan.run_sampled(q, samples, "sample_mean_topk", 8, want, queue_keys=queue,
+                                     queue_values=queue).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(tau, plan.tau_buf), rep
+        assert torch.equal(got, want), rep
+        assert float(got.abs().max()) > 0
