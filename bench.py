@@ -215,6 +215,9 @@ def main():
                     help="after the timed steps: append this many keys one per step, a search "
                          "after each, one level-2 subtree rebuilt every --rebuild-every steps")
     ap.add_argument("--rebuild-every", type=int, default=512)
+    ap.add_argument("--npz", default=None,
+                    help="keys and queries captured from a model (the reference sampler's .npz: "
+                         "keys (N,D), queries (N,D)) instead of the synthetic ones")
     ap.add_argument("--counters", action="store_true",
                     help="run the steps once, untimed, plus a kernel of known traffic "
                          "(for rocprofv3 --pmc runs)")
@@ -239,8 +242,11 @@ def main():
     K, W = a.steps, a.warmup
     total = K + W
     log(f"[bench] workload {w.name}: generating keys/values/queries on the host")
-    keys, values = synth.make_kv(w)
-    queries = synth.make_queries(w, keys, total)  # (total, B, H_q, D)
+    if a.npz:
+        w, keys, values, queries = synth.load_capture(a.npz, w, total)
+    else:
+        keys, values = synth.make_kv(w)
+        queries = synth.make_queries(w, keys, total)  # (total, B, H_q, D)
     keys_d, values_d = keys.to(dev), values.to(dev)
     niter = w.kmeans_iters if a.kmeans_iters < 0 else a.kmeans_iters
     t0 = time.perf_counter()
@@ -436,7 +442,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16" if w.dtype == torch.bfloat16 else "f32",
-        "data": "synthetic",
+        "data": "captured keys/queries, synthetic values" if a.npz else "synthetic",
         "config": {"workload": w.name, "h_q": w.h_q, "h_kv": w.h_kv, "context": w.n,
                    "head_dim": w.d, "batch": w.batch, "levels": w.num_levels, "bf": w.bf,
                    "select_per_head": ksel, "kmeans_iters": niter},

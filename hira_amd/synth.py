@@ -129,6 +129,39 @@ def make_queries(w: Workload, keys: torch.Tensor, steps: int, seed: int = 0) -> 
     return q.to(w.dtype)
 
 
+def load_capture(path: str, w: Workload, steps: int, seed: int = 0):
+    """Keys and queries captured from a model, in the file format of the reference's sampler
+    (benchmark_area/kv_sampling/collect_kv_data.py:393-397; read by
+    benchmark_area/utils/data_loader.py:5-22): an ``.npz`` with ``keys`` (N_k, D) and
+    ``queries`` (N_q, D) fp32, heads flattened into the rows.  The pool of keys is dealt to the
+    workload's B x H_kv trees (as many keys per tree as the pool allows, at most ``w.n``), the
+    queries are drawn from the pool of queries with replacement; values stay synthetic
+    (the sampler keeps none).  Returns (workload with the key count in use, keys, values,
+    queries (steps, B, H_q, D))."""
+    import dataclasses
+
+    import numpy as np
+
+    with np.load(path) as f:  # allow_pickle stays False
+        pool_k = torch.from_numpy(np.ascontiguousarray(f["keys"], dtype=np.float32))
+        pool_q = torch.from_numpy(np.ascontiguousarray(f["queries"], dtype=np.float32))
+    if pool_k.ndim != 2 or pool_q.ndim != 2 or pool_k.shape[1] != w.d or pool_q.shape[1] != w.d:
+        raise ValueError(f"{path}: keys {tuple(pool_k.shape)} / queries {tuple(pool_q.shape)}: "
+                         f"expected (N, {w.d}) each")
+    trees = w.batch * w.h_kv
+    n = min(w.n, pool_k.shape[0] // trees)
+    if n < w.bf:
+        raise ValueError(f"{path}: {pool_k.shape[0]} keys are too few for {trees} trees")
+    g = torch.Generator().manual_seed(SEED_BASE + 1000 * w.cfg + 999 + seed)
+    order = torch.randperm(pool_k.shape[0], generator=g)[: trees * n]
+    keys = pool_k[order].reshape(w.batch, w.h_kv, n, w.d)
+    values = torch.randn((w.batch, w.h_kv, n, w.d), generator=g)
+    pick = torch.randint(0, pool_q.shape[0], (steps, w.batch, w.h_q), generator=g)
+    queries = pool_q[pick]
+    w2 = dataclasses.replace(w, name=w.name + "+capture", n=n, massive=False)
+    return w2, keys.to(w.dtype), values.to(w.dtype), queries.to(w.dtype)
+
+
 def select_fractions(w: Workload) -> torch.Tensor:
     """(B,) fraction of keys each sequence's threshold targets."""
     lo, hi = w.select_frac

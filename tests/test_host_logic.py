@@ -157,3 +157,27 @@ def test_synthetic_workloads_are_seeded_and_shaped():
     assert big[d.massive].min() > 3 * big[others].mean()  # the 8 boosted channels stand out
     fr = synth.select_fractions(synth.WORKLOADS[3])
     assert fr.shape == (16,) and 0.005 <= float(fr.min()) and float(fr.max()) <= 0.05
+
+
+def test_capture_file_in_the_reference_samplers_format(tmp_path):
+    """benchmark_area/kv_sampling/collect_kv_data.py:393-397 writes keys (N, D) and queries
+    (N, D); the loader deals them to the workload's trees, seeded."""
+    w = synth.WORKLOADS[1]
+    rng = np.random.default_rng(0)
+    path = tmp_path / "capture.npz"
+    np.savez_compressed(path, keys=rng.normal(size=(8 * 300 + 5, w.d)).astype(np.float32),
+                        queries=rng.normal(size=(100, w.d)).astype(np.float32))
+    w2, k, v, q = synth.load_capture(str(path), w, 7)
+    assert w2.n == 300 and w2.name.endswith("+capture")
+    assert k.shape == (1, 8, 300, w.d) and v.shape == k.shape and q.shape == (7, 1, 32, w.d)
+    assert k.dtype == w.dtype
+    _, k2, _, q2 = synth.load_capture(str(path), w, 7)
+    assert torch.equal(k, k2) and torch.equal(q, q2)
+    # every key of the index comes from the file, none twice
+    pool = torch.from_numpy(np.load(path)["keys"]).to(w.dtype)
+    rows = {tuple(r.tolist()) for r in k.reshape(-1, w.d)[:, :4].float()}
+    assert rows <= {tuple(r.tolist()) for r in pool[:, :4].float()} and len(rows) == 8 * 300
+    np.savez_compressed(tmp_path / "bad.npz", keys=np.zeros((10, 3), np.float32),
+                        queries=np.zeros((10, 3), np.float32))
+    with pytest.raises(ValueError):
+        synth.load_capture(str(tmp_path / "bad.npz"), w, 1)
