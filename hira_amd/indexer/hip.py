@@ -116,6 +116,10 @@ class HIPIndexer(BaseIndexer):
         self.num_heads = 0
         self.num_trees = 0
         self.num_keys = 0  # keys given to the index so far, per tree
+        # appends whose level sizes have not been read back yet (update(sync=False)): then
+        # self.size holds upper bounds and _exact_size the sizes as of the last read-back
+        self._pending = 0
+        self._exact_size: Optional[List[int]] = None
         self.dtype: Optional[torch.dtype] = None
         self.size: List[int] = []
         self.cap: List[int] = []
@@ -309,6 +313,7 @@ class HIPIndexer(BaseIndexer):
 
         if self.keys_buf is None:
             raise ValueError("Indexer is not built: nothing to save.")
+        self.sync_sizes()
         rows = [(-(-s // 16) * 16 if self.tiled else s) for s in self.size]
         tensors = {"keys": self.keys_buf[:, : rows[0]], "perm": self.perm[:, : rows[0]]}
         if self.values_buf is not None:
@@ -423,11 +428,14 @@ class HIPIndexer(BaseIndexer):
         bf, nl = self.branching_factor, self.num_levels
         if nl == 1:
             return [self.num_keys + m]
+        # (new nodes appear only once every node of a level is full, so the bound holds for
+        # the total of several calls: count from the last sizes that were read back)
+        base = self._exact_size if self._pending else self.size
         need = [0] * nl
-        new = m
+        new = m + self._pending
         for l in range(1, nl):
             new = -(-new // bf) + 1
-            need[l] = self.size[l] + new
+            need[l] = base[l] + new
         for l in range(nl - 2, -1, -1):
             need[l] = max(need[l], need[l + 1] * bf)
         return need
@@ -460,10 +468,80 @@ class HIPIndexer(BaseIndexer):
         self._tree_struct = None
 
     @torch.no_grad()
-    def update(self, new_keys: torch.Tensor, new_values: Optional[torch.Tensor] = None):
+    def reserve(self, appends: int) -> "HIPIndexer":
+        """Room for `appends` more keys per tree, so that updates up to that many do not
+        re-allocate: device pointers (and with them captured graphs and plans) stay valid."""
+        if self.keys_buf is None:
+            raise ValueError("Indexer is not built: call build() first.")
+        self._grow(self._needed_caps(int(appends)))
+        return self
+
+    def begin_unsynced(self, appends: int) -> None:
+        """Prepare for `appends` updates whose sizes are not read back: room for all of them,
+        and level sizes fixed at their bound for the whole stretch (a launch captured now
+        stays right until ``sync_sizes``).  The caller reports what it appended through
+        ``note_unsynced``."""
+        if self.num_levels < 2:
+            raise ValueError("needs a tree of at least two levels")
+        self.sync_sizes()
+        need = self._needed_caps(int(appends))
+        self._grow(need)
+        if self._state is None:
+            self._init_state()
+        self._exact_size = list(self.size)
+        self.size = [need[1] * self.branching_factor] + list(need[1:])
+        self._unsynced_room = int(appends)
+        self._tree_struct = None
+
+    def note_unsynced(self, m: int) -> None:
+        """`m` keys per tree were appended by a launch outside ``update`` (a graph replay)."""
+        if m > getattr(self, "_unsynced_room", 0):
+            raise RuntimeError("more appends than begin_unsynced made room for")
+        self._unsynced_room -= m
+        self._pending += m
+        self.num_keys += m
+
+    def _init_state(self) -> None:
+        st = torch.zeros((self.num_trees, _lib.HIRA_MAX_LEVELS + 2), dtype=torch.int32)
+        for l in range(self.num_levels):
+            st[:, l] = self.size[l]
+        st[:, _lib.HIRA_MAX_LEVELS] = self.num_keys
+        self._state = st.to(self.device)
+
+    def sync_sizes(self) -> "HIPIndexer":
+        """Read the level sizes back after updates with ``sync=False`` (one small copy that
+        waits for the stream) and check that no key was dropped."""
+        if self._state is None or (self._pending == 0 and self._exact_size is None):
+            return self
+        self._adopt_state(self._state.cpu())
+        self._unsynced_room = 0
+        return self
+
+    def _adopt_state(self, st: torch.Tensor) -> None:
+        if int(st[:, _lib.HIRA_MAX_LEVELS + 1].max()) != 0:
+            raise RuntimeError("index update ran out of capacity")
+        if self.num_levels == 1:
+            self.size = [self.num_keys]
+        else:
+            size = [0] * self.num_levels
+            for l in range(1, self.num_levels):
+                size[l] = int(st[:, l].max())
+            size[0] = size[1] * self.branching_factor
+            self.size = size
+        self._pending, self._exact_size = 0, None
+        self._tree_struct = None
+
+    def update(self, new_keys: torch.Tensor, new_values: Optional[torch.Tensor] = None, *,
+               sync: bool = True):
         """Append new_keys (1, H, m, D) (and new_values (1, H, m, Dv)) in order
         (indexer/cuda.py:544-701).  One launch; afterwards the level sizes are read back
-        (one small device-to-host copy), as the next search needs them."""
+        (one small device-to-host copy), as the next search needs them.
+
+        ``sync=False`` skips the read-back: the host then carries upper bounds of the level
+        sizes (slots past a tree's real size hold nodes without children, which every search
+        prunes at once), nothing waits for the stream, and with ``reserve`` called beforehand
+        the call is a single launch on fixed pointers, fit for a captured graph.
+        ``sync_sizes`` (or the next update with ``sync=True``) brings the exact sizes back."""
         if self.keys_buf is None:
             raise ValueError("Indexer is not built: call build() first.")
         if new_keys.ndim != 4 or new_keys.shape[0] != self.batch or \
@@ -478,14 +556,14 @@ class HIPIndexer(BaseIndexer):
             raise ValueError("new_values must be aligned with new_keys")
         if m == 0:
             return self
-        self._grow(self._needed_caps(m))
+        if not sync and self.num_levels < 2:
+            raise ValueError("sync=False needs a tree of at least two levels (a one-level index "
+                             "has no node counts to tell empty key slots by)")
+        need = self._needed_caps(m)
+        self._grow(need)
         t = self.num_trees
         if self._state is None:
-            st = torch.zeros((t, _lib.HIRA_MAX_LEVELS + 2), dtype=torch.int32)
-            for l in range(self.num_levels):
-                st[:, l] = self.size[l]
-            st[:, _lib.HIRA_MAX_LEVELS] = self.num_keys
-            self._state = st.to(self.device)
+            self._init_state()
         kin = new_keys.to(device=self.device, dtype=self.dtype).reshape(t, m, self.dim).contiguous()
         vin = None
         if new_values is not None:
@@ -497,19 +575,17 @@ class HIPIndexer(BaseIndexer):
                                     None if vin is None else vin.data_ptr(), m,
                                     self._state.data_ptr(), stream)
         _lib.check(rc)
-        st = self._state.cpu()
-        if int(st[:, _lib.HIRA_MAX_LEVELS + 1].max()) != 0:
-            raise RuntimeError("index update ran out of capacity")
         self.num_keys += m
-        if self.num_levels == 1:
-            self.size = [self.num_keys]
-        else:
-            size = [0] * self.num_levels
-            for l in range(1, self.num_levels):
-                size[l] = int(st[:, l].max())
-            size[0] = size[1] * self.branching_factor
-            self.size = size
-        self._tree_struct = None
+        if sync:
+            self._adopt_state(self._state.cpu())
+            return self
+        if self._pending == 0:
+            self._exact_size = list(self.size)
+        self._pending += m
+        bound = [need[1] * self.branching_factor] + list(need[1:])
+        if bound != self.size:
+            self.size = bound
+            self._tree_struct = None
         return self
 
     @torch.no_grad()
@@ -527,6 +603,7 @@ class HIPIndexer(BaseIndexer):
         if self.num_levels < 3:
             raise ValueError("rebuild_subtree needs at least three levels")
         bf = self.branching_factor
+        self.sync_sizes()
         if not 0 <= node < self.size[2]:
             raise ValueError(f"level-2 node {node} not in 0..{self.size[2] - 1}")
         s0, n0 = node * bf * bf, node * bf

@@ -252,6 +252,7 @@ class DecodePlan:
     def __init__(self, searcher: HIPSearcher, indexer, num_q_heads: int, scaling, q_head_to_kv,
                  stats):
         self.indexer = indexer
+        self._searcher = searcher
         self.lib = _lib.lib()
         dev = indexer.device
         self.scaling = searcher._coerce_scaling(scaling, num_q_heads, dev)
@@ -329,3 +330,83 @@ class DecodePlan:
             _lib.check(rc)
         self.run(query, self.tau_buf, out, stream, queue_keys, queue_values)
         return self.tau_buf
+
+
+class StreamingStep:
+    """One decode step over a growing index as ONE captured HIP graph: append a key/value per
+    tree (``hira_update``), thresholds from a key sample (``hira_threshold``; optional),
+    search + sparse attention (``hira_search``) -- no host work between the launches and no
+    read-back.  The graph works on fixed device buffers that ``step`` fills:
+    ``new_keys`` (T, 1, D), ``new_values`` (T, 1, Dv), ``query`` (H_q, D), ``threshold`` (H_q)
+    and writes ``out`` (H_q, Dv).  It is good for ``horizon`` steps (the index reserves room for
+    that many appends and searches with level sizes fixed at their bound); ``refresh`` reads
+    the sizes back and captures anew.  The reference does the same three things per decode
+    token from Python with host synchronisation in between (cache/hira_cache.py:121-153,
+    indexer/cuda.py:544-701)."""
+
+    def __init__(self, searcher: HIPSearcher, indexer, num_q_heads: int, scaling=None, *,
+                 horizon: int = 512, samples: Optional[torch.Tensor] = None,
+                 method: str = "sample_mean_topk", k: int = 10, q_head_to_kv=None):
+        if indexer.values_buf is None:
+            raise ValueError("the index holds no values: nothing to attend to")
+        self.searcher, self.indexer = searcher, indexer
+        self.horizon = int(horizon)
+        self.samples, self.method, self.k = samples, method, int(k)
+        self._args = (num_q_heads, scaling, q_head_to_kv)
+        dev, t = indexer.device, indexer.num_trees
+        self.new_keys = torch.zeros((t, 1, indexer.dim), dtype=indexer.dtype, device=dev)
+        self.new_values = torch.zeros((t, 1, indexer.vdim), dtype=indexer.dtype, device=dev)
+        self.query = torch.zeros((num_q_heads, indexer.dim), dtype=indexer.dtype, device=dev)
+        self.threshold = torch.zeros((num_q_heads,), dtype=torch.float32, device=dev)
+        self.out = torch.zeros((num_q_heads, indexer.vdim), dtype=torch.float32, device=dev)
+        self.refresh()
+
+    def refresh(self) -> None:
+        """Exact level sizes from the device, room for another ``horizon`` appends, new capture."""
+        idx = self.indexer
+        idx.begin_unsynced(self.horizon)
+        h_q, scaling, q2kv = self._args
+        self.plan = self.searcher.plan_attention(idx, h_q, scaling=scaling, q_head_to_kv=q2kv)
+        lib, tree = _lib.lib(), idx.tree_struct()
+        stream = torch.cuda.Stream(device=idx.device)
+        stream.wait_stream(torch.cuda.current_stream(idx.device))
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(stream):
+            with torch.cuda.graph(self.graph, stream=stream):
+                _lib.check(lib.hira_update(C.byref(tree), self.new_keys.data_ptr(),
+                                           self.new_values.data_ptr(), 1, idx._state.data_ptr(),
+                                           stream.cuda_stream))
+                if self.samples is not None:
+                    self.plan.tau_buf = self.threshold
+                    self.plan.run_sampled(self.query, self.samples, self.method, self.k, self.out,
+                                          stream=stream.cuda_stream)
+                else:
+                    self.plan.run(self.query, self.threshold, self.out, stream=stream.cuda_stream)
+        torch.cuda.current_stream(idx.device).wait_stream(stream)
+        self.left = self.horizon
+
+    def step(self, new_keys: torch.Tensor, new_values: torch.Tensor, query: torch.Tensor,
+             threshold: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """new_keys / new_values: one row per tree (any shape with T*D / T*Dv elements), query
+        (H_q, D); threshold (H_q,) unless the step takes it from the key sample.  Returns
+        ``out`` (the graph's buffer: copy it before the next step if it has to survive)."""
+        if self.left == 0:
+            self.refresh()
+        self.new_keys.copy_(new_keys.reshape(self.new_keys.shape))
+        self.new_values.copy_(new_values.reshape(self.new_values.shape))
+        self.query.copy_(query.reshape(self.query.shape))
+        if self.samples is None:
+            if threshold is None:
+                raise ValueError("threshold missing (the step has no key sample to take it from)")
+            self.threshold.copy_(threshold.reshape(self.threshold.shape))
+        return self.replay()
+
+    def replay(self) -> torch.Tensor:
+        """The step on whatever the buffers hold (for callers that write new_keys, new_values,
+        query and threshold in place, e.g. as outputs of their own kernels)."""
+        if self.left == 0:
+            self.refresh()
+        self.graph.replay()
+        self.indexer.note_unsynced(1)
+        self.left -= 1
+        return self.out

@@ -291,3 +291,81 @@ def test_save_load_roundtrip(dtype, d, bf, nl, gpu_device, tmp_path):
     save_file({"x": torch.zeros(1)}, str(tmp_path / "other.safetensors"))
     with pytest.raises(ValueError):
         HIPIndexer.load(str(tmp_path / "other.safetensors"))
+
+
+@pytest.mark.parametrize("sampled", [False, True])
+def test_streaming_step_graph_matches_eager_updates(sampled, gpu_device):
+    """update + (thresholds) + search + attention captured as one graph and replayed once per
+    token == the same calls made one by one with the level sizes read back after each update;
+    afterwards both indexes hold the same tree."""
+    from hira_amd.cache import threshold_finder as tf
+    from hira_amd.indexer.hip import HIPIndexer
+    from hira_amd.searcher.hip import HIPSearcher, StreamingStep
+
+    t, h_q, d, bf, n0, steps = 2, 8, 128, 32, 4000, 70
+    keys = bf16_round(clustered_keys(t, n0 + steps, d, seed=31, clusters=40))
+    K = torch.from_numpy(keys)[None].to(torch.bfloat16).cuda()
+    a = HIPIndexer(3, 1, bf).build(K[:, :, :n0], K[:, :, :n0])
+    b = HIPIndexer(3, 1, bf).build(K[:, :, :n0], K[:, :, :n0])
+    se = HIPSearcher()
+    scale = torch.full((h_q,), d ** -0.5)
+    samples = K[0][:, ::8][:, :400].contiguous() if sampled else None
+    step = StreamingStep(se, b, h_q, scale, horizon=32, samples=samples, method="sample_mean_topk", k=6)
+    q2kv = ho.default_q2kv(h_q, t)
+    for i in range(steps):
+        if i % 10 == 0:
+            print(f"token {i}", flush=True)
+        nk = K[:, :, n0 + i:n0 + i + 1]
+        q = bf16_round(random_query(h_q, d, seed=500 + i))
+        qd = torch.from_numpy(q).to(torch.bfloat16).cuda()
+        a.update(nk, nk)
+        if sampled:
+            th = tf.sample_mean_topk(samples, qd, 6)
+        else:
+            s = ho.scores(keys[:, :n0 + i + 1], q, q2kv)
+            th = torch.from_numpy(midpoint_threshold(s, 60)).cuda()
+        want = se.search_attention(qd, th, a, scaling=scale)
+        got = step.step(nk, nk, qd, None if sampled else th)
+        assert rel_err(got.cpu().numpy(), want.cpu().numpy()) <= 1e-5, i
+        assert b.num_keys == a.num_keys
+    assert step.left == 32 * 3 - steps          # two refreshes on the way
+    b.sync_sizes()
+    assert a.size == b.size
+    s0 = a.size[0]
+    assert torch.equal(a.perm[:, :s0], b.perm[:, :s0])
+    for l in (1, 2):
+        assert torch.equal(a.counts[l][:, : a.size[l]], b.counts[l][:, : a.size[l]])
+        assert torch.equal(a.radii[l][:, : a.size[l]], b.radii[l][:, : a.size[l]])
+    _check_tree(b, keys, keys)
+
+
+def test_unsynced_updates_keep_search_exact(gpu_device):
+    """update(sync=False): the host only knows bounds of the level sizes, the search result is
+    the same; sync_sizes brings the exact sizes back."""
+    from hira_amd.indexer.hip import HIPIndexer
+    from hira_amd.searcher.hip import HIPSearcher
+
+    t, d, bf, n0 = 2, 64, 16, 1000
+    chunks = [1, 1, 40, 1, 300, 7]
+    n = n0 + sum(chunks)
+    keys = clustered_keys(t, n, d, seed=77, clusters=25)
+    K = torch.from_numpy(keys)[None]
+    a = HIPIndexer(3, 1, bf).build(K[:, :, :n0])
+    b = HIPIndexer(3, 1, bf).build(K[:, :, :n0])
+    se = HIPSearcher(index_space="position")
+    q = random_query(2 * t, d, seed=9)
+    q2kv = ho.default_q2kv(2 * t, t)
+    at = n0
+    for m in chunks:
+        a.update(K[:, :, at:at + m])
+        b.update(K[:, :, at:at + m], sync=False)
+        at += m
+        assert b.num_keys == a.num_keys and all(x >= y for x, y in zip(b.size, a.size))
+        s = ho.scores(keys[:, :at], q, q2kv)
+        th = midpoint_threshold(s, at // 25)
+        out = se.search(torch.from_numpy(q), torch.from_numpy(th), b)
+        assert_same_selection(out.cpu().numpy()[:, :at] != 0, s, th)
+    b.sync_sizes()
+    assert b.size == a.size
+    with pytest.raises(ValueError):
+        HIPIndexer(1, 1, bf).build(K[:, :, :n0]).update(K[:, :, n0:n0 + 1], sync=False)
