@@ -65,9 +65,12 @@ def measured_traffic(workload_name):
         return None
 
 
-def cpu_baseline(w, index, queries, taus, scale, budget_s=20.0):
-    """Reference CPU search (+ host softmax-V) on the same tree, first steps of the same
-    queries, for about `budget_s` seconds of CPU work."""
+def cpu_baseline(w, index, queries, taus, scale, budget_s=20.0, gpu_out=None, gpu_sel=None):
+    """Reference CPU search (+ host softmax-V) on the same trees, first steps of the same
+    queries, for about `budget_s` seconds of CPU work; one sequence after the other when the
+    workload holds several.  With the GPU's results for the same steps (`gpu_out` (steps,
+    B*H_q, Dv) attention outputs, `gpu_sel(i)` -> (B*H_q, N_slots) bool selection of step i) the
+    two are compared on the way: selected sets outside a 1e-5 |tau| band, attention outputs."""
     import numpy as np
     import torch
     from oracle import hira_oracle as ho
@@ -76,19 +79,12 @@ def cpu_baseline(w, index, queries, taus, scale, budget_s=20.0):
     threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")), w.h_q)
     torch.set_num_threads(threads)
     n0 = index.size[0]
-    ff = ho.FixedFanoutTree(
-        bf=index.branching_factor,
-        keys=index.keys_rowmajor().float().cpu().numpy(),
-        perm=index.perm[:, :n0].cpu().numpy().astype(np.int64),
-        centers=[None] + [index.centers_rowmajor(l).float().cpu().numpy()
-                          for l in range(1, index.num_levels)],
-        radii=[None] + [index.radii[l][:, : index.size[l]].cpu().numpy()
-                        for l in range(1, index.num_levels)],
-        counts=[None] + [index.counts[l][:, : index.size[l]].cpu().numpy()
-                         for l in range(1, index.num_levels)],
-        sizes=list(index.size))
-    vals = index.values_buf[:, :n0].float().cpu().numpy()
-    tree, csr = ho.fixed_fanout_as_cpu_tree(ff)
+    keys_all = index.keys_rowmajor().float().cpu().numpy()
+    perm_all = index.perm[:, :n0].cpu().numpy().astype(np.int64)
+    cen_all = [None] + [index.centers_rowmajor(l).float().cpu().numpy() for l in range(1, index.num_levels)]
+    rad_all = [None] + [index.radii[l][:, : index.size[l]].cpu().numpy() for l in range(1, index.num_levels)]
+    cnt_all = [None] + [index.counts[l][:, : index.size[l]].cpu().numpy() for l in range(1, index.num_levels)]
+    vals_all = index.values_buf[:, :n0].float().cpu().numpy()
     ref = None
     try:
         ref = load_ref("hira_ref_v3")
@@ -96,52 +92,103 @@ def cpu_baseline(w, index, queries, taus, scale, budget_s=20.0):
         log(f"[cpu_baseline] compiled reference not loadable ({ex}); timing the C port")
     q2kv = ho.default_q2kv(w.h_q, w.h_kv)
     T = torch.from_numpy
-    if ref is not None:
-        os.environ["OMP_NUM_THREADS"] = str(threads)
-        args_tree = ([T(l.ball_centers) for l in tree.levels], [T(l.ball_radii) for l in tree.levels],
-                     [T(l.child2parent) if l.child2parent is not None
-                      else torch.empty(0, dtype=torch.long) for l in tree.levels],
-                     [l.size for l in tree.levels], [T(o) for o in csr[0]], [T(c) for c in csr[1]])
-        keys_t = T(ff.keys)
-
-    def one_step(i):
-        q = queries[i].float().cpu().numpy().reshape(w.h_q, w.d)
-        th = taus[i].cpu().numpy().reshape(w.h_q)
-        qn = np.linalg.norm(q, axis=1).astype(np.float32)
-        sc = np.full(w.h_q, scale, np.float32)
-        t0 = time.perf_counter()
+    seqs = []
+    for b in range(w.batch):
+        hs = slice(b * w.h_kv, (b + 1) * w.h_kv)
+        pick = lambda arr: [None] + [a[hs] for a in arr[1:]]  # noqa: E731
+        ff = ho.FixedFanoutTree(bf=index.branching_factor, keys=keys_all[hs], perm=perm_all[hs],
+                                centers=pick(cen_all), radii=pick(rad_all), counts=pick(cnt_all),
+                                sizes=list(index.size))
+        tree, csr = ho.fixed_fanout_as_cpu_tree(ff)
+        args_tree = None
         if ref is not None:
-            # unit-norm query, threshold and scaling rescaled: the same set, the bound the
-            # reference assumes (searcher/cpu.py:61-63)
-            out = ref.fused_tree_search_v3(keys_t, T(q / qn[:, None]), T(th / qn), *args_tree,
-                                           T(q2kv), T(sc * qn)).numpy()
-        else:
-            out = ho.search_v3(tree, q, th, sc, rscale=qn, q2kv=q2kv, csr=csr, fast=True,
-                               num_threads=threads)
-        # host attention over the selected keys, fp32
-        o = np.zeros((w.h_q, w.d), np.float32)
-        for h in range(w.h_q):
-            idx = np.nonzero(out[h])[0]
-            if idx.size:
-                z = out[h, idx]
-                p = np.exp(z - z.max())
-                o[h] = (p[:, None] * vals[q2kv[h], idx]).sum(0) / p.sum()
-        return time.perf_counter() - t0, out, o
+            args_tree = ([T(l.ball_centers) for l in tree.levels], [T(l.ball_radii) for l in tree.levels],
+                         [T(l.child2parent) if l.child2parent is not None
+                          else torch.empty(0, dtype=torch.long) for l in tree.levels],
+                         [l.size for l in tree.levels], [T(o) for o in csr[0]], [T(c) for c in csr[1]])
+        seqs.append((ff, tree, csr, args_tree, T(ff.keys), vals_all[hs]))
 
-    one_step(0)  # warm-up
-    times = []
+    def one_step(i, nthreads):
+        if ref is not None:
+            os.environ["OMP_NUM_THREADS"] = str(nthreads)
+            torch.set_num_threads(nthreads)
+        qa = queries[i].float().cpu().numpy().reshape(w.batch, w.h_q, w.d)
+        tha = taus[i].cpu().numpy().reshape(w.batch, w.h_q)
+        sc = np.full(w.h_q, scale, np.float32)
+        outs, os_ = [], []
+        t0 = time.perf_counter()
+        for b, (ff, tree, csr, args_tree, keys_t, vals) in enumerate(seqs):
+            q, th = qa[b], tha[b]
+            qn = np.linalg.norm(q, axis=1).astype(np.float32)
+            if ref is not None:
+                # unit-norm query, threshold and scaling rescaled: the same set, the bound the
+                # reference assumes (searcher/cpu.py:61-63)
+                out = ref.fused_tree_search_v3(keys_t, T(q / qn[:, None]), T(th / qn), *args_tree,
+                                               T(q2kv), T(sc * qn)).numpy()
+            else:
+                out = ho.search_v3(tree, q, th, sc, rscale=qn, q2kv=q2kv, csr=csr, fast=True,
+                                   num_threads=nthreads)
+            # host attention over the selected keys, fp32
+            o = np.zeros((w.h_q, w.d), np.float32)
+            for h in range(w.h_q):
+                idx = np.nonzero(out[h])[0]
+                if idx.size:
+                    z = out[h, idx]
+                    p = np.exp(z - z.max())
+                    o[h] = (p[:, None] * vals[q2kv[h], idx]).sum(0) / p.sum()
+            outs.append(out)
+            os_.append(o)
+        return time.perf_counter() - t0, np.concatenate(outs), np.concatenate(os_)
+
+    one_step(0, threads)  # warm-up
+    times, times1 = [], []
+    attn_err, set_diff, band_flips, compared = 0.0, 0, 0, 0
     t_start = time.perf_counter()
     i = 0
-    while i < len(queries) and (time.perf_counter() - t_start) < budget_s:
-        dt, _, _ = one_step(i)
+    while i < len(queries) and (time.perf_counter() - t_start) < budget_s * 0.75:
+        dt, out, o = one_step(i, threads)
         times.append(dt)
+        if gpu_out is not None:
+            # the sets first: only scores within rounding of tau may be decided differently;
+            # the heads where that happened are left out of the comparison of the outputs
+            same_set = np.ones(w.batch * w.h_q, bool)
+            if gpu_sel is not None:
+                tha = taus[i].cpu().numpy().reshape(-1)
+                qa = queries[i].float().cpu().numpy().reshape(-1, w.d)
+                kv = np.repeat(np.arange(w.batch * w.h_kv), w.h_q // w.h_kv)
+                diff = (out != 0) != gpu_sel(i)
+                for h, j in zip(*np.nonzero(diff)):
+                    same_set[h] = False
+                    sco = float(keys_all[kv[h], j] @ qa[h])
+                    if abs(sco - tha[h]) > 1e-5 * abs(tha[h]):
+                        set_diff += 1
+                    else:
+                        band_flips += 1
+            g = gpu_out[i].float().cpu().numpy()
+            den = np.abs(o).max(axis=1, keepdims=True) + 1e-30
+            err = (np.abs(g - o) / den).max(axis=1)
+            if same_set.any():
+                attn_err = max(attn_err, float(err[same_set].max()))
+            compared += 1
         i += 1
-    times = np.array(times)
-    return dict(value=float(np.median(times) * 1e6), unit="us/layer", cores=threads,
-                kind="reference" if ref is not None else "port",
-                sample=f"first {len(times)} of the timed decode steps (same tree, queries, "
-                       f"thresholds); median; p99 {float(np.percentile(times, 99) * 1e6):.0f} us; "
-                       f"search = reference v3 C++ kernel, attention = numpy fp32")
+    t_start = time.perf_counter()
+    j = 0
+    while j < len(queries) and (time.perf_counter() - t_start) < budget_s * 0.25:
+        dt, _, _ = one_step(j, 1)
+        times1.append(dt)
+        j += 1
+    times, times1 = np.array(times), np.array(times1)
+    res = dict(value=float(np.median(times) * 1e6), unit="us/layer", cores=threads,
+               kind="reference" if ref is not None else "port",
+               sample=f"first {len(times)} of the timed decode steps (same trees, queries, "
+                      f"thresholds); median; p99 {float(np.percentile(times, 99) * 1e6):.0f} us; "
+                      f"search = reference v3 C++ kernel, attention = numpy fp32",
+               one_thread_us=float(np.median(times1) * 1e6), one_thread_steps=len(times1))
+    if gpu_out is not None:
+        res["gpu_vs_cpu"] = {"steps_compared": compared, "attn_max_rel_err": attn_err,
+                             "selected_set_mismatches": set_diff if gpu_sel is not None else None,
+                             "decided_differently_within_1e-5_of_tau": band_flips}
+    return res
 
 
 def searcher_of(plan):
@@ -492,8 +539,13 @@ def main():
         result["streaming"] = streaming(a, w, index, plan, q_d, taus, scratch, dev)
     if not a.no_cpu:
         try:
-            result["cpu_baseline"] = cpu_baseline(w, index, q_d[W:], taus[W:], scale,
-                                                  a.cpu_budget)
+            if a.stream > 0:  # the index has grown since the timed steps: timing only
+                result["cpu_baseline"] = cpu_baseline(w, index, q_d[W:], taus[W:], scale, a.cpu_budget)
+            else:
+                dense_searcher = HIPSearcher()
+                result["cpu_baseline"] = cpu_baseline(
+                    w, index, q_d[W:], taus[W:], scale, a.cpu_budget, gpu_out=outs[W:],
+                    gpu_sel=lambda i: (dense_searcher.search(q_d[W + i], taus[W + i], index) != 0).cpu().numpy())
         except Exception as ex:  # noqa: BLE001
             log(f"[bench] cpu baseline failed: {ex!r}")
             result["cpu_baseline"] = None
