@@ -116,10 +116,37 @@ class HiraCacheLayer(CacheLayerMixin):
         if kw.get("method") not in ("sample_max", "sample_mean_topk") or kw.get("sample_size", 0) <= 0:
             return
         n = key_states.shape[-2]
-        s = min(int(kw["sample_size"]), n, 4096)
-        pick = torch.randperm(n, generator=torch.Generator().manual_seed(12345))[:s].sort().values
+        self._sample_target = min(int(kw["sample_size"]), 4096)
+        s = min(self._sample_target, n)
+        self._sample_gen = torch.Generator().manual_seed(12345)
+        pick = torch.randperm(n, generator=self._sample_gen)[:s].sort().values
         k4 = key_states if key_states.ndim == 4 else key_states[None]
         self.samples = k4[:, :, pick.to(k4.device)].reshape(-1, s, self.dim).contiguous()
+
+    def _refresh_samples(self, new_keys, seen: int):
+        """Keep the sample uniform over all indexed keys as the index grows (reservoir
+        sampling, the same positions for every head): key number i (0-based) of the sequence
+        joins with probability S/(i+1) in place of a random member; while the sample is still
+        smaller than S every new key joins."""
+        if self.samples is None:
+            return
+        k4 = new_keys if new_keys.ndim == 4 else new_keys[None]
+        m = k4.shape[-2]
+        rows = k4.reshape(-1, m, self.dim).to(self.samples.dtype)
+        room = self._sample_target - self.samples.shape[1]
+        if room > 0:  # a short prompt: the sample holds every key so far
+            take = min(room, m)
+            self.samples = torch.cat([self.samples, rows[:, :take]], dim=1).contiguous()
+            rows, seen, m = rows[:, take:], seen + take, m - take
+            if m == 0:
+                return
+        s = self.samples.shape[1]
+        idx = seen + torch.arange(m)
+        join = torch.rand(m, generator=self._sample_gen) < s / (idx + 1).double()
+        if bool(join.any()):
+            who = join.nonzero().squeeze(1)
+            slots = torch.randint(0, s, (who.numel(),), generator=self._sample_gen)
+            self.samples[:, slots.to(self.samples.device)] = rows[:, who.to(rows.device)]
 
     def _output(self, prefill_keys=None, prefill_values=None):
         kw = self.threshold_kwargs
@@ -138,6 +165,7 @@ class HiraCacheLayer(CacheLayerMixin):
 
     def update_index(self):
         self.indexer.update(self.queued_keys, self.queued_values)
+        self._refresh_samples(self.queued_keys, self.indexed_len)
         self.queued_keys = self._empty_queue()
         self.queued_values = self._empty_queue()
         self.indexed_len += self.queued_len

@@ -108,3 +108,23 @@ def test_cache_layer_count_derivation(patched):
     assert none is None and isinstance(out, hc.CacheOutput)
     assert c.layers[1].get_seq_length() == 5 and c.layers[0].get_seq_length() == 0
     assert c.layers[0].update_every == 2
+
+
+def test_key_sample_follows_the_index(patched):
+    """The sample for the threshold rules: taken from the prompt, then kept uniform over the
+    indexed keys as queued keys are flushed into the index (never a key that is still queued)."""
+    l = hc.HiraCacheLayer(DeviceMode.CUDA_ONLY, 4, {}, {},
+                          {"method": "sample_mean_topk", "sample_size": 16, "topk": 3})
+    d = 8
+    allk = torch.arange(2 * 400, dtype=torch.float32).reshape(1, 2, 400, 1).repeat(1, 1, 1, d)
+    out, _ = l.update(allk[:, :, :10], allk[:, :, :10])       # prompt shorter than the sample
+    assert out.samples.shape == (2, 10, d) and out.threshold_topk == 3
+    for i in range(10, 400):
+        out, _ = l.update(allk[:, :, i:i + 1], allk[:, :, i:i + 1])
+        ids = out.samples[0, :, 0].long()
+        assert out.samples.shape[1] == min(16, l.indexed_len)
+        assert int(ids.max()) < l.indexed_len                   # nothing from the queue
+        assert len(set(ids.tolist())) == ids.numel()            # no key twice
+        assert torch.equal(out.samples[1, :, 0].long() - 400, ids)  # same positions per head
+    assert int((ids >= 200).sum()) >= 3 and int((ids < 200).sum()) >= 3  # old and new keys
+    assert hc.HiraCacheLayer(DeviceMode.CUDA_ONLY, 4, {}, {}).update(allk, allk)[0].samples is None
