@@ -287,6 +287,9 @@ def main():
                     help="after the timed steps: append this many keys one per step, a search "
                          "after each, one level-2 subtree rebuilt every --rebuild-every steps")
     ap.add_argument("--rebuild-every", type=int, default=512)
+    ap.add_argument("--context", type=int, default=0,
+                    help="keys per KV head instead of the configuration's (a sweep point, not a "
+                         "benchmark configuration)")
     ap.add_argument("--npz", default=None,
                     help="keys and queries captured from a model (the reference sampler's .npz: "
                          "keys (N,D), queries (N,D)) instead of the synthetic ones")
@@ -311,6 +314,10 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     dev = torch.device("cuda:0")
     w = synth.WORKLOADS[a.config]
+    if a.context > 0:
+        import dataclasses
+
+        w = dataclasses.replace(w, n=a.context, name=f"{w.name}@ctx{a.context}")
     K, W = a.steps, a.warmup
     total = K + W
     log(f"[bench] workload {w.name}: generating keys/values/queries on the host")
