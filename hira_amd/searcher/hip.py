@@ -25,6 +25,17 @@ from .base import BaseSearcher
 DEFAULT_OUTPUT_FILL_VALUE = 0.0
 
 
+def _on(t: torch.Tensor, device) -> bool:
+    """Is tensor `t` on `device`?  ("cuda" without an index means the current device, which a
+    tensor's own device always spells out.)"""
+    device = torch.device(device)
+    if t.device.type != device.type:
+        return False
+    if device.index is None:
+        return device.type != "cuda" or t.device.index == torch.cuda.current_device()
+    return t.device.index == device.index
+
+
 class HIPSearcher(BaseSearcher):
     def __init__(self, block_c=None, output_fill_value: float = DEFAULT_OUTPUT_FILL_VALUE,
                  *, index_space: str = "slot", block_threads: int = 0, nodes_per_wave: int = 0,
@@ -140,7 +151,7 @@ class HIPSearcher(BaseSearcher):
 
     def _get_workspace(self, nbytes: int, device) -> torch.Tensor:
         if self._workspace is None or self._workspace.numel() < nbytes or \
-                self._workspace.device != device:
+                not _on(self._workspace, device):
             # zero once: the arrival counters inside must start at zero and are left at
             # zero by every call
             self._workspace = torch.zeros(max(nbytes, 1), dtype=torch.uint8, device=device)
@@ -148,7 +159,7 @@ class HIPSearcher(BaseSearcher):
 
     def _prepare_output_buffer(self, h_q: int, n: int, device) -> torch.Tensor:
         """searcher/cuda.py:35-54."""
-        if self._tmp_out is None or self._tmp_out.device != device or \
+        if self._tmp_out is None or not _on(self._tmp_out, device) or \
                 tuple(self._tmp_out.shape) != (h_q, n):
             self._tmp_out = torch.full((h_q, n), self.output_fill_value, device=device,
                                        dtype=torch.float32)
@@ -198,7 +209,7 @@ class HIPSearcher(BaseSearcher):
         qs, keep = self._query_struct(query, threshold, indexer, q_head_to_kv, scaling)
         cap = int(capacity or indexer.size[0])
         h_q, dev = qs.num_q_heads, indexer.device
-        if self._sel is None or self._sel[0].shape != (h_q, cap) or self._sel[0].device != dev:
+        if self._sel is None or self._sel[0].shape != (h_q, cap) or not _on(self._sel[0], dev):
             self._sel = (torch.empty((h_q, cap), dtype=torch.int32, device=dev),
                          torch.empty((h_q, cap), dtype=torch.float32, device=dev),
                          torch.zeros((h_q,), dtype=torch.int32, device=dev))
@@ -219,6 +230,8 @@ class HIPSearcher(BaseSearcher):
                          stats: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Fused search + softmax(scaling * q.K_S^T) V_S over the selected keys and, when
         given, every queued key (T, m, D) / value (T, m, Dv).  Returns (H_q, Dv) fp32."""
+        if indexer.values_buf is None:
+            raise ValueError("the index was built without values: nothing to attend to")
         qs, keep = self._query_struct(query, threshold, indexer, q_head_to_kv, scaling)
         h_q, dev = qs.num_q_heads, indexer.device
         if out is None:
@@ -251,6 +264,8 @@ class DecodePlan:
 
     def __init__(self, searcher: HIPSearcher, indexer, num_q_heads: int, scaling, q_head_to_kv,
                  stats):
+        if indexer.values_buf is None:
+            raise ValueError("the index was built without values: nothing to attend to")
         self.indexer = indexer
         self._searcher = searcher
         self.lib = _lib.lib()

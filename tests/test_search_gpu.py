@@ -309,3 +309,35 @@ def test_bad_inputs_raise_value_error(gpu_device):
         se.search(q, torch.from_numpy(c["th"]), c["idx"], scaling=torch.ones(5))
     with pytest.raises(ValueError):
         se.search(torch.zeros(3, 64), torch.zeros(3), c["idx"])         # 3 heads over 2 trees
+
+
+def test_wrapper_contract_of_the_reference_searcher(gpu_device):
+    """tests/test_triton_kernels.py:152-199 (2-D and 4-D queries agree), :283-332 (scaling
+    scales the scores and leaves the mask alone), searcher/cuda.py:35-54 (a persistent output
+    buffer, pre-filled with output_fill_value), tests/test_cuda_pipeline.py:517-523 (no values
+    given: none kept) of the reference."""
+    from hira_amd.indexer.hip import HIPIndexer
+    from hira_amd.searcher.hip import HIPSearcher
+
+    h_kv, h_q, n, d = 2, 4, 700, 64
+    keys = clustered_keys(h_kv, n, d, seed=12, clusters=20)
+    q = random_query(h_q, d, seed=13)
+    K = torch.from_numpy(keys)[None]
+    idx = HIPIndexer(3, 1, 8).build(K)
+    assert idx.values is None and idx.values_buf is None
+    s = ho.scores(keys, q, ho.default_q2kv(h_q, h_kv))
+    th = torch.from_numpy(midpoint_threshold(s, 35))
+    q2, q4 = torch.from_numpy(q), torch.from_numpy(q).view(1, h_q, 1, d)
+    se = HIPSearcher(block_c=8, output_fill_value=-7.0)
+    a = se.search(q2, th, idx).clone()
+    b = se.search(q4, th, idx)
+    assert torch.equal(a, b)
+    assert b.data_ptr() == se.search(q2, th, idx).data_ptr()       # the same buffer every call
+    sel = a != -7.0
+    assert int(sel.sum()) == h_q * 35 and float(a[~sel].abs().max()) == 7.0
+    sc = torch.tensor([2.0, 0.5, 1.0, 3.0])
+    c = se.search(q2, th, idx, scaling=sc).clone()
+    assert torch.equal(c != -7.0, sel)
+    assert torch.allclose(c[sel], (a * sc.cuda()[:, None])[sel], rtol=1e-6)
+    with pytest.raises(ValueError):
+        se.search_attention(q2, th, idx)                           # nothing to attend to
