@@ -16,7 +16,7 @@ LIB_PATH = CSRC / "libhira_hip.so"
 HIRA_MAX_LEVELS = 8
 HIRA_F32, HIRA_BF16 = 0, 1
 HIRA_ROW_MAJOR, HIRA_TILE16 = 0, 1
-HIRA_ABI_VERSION = 2
+HIRA_ABI_VERSION = 3
 
 _vp = C.c_void_p
 
@@ -102,6 +102,10 @@ SYMBOLS = {
          C.c_size_t, _vp],
     ),
     "hira_update": (C.c_int, [C.POINTER(HiraTree), _vp, _vp, C.c_int32, _vp, _vp]),
+    "hira_sparse_attention": (
+        C.c_int,
+        [C.POINTER(HiraTree), C.POINTER(HiraQuery), _vp, _vp, _vp, C.c_int32, _vp, _vp],
+    ),
     "hira_threshold": (
         C.c_int,
         [_vp, C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.POINTER(HiraQuery), C.c_int32,

@@ -223,6 +223,35 @@ class HIPSearcher(BaseSearcher):
         del keep
         return idx, score, count
 
+    def sparse_attention(self, index: torch.Tensor, score: torch.Tensor, count: torch.Tensor,
+                         indexer, q_head_to_kv=None, scaling=None,
+                         out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """softmax(scaling * score) V over given lists (``search_compact`` in the slot index
+        space, possibly edited): index (H_q, cap) int32 key slots, score (H_q, cap) fp32 raw
+        q.k, count (H_q,) int32.  Returns (H_q, Dv) fp32; zeros where a list is empty."""
+        if indexer.values_buf is None:
+            raise ValueError("the index was built without values: nothing to attend to")
+        if index.ndim != 2 or index.shape != score.shape or count.shape != (index.shape[0],):
+            raise ValueError(f"lists must be (H_q, cap), (H_q, cap), (H_q,): got "
+                             f"{tuple(index.shape)}, {tuple(score.shape)}, {tuple(count.shape)}")
+        h_q, cap = index.shape
+        dev = indexer.device
+        index = index.to(device=dev, dtype=torch.int32).contiguous()
+        score = score.to(device=dev, dtype=torch.float32).contiguous()
+        count = count.to(device=dev, dtype=torch.int32).contiguous()
+        sc = self._coerce_scaling(scaling, h_q, dev)
+        off, heads, gmax, group = self._head_map(h_q, indexer, q_head_to_kv)
+        qs = _lib.HiraQuery(h_q, None, None, sc.data_ptr(), off.data_ptr(), heads.data_ptr(),
+                            gmax, group)
+        if out is None:
+            out = torch.empty((h_q, indexer.vdim), dtype=torch.float32, device=dev)
+        tree = indexer.tree_struct()
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        _lib.check(_lib.lib().hira_sparse_attention(
+            C.byref(tree), C.byref(qs), index.data_ptr(), score.data_ptr(), count.data_ptr(),
+            int(cap), out.data_ptr(), stream))
+        return out
+
     def search_attention(self, query, threshold, indexer, q_head_to_kv=None, scaling=None, *,
                          queue_keys: Optional[torch.Tensor] = None,
                          queue_values: Optional[torch.Tensor] = None,

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define HIRA_ABI_VERSION 2
+#define HIRA_ABI_VERSION 3
 #define HIRA_MAX_LEVELS 8
 
 enum { HIRA_F32 = 0, HIRA_BF16 = 1 };
@@ -218,6 +218,23 @@ enum { HIRA_TAU_SAMPLE_MAX = 0, HIRA_TAU_SAMPLE_MEAN_TOPK = 1 };
 int hira_threshold(const void* samples, int32_t dtype, int32_t num_trees, int32_t num_samples,
                    int32_t dim, const HiraQuery* query, int32_t method, int32_t k,
                    float* tau_out, void* stream);
+
+/*
+ * Softmax attention over given lists of selected keys, for callers that edit the selection
+ * between search and attention (hira_search with attn_out does both in one launch):
+ *   out[h] = sum_j softmax_j(scaling[h] * sel_score[h][j]) * values[tree(h)][sel_index[h][j]]
+ * This is the attention the reference leaves unwritten (attention/hira_attention.py:1-3) over
+ * the result of its searchers (searcher/cuda.py:56-143).
+ *   tree       values, vdim, dtype, cap[0] and num_trees are read
+ *   query      num_q_heads, scaling and the head map are read
+ *   sel_*      the lists as hira_search writes them: sel_index key SLOTS (dense_by_position
+ *              = 0), sel_score raw q.k, sel_count entries per head (more than sel_cap: the
+ *              first sel_cap count); an index outside [0, cap[0]) is clamped
+ *   attn_out   (H_q, Dv) fp32; zeros for a head with an empty list
+ */
+int hira_sparse_attention(const HiraTree* tree, const HiraQuery* query, const int32_t* sel_index,
+                          const float* sel_score, const int32_t* sel_count, int32_t sel_cap,
+                          float* attn_out, void* stream);
 
 #ifdef __cplusplus
 }

@@ -341,3 +341,39 @@ def test_wrapper_contract_of_the_reference_searcher(gpu_device):
     assert torch.allclose(c[sel], (a * sc.cuda()[:, None])[sel], rtol=1e-6)
     with pytest.raises(ValueError):
         se.search_attention(q2, th, idx)                           # nothing to attend to
+
+
+@pytest.mark.parametrize("h_kv,h_q,n,d,bf,nl,dtype", [(2, 8, 2048, 128, 32, 3, torch.bfloat16),
+                                                      (1, 3, 600, 64, 8, 3, torch.float32),
+                                                      (2, 4, 500, 256, 16, 2, torch.bfloat16),
+                                                      (2, 2, 333, 16, 5, 3, torch.float32)])
+def test_attention_over_given_lists(h_kv, h_q, n, d, bf, nl, dtype, gpu_device):
+    """hira_sparse_attention on the lists search_compact returns == the fused launch == the
+    float64 oracle; on edited lists (entries dropped, one list emptied) == the oracle over what
+    is left."""
+    from hira_amd.searcher.hip import HIPSearcher
+
+    c = _setup(h_kv, h_q, n, d, bf, nl, dtype, seed=90 + n, keep=max(4, n // 20))
+    se = HIPSearcher()
+    q, th = torch.from_numpy(c["q"]), torch.from_numpy(c["th"])
+    sc = torch.full((h_q,), d ** -0.5)
+    idx, sco, cnt = se.search_compact(q, th, c["idx"])
+    got = se.sparse_attention(idx, sco, cnt, c["idx"], scaling=sc).cpu().numpy()
+    fused = se.search_attention(q, th, c["idx"], scaling=sc).cpu().numpy()
+    mask = (c["s"] >= c["th"][:, None]) & c["valid"]
+    ref = ho.attention(c["ff"].keys, c["vslot"], c["q"], sc.numpy(), mask, c["q2kv"])
+    tol = 2e-3 if dtype == torch.bfloat16 else 1e-5
+    assert rel_err(got, ref) <= tol and rel_err(got, fused) <= 1e-5
+    # edited lists: every head keeps the first half of its entries, head 0 none
+    idx2, sco2, cnt2 = idx.clone(), sco.clone(), (cnt // 2).clone()
+    cnt2[0] = 0
+    got2 = se.sparse_attention(idx2, sco2, cnt2, c["idx"], scaling=sc).cpu().numpy()
+    mask2 = np.zeros_like(mask)
+    ic, cc = idx2.cpu().numpy(), cnt2.cpu().numpy()
+    for h in range(h_q):
+        mask2[h, ic[h, : cc[h]]] = True
+    ref2 = ho.attention(c["ff"].keys, c["vslot"], c["q"], sc.numpy(), mask2, c["q2kv"])
+    assert np.all(got2[0] == 0)
+    assert rel_err(got2[1:], ref2[1:]) <= tol
+    with pytest.raises(ValueError):
+        se.sparse_attention(idx, sco[:, :-1], cnt, c["idx"], scaling=sc)
