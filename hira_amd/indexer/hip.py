@@ -88,6 +88,7 @@ class HIPIndexer(BaseIndexer):
         pack_rounds: int = 8,
         layout: str = "auto",
         device: str = "cuda",
+        graft_min: Optional[int] = None,
     ):
         if isinstance(num_levels, HIPIndexer.DEPTH):
             num_levels = num_levels.value
@@ -108,6 +109,10 @@ class HIPIndexer(BaseIndexer):
         self.layout_request = layout
         self.tiled = False  # keys / centers stored in the MFMA tile arrangement
         self.capacity = capacity  # key slots to reserve per tree (room for appends)
+        # update() calls with at least this many keys per tree build a sub-tree over the new
+        # keys and graft it at the tail instead of placing the keys one by one
+        # (default: half of what one root node holds, at least 256)
+        self.graft_min = graft_min
         self.device = torch.device(device)
 
         self.dim = 0
@@ -468,6 +473,62 @@ class HIPIndexer(BaseIndexer):
         self._tree_struct = None
 
     @torch.no_grad()
+    @torch.no_grad()
+    def _graft(self, new_keys, new_values, m: int) -> "HIPIndexer":
+        """A large window of new keys: cluster them among themselves (one ``hira_build`` over
+        all trees) and graft the resulting sub-tree at the tail of every level: new root nodes
+        after the existing ones, their descendants in the slot ranges those own.  This is the
+        shape of the reference's CPU update (indexer/cpu.py:124-190: an independent sub-tree
+        over the new keys, concatenated level by level) in the fixed-fan-out layout; placing
+        the keys one by one (the small-window path) costs a few microseconds per key and
+        tree, serially."""
+        self.sync_sizes()
+        bf, nl, t = self.branching_factor, self.num_levels, self.num_trees
+        sub = HIPIndexer(nl, self.max_iterations, bf, seed=self.seed + self.num_keys,
+                         device=str(self.device), pack_rounds=self.pack_rounds,
+                         layout="tiled" if self.tiled else "row_major", graft_min=1 << 62)
+        sub.build(new_keys.to(self.device, self.dtype),
+                  None if new_values is None else new_values.to(self.device, self.dtype))
+        if sub.tiled != self.tiled:
+            raise RuntimeError("sub-tree layout differs from the index's")
+        off = [0] * nl
+        off[nl - 1] = self.size[nl - 1]
+        for l in range(nl - 2, -1, -1):
+            off[l] = off[l + 1] * bf
+        r16 = (lambda n: -(-n // 16) * 16) if self.tiled else (lambda n: n)
+        self._grow([off[l] + r16(sub.size[l]) for l in range(nl)])
+        if self._state is None:
+            self._init_state()
+        n0 = sub.size[0]
+        # level 0 and the inner levels start at multiples of bf (of 16 where tiled): whole
+        # tiles copy as they are
+        self.keys_buf[:, off[0]:off[0] + r16(n0)] = sub.keys_buf[:, : r16(n0)]
+        if self.values_buf is not None:
+            self.values_buf[:, off[0]:off[0] + n0] = sub.values_buf[:, :n0]
+        sp = sub.perm[:, :n0]
+        self.perm[:, off[0]:off[0] + n0] = torch.where(sp >= 0, sp + self.num_keys,
+                                                       torch.full_like(sp, -1))
+        for l in range(1, nl):
+            k = sub.size[l]
+            self.radii[l][:, off[l]:off[l] + k] = sub.radii[l][:, :k]
+            self.counts[l][:, off[l]:off[l] + k] = sub.counts[l][:, :k]
+            if not self.tiled:
+                self.centers[l][:, off[l]:off[l] + k] = sub.centers[l][:, :k]
+            elif off[l] % 16 == 0:
+                self.centers[l][:, off[l]:off[l] + r16(k)] = sub.centers[l][:, : r16(k)]
+            else:  # the root level starts where the old roots end: through row-major
+                lo, hi = off[l] // 16 * 16, r16(off[l] + k)
+                rows = from_tiled(self.centers[l][:, lo:hi])
+                rows[:, off[l] - lo:off[l] - lo + k] = sub.centers_rowmajor(l)[:, :k]
+                self.centers[l][:, lo:hi] = to_tiled(rows)
+        self.size = [off[l] + sub.size[l] for l in range(nl)]
+        for l in range(1, nl):
+            self._state[:, l] = self.size[l]
+        self._state[:, _lib.HIRA_MAX_LEVELS] += m
+        self.num_keys += m
+        self._tree_struct = None
+        return self
+
     def reserve(self, appends: int) -> "HIPIndexer":
         """Room for `appends` more keys per tree, so that updates up to that many do not
         re-allocate: device pointers (and with them captured graphs and plans) stay valid."""
@@ -559,6 +620,11 @@ class HIPIndexer(BaseIndexer):
         if not sync and self.num_levels < 2:
             raise ValueError("sync=False needs a tree of at least two levels (a one-level index "
                              "has no node counts to tell empty key slots by)")
+        gmin = self.graft_min
+        if gmin is None:
+            gmin = max(256, self.branching_factor ** (self.num_levels - 1) // 2)
+        if self.num_levels >= 2 and m >= gmin and (not self.tiled or self.branching_factor % 16 == 0):
+            return self._graft(new_keys, new_values, m)
         need = self._needed_caps(m)
         self._grow(need)
         t = self.num_trees

@@ -56,6 +56,11 @@ UPDATE_CASES = [
     (3, 50, [5, 5, 100], 64, 4, 2, torch.float32),
     (2, 40, [1, 2, 3, 50], 32, 8, 1, torch.float32),                # one level: plain append
     (1, 64, [1] * 70, 128, 32, 4, torch.bfloat16),                  # tree smaller than a block
+    # large windows are clustered among themselves and grafted at the tail, small ones in between
+    (2, 3000, [600, 1, 1, 1100, 5, 2048, 3], 128, 32, 3, torch.bfloat16),
+    (2, 500, [300, 3, 700, 1], 32, 8, 3, torch.float32),
+    (1, 400, [260, 1, 1, 256], 64, 16, 2, torch.bfloat16),
+    (3, 100, [256, 2], 64, 16, 4, torch.bfloat16),                  # less than one root's worth: one by one
 ]
 
 
