@@ -262,6 +262,15 @@ def streaming(a, w, index, plan, q_d, taus, out, dev):
     res["graph_step"] = {"steps": S - 8, "us_per_step_wall": round(wall, 2),
                          "us_per_step_events": round(g0.elapsed_time(g1) * 1e3 / (S - 8), 2),
                          "keys_after": index.num_keys}
+    # the graph alone, for callers whose own kernels write the step's buffers (no copies in)
+    n2 = 256
+    step.replay()  # (may be the one that re-captures)
+    torch.cuda.synchronize()
+    h0 = time.perf_counter()
+    for _ in range(n2):
+        step.replay()
+    torch.cuda.synchronize()
+    res["graph_step"]["us_per_step_replay_only"] = round((time.perf_counter() - h0) * 1e6 / max(n2, 1), 2)
     log(f"[bench] streaming: {res}")
     return res
 
