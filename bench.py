@@ -296,6 +296,10 @@ def main():
                     help="after the timed steps: append this many keys one per step, a search "
                          "after each, one level-2 subtree rebuilt every --rebuild-every steps")
     ap.add_argument("--rebuild-every", type=int, default=512)
+    ap.add_argument("--layers", type=int, default=-1,
+                    help="also time the steps over this many copies of the index in turn "
+                         "(each with its own memory, like the layers of a model); default: 8 "
+                         "where one index fits the Infinity Cache, else none")
     ap.add_argument("--context", type=int, default=0,
                     help="keys per KV head instead of the configuration's (a sweep point, not a "
                          "benchmark configuration)")
@@ -451,6 +455,37 @@ def main():
     us_per_step = wall_ms * 1e3 / K
     kernel_us = graph_ms * 1e3 / K
 
+    # ---- the same steps over several copies of the index in turn (a model's layers each have
+    # their own): what one index alone leaves in the 256 MB Infinity Cache between steps is
+    # gone by the time its turn comes again
+    rot = None
+    if a.layers < 0:
+        one_index = 2 * keys_d.numel() * keys_d.element_size()
+        a.layers = 8 if one_index <= 256 * 1024 * 1024 else 0
+    if a.layers > 1 and not a.profile:
+        copies = [index] + [HIPIndexer(w.num_levels, niter, w.bf, device="cuda:0").build(keys_d, values_d)
+                            for _ in range(a.layers - 1)]
+        plans = [plan] + [searcher.plan_attention(c, h_all, scaling=torch.full((h_all,), scale))
+                          for c in copies[1:]]
+        outs2 = torch.empty_like(outs)
+        g3 = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(stream):
+            with torch.cuda.graph(g3, stream=stream):
+                for i in range(W, total):
+                    plans[i % a.layers].run(q_d[i], taus[i], outs2[i])
+            g3.replay()
+            stream.synchronize()
+            r0, r1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            r0.record(stream)
+            g3.replay()
+            r1.record(stream)
+            stream.synchronize()
+        same = bool(torch.equal(outs2[W:], outs[W:]))
+        rot = {"indexes": a.layers, "us_per_step": round(r0.elapsed_time(r1) * 1e3 / K, 3),
+               "bytes_of_all_indexes": int(a.layers * 2 * keys_d.numel() * keys_d.element_size()),
+               "same_outputs": same}
+        del copies, plans, g3
+
     # ---- dense comparators ------------------------------------------------------------
     dense_us = {}
     if a.profile:
@@ -544,6 +579,7 @@ def main():
                           "median": round(float(np.median(per_step)), 2),
                           "p99": round(float(np.percentile(per_step, 99)), 2)},
         "streaming_add_GBps": round(stream_gbs, 1),
+        "rotating_indexes": rot,
         "sample_threshold_us": round(thr_us, 2),
         "dense_attention_us": {k: round(v, 2) for k, v in dense_us.items()},
         "dense_attention_bytes": dense_bytes,
