@@ -191,10 +191,6 @@ def cpu_baseline(w, index, queries, taus, scale, budget_s=20.0, gpu_out=None, gp
     return res
 
 
-def searcher_of(plan):
-    return plan._searcher
-
-
 def streaming(a, w, index, plan, q_d, taus, out, dev):
     """Decode with a growing index: per step one key/value per tree is appended (one update
     launch), then one search + attention over the index as it stands; every
@@ -247,7 +243,7 @@ def streaming(a, w, index, plan, q_d, taus, out, dev):
 
     sk2, sv2 = synth.make_stream(w, S)  # (same drift again: only the timing matters here)
     sk2, sv2 = sk2.to(dev), sv2.to(dev)
-    step = StreamingStep(searcher_of(plan), index, q_d.shape[1], plan.scaling, horizon=512)
+    step = StreamingStep(plan.searcher, index, q_d.shape[1], plan.scaling, horizon=512)
     for t in range(8):
         step.step(sk2[:, :, t], sv2[:, :, t], q_d[t % nq], taus[t % nq])
     torch.cuda.synchronize()

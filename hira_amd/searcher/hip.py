@@ -296,7 +296,7 @@ class DecodePlan:
         if indexer.values_buf is None:
             raise ValueError("the index was built without values: nothing to attend to")
         self.indexer = indexer
-        self._searcher = searcher
+        self.searcher = searcher
         self.lib = _lib.lib()
         dev = indexer.device
         self.scaling = searcher._coerce_scaling(scaling, num_q_heads, dev)
