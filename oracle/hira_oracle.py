@@ -10,6 +10,12 @@ Host-side helpers restate the reference's Python glue:
   fixed_fanout_tree    indexer/cuda.py:200-336, 338-538 (padded child blocks of exactly bf
                        slots per parent), with Lloyd centroids instead of sampled points
   radii_from_layout    indexer/cuda.py:114-198
+  sample_thresholds    cache/threshold_finder.py:1-14 (the two rules the reference names and
+                       leaves unwritten), float64 numpy; pinned against torch's topk / max /
+                       mean and the special cases k = 1 (the maximum) and k = all (the mean)
+
+Centroid values of the k-means against faiss (indexer/cpu.py:239-250; faiss is not installed
+and not vendored): parity unpinned; see the pinning table at the top of hira_oracle.c.
 """
 from __future__ import annotations
 
