@@ -51,6 +51,7 @@ struct SearchParams {
     int32_t gmax_state; // MFMA kernel: heads per pass its LDS state rows are sized for
     float* attn_out;    // (H_q, Dv): written by the kernel itself when `done` is set
     int32_t* done;      // (T, passes) arrival counters, zero between launches; NULL: no fold
+    int32_t fold_dvl;   // vector-ALU kernel's fold: threads per partial (four columns each)
     unsigned long long* stats;
 };
 

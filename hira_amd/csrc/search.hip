@@ -21,6 +21,60 @@ namespace hira {
 
 constexpr int kUnroll = 8;  // row loads in flight per lane while scanning a block
 
+// out[:] = sum_p 2^(m_p - M) acc_p / sum_p 2^(m_p - M) l_p over the P partials of one head, by
+// all threads of the workgroup (a multiple of 64, at least dvl).  Thread t owns four columns of
+// the output (t % dvl) for the partials p = t / dvl (mod ng).  rows: (ng, Dv + 1) floats of
+// LDS, red: one float per wave.  The partials are read with device-scope loads: they may have
+// been written by workgroups behind another L2.
+__device__ __forceinline__ void fold_partials(const float* pm, const float* pl, const float* pa,
+                                              int P, int Dv, int dvl, float* out, float* rows,
+                                              float* red) {
+    auto ld = [](const float* q) {
+        return __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    };
+    const int t = threadIdx.x, nt = blockDim.x, nw = nt >> 6;
+    float mx = -INFINITY;
+    for (int i = t; i < P; i += nt) mx = fmaxf(mx, ld(pm + i));
+    mx = wave_max(mx);
+    if ((t & 63) == 0) red[t >> 6] = mx;
+    __syncthreads();
+    float M = red[0];
+    for (int w = 1; w < nw; ++w) M = fmaxf(M, red[w]);
+    if (M == -INFINITY) {  // nothing selected for this head (uniform)
+        for (int e = t; e < Dv; e += nt) out[e] = 0.0f;
+        return;
+    }
+    const int ng = nt / dvl;
+    const int gi = t / dvl, li = t % dvl;
+    float a[4] = {0.f, 0.f, 0.f, 0.f};
+    float lsum = 0.0f;
+    const bool lane_ok = li * 4 < Dv;
+    for (int i = gi; i < P; i += ng) {
+        const float mp = ld(pm + i);
+        if (mp == -INFINITY) continue;
+        const float w = exp2f(mp - M);
+        lsum += w * ld(pl + i);
+        if (lane_ok) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) a[c] += w * ld(pa + (size_t)i * Dv + li * 4 + c);
+        }
+    }
+    float* row = rows + (size_t)gi * (Dv + 1);
+    if (lane_ok) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) row[li * 4 + c] = a[c];
+    }
+    if (li == 0) row[Dv] = lsum;
+    __syncthreads();
+    float ltot = 0.0f;
+    for (int g = 0; g < ng; ++g) ltot += rows[(size_t)g * (Dv + 1) + Dv];
+    for (int e = t; e < Dv; e += nt) {
+        float sum = 0.0f;
+        for (int g = 0; g < ng; ++g) sum += rows[(size_t)g * (Dv + 1) + e];
+        out[e] = sum / ltot;
+    }
+}
+
 template <typename T, int LPR, int GMAX>
 __global__ __launch_bounds__(256) void search_kernel(const SearchParams p) {
     constexpr int EPL = Elem<T>::kPerChunk;
@@ -317,72 +371,48 @@ __global__ __launch_bounds__(256) void search_kernel(const SearchParams p) {
         }
         const int head = p.tree_q_heads[hoff + g];
         const size_t slot = (size_t)head * p.num_parts + blockIdx.x;
-        p.part_acc[slot * Dv + e] = a;
+        // device-scope stores: written through, so that the workgroup that folds the partials
+        // (maybe behind another L2) reads them without cache-wide flushes
+        __hip_atomic_store(&p.part_acc[slot * Dv + e], a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (e == 0) {
-            p.part_m[slot] = mall;
-            p.part_l[slot] = lsum;
+            __hip_atomic_store(&p.part_m[slot], mall, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&p.part_l[slot], lsum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
+    }
+    if (p.done == nullptr) return;  // the caller folds the partials in a second launch
+
+    // ---- the last workgroup of this tree (and head pass) to arrive folds its partials ----
+    __shared__ int s_last;
+    __shared__ float s_fold_red[4];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // my stores have completed
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int* ctr = p.done + (size_t)tree * gridDim.z + blockIdx.z;
+        const int ticket = __hip_atomic_fetch_add(ctr, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = ticket == (int)gridDim.x - 1;
+        if (s_last) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    for (int g = 0; g < G; ++g) {  // uniform
+        const int head = p.tree_q_heads[hoff + g];
+        fold_partials(p.part_m + (size_t)head * p.num_parts, p.part_l + (size_t)head * p.num_parts,
+                      p.part_acc + (size_t)head * p.num_parts * Dv, p.num_parts, Dv, p.fold_dvl,
+                      p.attn_out + (size_t)head * Dv, smem, s_fold_red);
+        __syncthreads();
     }
 }
 
-// out[h] = sum_p 2^(m_p - M) acc_p / sum_p 2^(m_p - M) l_p over the P partials of head h.
-// Thread t owns a float4 of the output (t % DVL) for the partials p = t / DVL (mod NG).
+// The fold as a launch of its own: one workgroup per head.
 __global__ __launch_bounds__(256) void merge_kernel(const float* __restrict__ part_m,
                                                     const float* __restrict__ part_l,
                                                     const float* __restrict__ part_acc, int P,
                                                     int Dv, int dvl, float* __restrict__ out) {
-    __shared__ float red[256];
+    __shared__ float red[4];
     extern __shared__ float smem[];  // (NG, Dv + 1)
-    const int t = threadIdx.x;
     const int head = blockIdx.x;
-    const float* pm = part_m + (size_t)head * P;
-    const float* pl = part_l + (size_t)head * P;
-    const float* pa = part_acc + (size_t)head * P * Dv;
-
-    float mx = -INFINITY;
-    for (int i = t; i < P; i += 256) mx = fmaxf(mx, pm[i]);
-    mx = wave_max(mx);
-    if ((t & 63) == 0) red[t >> 6] = mx;
-    __syncthreads();
-    const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    if (M == -INFINITY) {  // nothing selected for this head
-        for (int e = t; e < Dv; e += 256) out[(size_t)head * Dv + e] = 0.0f;
-        return;
-    }
-    const int ng = 256 / dvl;
-    const int gi = t / dvl, li = t % dvl;
-    float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
-    float lsum = 0.0f;
-    const bool lane_ok = li * 4 < Dv;
-    for (int i = gi; i < P; i += ng) {
-        const float mp = pm[i];
-        if (mp == -INFINITY) continue;
-        const float w = exp2f(mp - M);
-        lsum += w * pl[i];
-        if (lane_ok) {
-            const float4 v = *reinterpret_cast<const float4*>(pa + (size_t)i * Dv + li * 4);
-            a.x += w * v.x;
-            a.y += w * v.y;
-            a.z += w * v.z;
-            a.w += w * v.w;
-        }
-    }
-    float* row = smem + (size_t)gi * (Dv + 1);
-    if (lane_ok) {
-        row[li * 4 + 0] = a.x;
-        row[li * 4 + 1] = a.y;
-        row[li * 4 + 2] = a.z;
-        row[li * 4 + 3] = a.w;
-    }
-    if (li == 0) row[Dv] = lsum;
-    __syncthreads();
-    float ltot = 0.0f;
-    for (int g = 0; g < ng; ++g) ltot += smem[(size_t)g * (Dv + 1) + Dv];
-    for (int e = t; e < Dv; e += 256) {
-        float s = 0.0f;
-        for (int g = 0; g < ng; ++g) s += smem[(size_t)g * (Dv + 1) + e];
-        out[(size_t)head * Dv + e] = s / ltot;
-    }
+    fold_partials(part_m + (size_t)head * P, part_l + (size_t)head * P,
+                  part_acc + (size_t)head * P * Dv, P, Dv, dvl, out + (size_t)head * Dv, smem, red);
 }
 
 // ---- host side ------------------------------------------------------------------------
@@ -508,6 +538,13 @@ static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* que
     plan->tree_blocks = (plan->num_nodes + per_block - 1) / per_block;
     plan->queue_blocks = (plan->num_queue_blocks + per_block - 1) / per_block;
     plan->smem = (size_t)(threads / 64) * plan->gmax * (lpr * epl + 2) * sizeof(float);
+    {   // the fold of the last workgroup reuses the same LDS: (ng, vdim + 1) floats
+        const int dvl = round_pow2((t->vdim + 3) / 4);
+        if (dvl > 0 && dvl <= threads) {
+            const size_t fold = (size_t)(threads / dvl) * (t->vdim + 1) * sizeof(float);
+            if (fold > plan->smem) plan->smem = fold;
+        }
+    }
     return HIRA_OK;
 }
 
@@ -649,9 +686,15 @@ extern "C" int hira_search(const HiraTree* tree, const HiraQuery* query, const H
         p.part_m = w + (size_t)query->num_q_heads * P * tree->vdim;
         p.part_l = p.part_m + (size_t)query->num_q_heads * P;
         p.attn_out = out->attn_out;
-        // the MFMA kernel folds the partials itself (the last workgroup of a tree to arrive
+        // the search kernel folds the partials itself (the last workgroup of a tree to arrive
         // does it) unless the caller asks for the second launch
-        if (plan.kernel == 2 && !(launch && launch->separate_merge))
+        p.fold_dvl = round_pow2((tree->vdim + 3) / 4);
+        // (vector-ALU kernel: its last workgroup folds the heads of its pass one after the
+        // other, which only pays for a single head with few partials; the second launch has
+        // a workgroup per head)
+        const bool can_fold = plan.kernel == 2 ||
+                              (p.fold_dvl <= plan.threads && plan.gmax == 1 && P <= 64);
+        if (can_fold && !(launch && launch->separate_merge))
             p.done = reinterpret_cast<int32_t*>(workspace);
     }
     p.group_size = query->group_size > 0 ? query->group_size : 0;
