@@ -181,3 +181,15 @@ def test_capture_file_in_the_reference_samplers_format(tmp_path):
                         queries=np.zeros((10, 3), np.float32))
     with pytest.raises(ValueError):
         synth.load_capture(str(tmp_path / "bad.npz"), w, 1)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The path is built and measured on one GPU: bench.py --gpus N > 1 says so and exits."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parents[1]
+    r = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True,
+                       text=True, timeout=120)
+    assert r.returncode == 2 and "ONE GPU" in (r.stdout + r.stderr)
