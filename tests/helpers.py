@@ -40,6 +40,15 @@ def assert_same_selection(got_mask: np.ndarray, scores: np.ndarray, th: np.ndarr
     return int(band.sum())
 
 
+def band_free_heads(scores: np.ndarray, th: np.ndarray, valid=None, rel_band: float = 1e-5) -> np.ndarray:
+    """Heads none of whose (valid) keys scores within rel_band * |th| of the threshold: only
+    for those is the selected set, and with it the attention output, fixed by the inputs."""
+    band = np.abs(scores - th[:, None]) <= rel_band * np.abs(th[:, None])
+    if valid is not None:
+        band &= valid
+    return ~band.any(axis=1)
+
+
 def clustered_keys(h: int, n: int, d: int, seed: int, clusters: int = 16,
                    spread: float = 0.15) -> np.ndarray:
     """Keys around `clusters` well-separated centres, so that ball bounds really prune."""

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from oracle import hira_oracle as ho
-from helpers import (assert_same_selection, bf16_round, clustered_keys, midpoint_threshold,
+from helpers import (assert_same_selection, band_free_heads, bf16_round, clustered_keys, midpoint_threshold,
                      normalized_keys, random_query, rel_err)
 
 pytestmark = pytest.mark.gpu
@@ -238,7 +238,9 @@ def test_fused_attention_matches_fp64_oracle(case, gpu_device):
                                          c["idx"], scaling=sc).cpu().numpy()
     mask = (c["s"] >= c["th"][:, None]) & c["valid"]
     ref = ho.attention(c["ff"].keys, c["vslot"], c["q"], sc.numpy(), mask, c["q2kv"])
-    assert rel_err(out, ref) <= tol, rel_err(out, ref)
+    ok = band_free_heads(c["s"], c["th"], c["valid"])   # (a key within rounding of tau may go either way)
+    assert ok.sum() >= max(1, h_q - 1)
+    assert rel_err(out[ok], ref[ok]) <= tol, rel_err(out[ok], ref[ok])
 
 
 def test_attention_with_queue_and_empty_selection(gpu_device):
