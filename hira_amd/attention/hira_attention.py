@@ -85,12 +85,7 @@ def hira_attention_forward(module, query, key, value, attention_mask=None, dropo
     if hira_threshold is None and not sampled:
         hira_threshold = index_thresholds(indexer, query, hira_topk or max(1, indexer.num_keys // 100))
     # one plan per (index, head count, scale): a decode step is then a single library call
-    plans = searcher.__dict__.setdefault("_decode_plans", {})
-    key_ = (id(indexer), b * h_q, float(scaling))
-    plan = plans.get(key_)
-    if plan is None or plan.indexer is not indexer:
-        scale = torch.full((b * h_q,), float(scaling), dtype=torch.float32, device=indexer.device)
-        plan = plans[key_] = searcher.plan_attention(indexer, b * h_q, scaling=scale)
+    plan = searcher.decode_plan(indexer, b * h_q, scaling)
     q2 = query.reshape(b * h_q, d).to(device=indexer.device, dtype=indexer.dtype).contiguous()
     out = torch.empty((b * h_q, indexer.vdim), dtype=torch.float32, device=indexer.device)
     qk, qv = cache.queued_keys, cache.queued_values

@@ -51,6 +51,7 @@ class HIPSearcher(BaseSearcher):
         self._tmp_out: Optional[torch.Tensor] = None
         self._map_cache = {}
         self._workspace: Optional[torch.Tensor] = None
+        self._decode_plans: dict = {}
         self._sel = None
 
     # -------------------------------------------------------------- input coercion
@@ -280,6 +281,19 @@ class HIPSearcher(BaseSearcher):
         del keep
         return out
 
+    def decode_plan(self, indexer, num_q_heads: int, scaling: float) -> "DecodePlan":
+        """The plan for (this index, head count, one softmax scale for all heads), made on
+        first use and kept: callers that come once per decode step and layer (the attention
+        function) then pay one library call per step."""
+        plans = self._decode_plans
+        key = (id(indexer), int(num_q_heads), float(scaling))
+        plan = plans.get(key)
+        if plan is None or plan.indexer is not indexer:  # (ids are reused once an index is gone)
+            scale = torch.full((num_q_heads,), float(scaling), dtype=torch.float32,
+                               device=indexer.device)
+            plan = plans[key] = self.plan_attention(indexer, num_q_heads, scaling=scale)
+        return plan
+
     def plan_attention(self, indexer, num_q_heads: int, scaling=None, q_head_to_kv=None,
                        stats: Optional[torch.Tensor] = None) -> "DecodePlan":
         """Pre-resolve everything that does not change between decode steps (head map,
@@ -309,6 +323,7 @@ class DecodePlan:
         self.launch = searcher.launch
         self.tree = indexer.tree_struct()
         self.queue = _lib.HiraQueue(1, 1, 1, 1)  # sizes only: room for a queue's partials
+        self.tau_buf: Optional[torch.Tensor] = None  # (H_q,) thresholds written by run_sampled
         self.ws_bytes = self._workspace_need()
         self.ws = torch.zeros(max(self.ws_bytes, 1), dtype=torch.uint8, device=dev)
         self._refs = (C.byref(self.tree), C.byref(self.query), C.byref(self.out),
@@ -355,7 +370,7 @@ class DecodePlan:
         """A decode step whose thresholds come from a key sample (T, S, D), tree dtype,
         contiguous: ``hira_threshold`` ("sample_max" or "sample_mean_topk" with k) writes them
         into a buffer of the plan, ``run`` follows on the same stream.  Returns that buffer."""
-        if getattr(self, "tau_buf", None) is None:
+        if self.tau_buf is None:
             self.tau_buf = torch.empty((self.query.num_q_heads,), dtype=torch.float32,
                                        device=self.indexer.device)
         if samples.ndim != 3 or samples.shape[0] != self.tree.num_trees or \
