@@ -59,3 +59,25 @@ def test_struct_layout_matches_header():
     assert ctypes.sizeof(_lib.HiraLaunch) == 16
     assert _lib.HiraQuery.max_group.offset == 48 and _lib.HiraQuery.group_size.offset == 52
     assert _lib.HiraSearchOut.attn_out.offset == 56
+
+
+def test_new_entry_points_validate_without_a_gpu():
+    """hira_threshold and hira_sparse_attention reject bad arguments before any launch."""
+    lib = _lib.lib()
+    q = _lib.HiraQuery(4, 1, None, 1, None, None, 2, 2)
+    one = ctypes.c_void_p(1)
+    # too many samples, odd row width, k out of range, heads that do not fit the trees
+    assert lib.hira_threshold(one, _lib.HIRA_F32, 2, 5000, 32, ctypes.byref(q), 0, 1, one, None) == -1
+    assert b"samples" in lib.hira_last_error()
+    assert lib.hira_threshold(one, _lib.HIRA_BF16, 2, 100, 20, ctypes.byref(q), 0, 1, one, None) == -1
+    assert lib.hira_threshold(one, _lib.HIRA_F32, 2, 100, 32, ctypes.byref(q), 1, 101, one, None) == -1
+    assert lib.hira_threshold(one, _lib.HIRA_F32, 3, 100, 32, ctypes.byref(q), 0, 1, one, None) == -1
+    assert lib.hira_threshold(None, _lib.HIRA_F32, 2, 100, 32, ctypes.byref(q), 0, 1, one, None) == -1
+    t = _lib.HiraTree()
+    t.num_trees, t.num_levels, t.bf, t.dim, t.vdim, t.dtype = 2, 2, 8, 32, 0, _lib.HIRA_F32
+    assert lib.hira_sparse_attention(ctypes.byref(t), ctypes.byref(q), one, one, one, 8, one, None) == -1
+    assert b"no values" in lib.hira_last_error()
+    t.values, t.vdim = 1, 1024   # rows of 4 KiB: too wide
+    assert lib.hira_sparse_attention(ctypes.byref(t), ctypes.byref(q), one, one, one, 8, one, None) == -1
+    t.vdim = 32
+    assert lib.hira_sparse_attention(ctypes.byref(t), ctypes.byref(q), one, one, one, 0, one, None) == -1
