@@ -473,57 +473,114 @@ class HIPIndexer(BaseIndexer):
         self._tree_struct = None
 
     @torch.no_grad()
-    @torch.no_grad()
-    def _graft(self, new_keys, new_values, m: int) -> "HIPIndexer":
-        """A large window of new keys: cluster them among themselves (one ``hira_build`` over
-        all trees) and graft the resulting sub-tree at the tail of every level: new root nodes
-        after the existing ones, their descendants in the slot ranges those own.  This is the
-        shape of the reference's CPU update (indexer/cpu.py:124-190: an independent sub-tree
-        over the new keys, concatenated level by level) in the fixed-fan-out layout; placing
-        the keys one by one (the small-window path) costs a few microseconds per key and
-        tree, serially."""
+    def _room_under_a_root(self, new_keys, m: int):
+        """Per tree, the root node nearest to the window's mean among those with free child
+        slots for a sub-tree of one level less over m keys: (roots (T,), their child counts
+        (T,)) on the host, or None when some tree has no such root (then the keys go one by
+        one, or, if there are enough of them, under new roots)."""
         self.sync_sizes()
-        bf, nl, t = self.branching_factor, self.num_levels, self.num_trees
-        sub = HIPIndexer(nl, self.max_iterations, bf, seed=self.seed + self.num_keys,
+        bf, top = self.branching_factor, self.num_levels - 1
+        nroot = self.size[top]
+        if nroot <= 0:
+            return None
+        cnt = self.counts[top][:, :nroot]
+        k = level_sizes(m, bf, top)[-1]  # nodes the sub-tree puts under the root
+        ok = (cnt > 0) & (cnt + k <= bf)
+        if not bool(ok.any(dim=1).all()):
+            return None
+        mean = new_keys.to(self.device).reshape(self.num_trees, m, self.dim).float().mean(dim=1)
+        c = self.centers_rowmajor(top)[:, :nroot].float()
+        dist = (c - mean[:, None]).norm(dim=-1).masked_fill(~ok, float("inf"))
+        roots = dist.argmin(dim=1)
+        have = cnt.gather(1, roots[:, None]).squeeze(1)
+        return roots.cpu(), have.cpu()
+
+    @torch.no_grad()
+    def _graft(self, new_keys, new_values, m: int, sub_levels: int, under) -> "HIPIndexer":
+        """A large window of new keys: cluster them among themselves (one ``hira_build`` over
+        all trees) and graft the resulting sub-tree into the tail of the index.  With
+        ``sub_levels == num_levels`` its roots become new root nodes after the existing ones;
+        with one level less (``under = (roots, child counts)``, per tree) they become further
+        children of an existing root, whose radius grows to cover them.  Either way the descendants sit in
+        the slot ranges their parents own.  This is the shape of the reference's CPU update
+        (indexer/cpu.py:124-190: an independent sub-tree over the new keys, concatenated level
+        by level) in the fixed-fan-out layout; placing the keys one by one (the small-window
+        path) costs a few microseconds per key and tree, serially."""
+        self.sync_sizes()
+        bf, nl = self.branching_factor, self.num_levels
+        sub = HIPIndexer(sub_levels, self.max_iterations, bf, seed=self.seed + self.num_keys,
                          device=str(self.device), pack_rounds=self.pack_rounds,
                          layout="tiled" if self.tiled else "row_major", graft_min=1 << 62)
         sub.build(new_keys.to(self.device, self.dtype),
                   None if new_values is None else new_values.to(self.device, self.dtype))
         if sub.tiled != self.tiled:
             raise RuntimeError("sub-tree layout differs from the index's")
-        off = [0] * nl
-        off[nl - 1] = self.size[nl - 1]
-        for l in range(nl - 2, -1, -1):
-            off[l] = off[l + 1] * bf
+        stop = sub_levels - 1  # the sub-tree's top level, as a level of the index
         r16 = (lambda n: -(-n // 16) * 16) if self.tiled else (lambda n: n)
-        self._grow([off[l] + r16(sub.size[l]) for l in range(nl)])
+        # where the sub-tree's top nodes go: after the existing roots (the same place in every
+        # tree), or after the children the chosen root already has (tree by tree)
+        if under is None:
+            groups = [(slice(None), self.size[stop])]
+        else:
+            roots, have = under
+            place = roots.long() * bf + have.long()  # (T,) first free child slot of the chosen root
+            groups = [((place == v).nonzero().squeeze(1).to(self.device), int(v))
+                      for v in torch.unique(place).tolist()]
+        offs = []
+        for _, top_off in groups:
+            off = [0] * sub_levels
+            off[stop] = top_off
+            for l in range(stop - 1, -1, -1):
+                off[l] = off[l + 1] * bf
+            offs.append(off)
+        need = list(self.size)
+        for off in offs:
+            for l in range(sub_levels):
+                need[l] = max(need[l], off[l] + r16(sub.size[l]))
+        self._grow(need)
         if self._state is None:
             self._init_state()
         n0 = sub.size[0]
-        # level 0 and the inner levels start at multiples of bf (of 16 where tiled): whole
-        # tiles copy as they are
-        self.keys_buf[:, off[0]:off[0] + r16(n0)] = sub.keys_buf[:, : r16(n0)]
-        if self.values_buf is not None:
-            self.values_buf[:, off[0]:off[0] + n0] = sub.values_buf[:, :n0]
         sp = sub.perm[:, :n0]
-        self.perm[:, off[0]:off[0] + n0] = torch.where(sp >= 0, sp + self.num_keys,
-                                                       torch.full_like(sp, -1))
+        sp = torch.where(sp >= 0, sp + self.num_keys, torch.full_like(sp, -1))
+        for (trees, _), off in zip(groups, offs):
+            # level 0 and the inner levels start at multiples of bf (of 16 where tiled): whole
+            # tiles copy as they are
+            self.keys_buf[trees, off[0]:off[0] + r16(n0)] = sub.keys_buf[trees, : r16(n0)]
+            if self.values_buf is not None:
+                self.values_buf[trees, off[0]:off[0] + n0] = sub.values_buf[trees, :n0]
+            self.perm[trees, off[0]:off[0] + n0] = sp[trees]
+            for l in range(1, sub_levels):
+                k = sub.size[l]
+                self.radii[l][trees, off[l]:off[l] + k] = sub.radii[l][trees, :k]
+                self.counts[l][trees, off[l]:off[l] + k] = sub.counts[l][trees, :k]
+                if not self.tiled:
+                    self.centers[l][trees, off[l]:off[l] + k] = sub.centers[l][trees, :k]
+                elif off[l] % 16 == 0:
+                    self.centers[l][trees, off[l]:off[l] + r16(k)] = sub.centers[l][trees, : r16(k)]
+                else:  # the top level starts where the old nodes end: through row-major
+                    lo, hi = off[l] // 16 * 16, r16(off[l] + k)
+                    rows = from_tiled(self.centers[l][trees, lo:hi])
+                    rows[:, off[l] - lo:off[l] - lo + k] = sub.centers_rowmajor(l)[trees, :k]
+                    self.centers[l][trees, lo:hi] = to_tiled(rows)
+        if under is not None:  # the roots take the sub-tree's top nodes as further children
+            k = sub.size[stop]
+            ar = torch.arange(self.num_trees, device=self.device)
+            rt = under[0].to(self.device)
+            c_root = self.centers_rowmajor(nl - 1)[ar, rt].float()
+            c_new = sub.centers_rowmajor(stop)[:, :k].float()
+            reach = ((c_new - c_root[:, None]).norm(dim=-1) + sub.radii[stop][:, :k]).max(dim=1).values
+            self.radii[nl - 1][ar, rt] = torch.maximum(self.radii[nl - 1][ar, rt], reach * (1 + 1e-6))
+            self.counts[nl - 1][ar, rt] += k
+        size = list(self.size)
+        for off in offs:
+            for l in range(sub_levels):
+                size[l] = max(size[l], off[l] + sub.size[l])
+        self.size = size
         for l in range(1, nl):
-            k = sub.size[l]
-            self.radii[l][:, off[l]:off[l] + k] = sub.radii[l][:, :k]
-            self.counts[l][:, off[l]:off[l] + k] = sub.counts[l][:, :k]
-            if not self.tiled:
-                self.centers[l][:, off[l]:off[l] + k] = sub.centers[l][:, :k]
-            elif off[l] % 16 == 0:
-                self.centers[l][:, off[l]:off[l] + r16(k)] = sub.centers[l][:, : r16(k)]
-            else:  # the root level starts where the old roots end: through row-major
-                lo, hi = off[l] // 16 * 16, r16(off[l] + k)
-                rows = from_tiled(self.centers[l][:, lo:hi])
-                rows[:, off[l] - lo:off[l] - lo + k] = sub.centers_rowmajor(l)[:, :k]
-                self.centers[l][:, lo:hi] = to_tiled(rows)
-        self.size = [off[l] + sub.size[l] for l in range(nl)]
-        for l in range(1, nl):
-            self._state[:, l] = self.size[l]
+            self._state[:, l] = torch.maximum(self._state[:, l], torch.tensor(
+                [max(off[l] + sub.size[l] for off in offs) if l < sub_levels else 0],
+                dtype=torch.int32, device=self.device))
         self._state[:, _lib.HIRA_MAX_LEVELS] += m
         self.num_keys += m
         self._tree_struct = None
@@ -620,11 +677,19 @@ class HIPIndexer(BaseIndexer):
         if not sync and self.num_levels < 2:
             raise ValueError("sync=False needs a tree of at least two levels (a one-level index "
                              "has no node counts to tell empty key slots by)")
-        gmin = self.graft_min
-        if gmin is None:
-            gmin = max(256, self.branching_factor ** (self.num_levels - 1) // 2)
-        if self.num_levels >= 2 and m >= gmin and (not self.tiled or self.branching_factor % 16 == 0):
-            return self._graft(new_keys, new_values, m)
+        if self.num_levels >= 2 and (not self.tiled or self.branching_factor % 16 == 0):
+            bf, nl = self.branching_factor, self.num_levels
+            full = self.graft_min if self.graft_min is not None else max(256, bf ** (nl - 1) // 2)
+            part = self.graft_min if self.graft_min is not None else max(256, bf ** (nl - 2) // 2)
+            if m >= full:
+                return self._graft(new_keys, new_values, m, nl, None)
+            if nl >= 3 and m >= part:
+                # a mid-size window: further children of an existing root where every tree has
+                # one with room, else a new root (whose free child slots take the next ones)
+                where = self._room_under_a_root(new_keys, m)
+                if where is not None:
+                    return self._graft(new_keys, new_values, m, nl - 1, where)
+                return self._graft(new_keys, new_values, m, nl, None)
         need = self._needed_caps(m)
         self._grow(need)
         t = self.num_trees

@@ -60,7 +60,11 @@ UPDATE_CASES = [
     (2, 3000, [600, 1, 1, 1100, 5, 2048, 3], 128, 32, 3, torch.bfloat16),
     (2, 500, [300, 3, 700, 1], 32, 8, 3, torch.float32),
     (1, 400, [260, 1, 1, 256], 64, 16, 2, torch.bfloat16),
-    (3, 100, [256, 2], 64, 16, 4, torch.bfloat16),                  # less than one root's worth: one by one
+    (3, 100, [256, 2], 64, 16, 4, torch.bfloat16),                  # fits under the only root
+    # mid-size windows become further children of the last root while it has room
+    (2, 5000, [600, 3, 300, 2100, 400, 1, 3000, 5], 64, 16, 4, torch.bfloat16),
+    (2, 3000, [300, 2, 600, 260, 1, 270, 280, 290], 128, 32, 3, torch.bfloat16),
+    (2, 900, [260, 1, 300], 32, 16, 3, torch.float32),
 ]
 
 
