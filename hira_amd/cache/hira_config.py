@@ -1,40 +1,60 @@
-"""HiraConfig / DeviceMode: the reference's cache/hira_config.py:5-46, with the two
-loaders it leaves unimplemented (from_dict / from_yaml, :27-33) filled in."""
+"""Settings of the cache and its index (the reference's cache/hira_config.py:5-46, same field
+names and defaults apart from the device mode, which is the GPU here), with validation and with
+the two loaders the reference leaves unimplemented (``from_dict`` / ``from_yaml``, :27-33).
+"""
 from __future__ import annotations
 
-from dataclasses import dataclass, fields
+import dataclasses
+from typing import Any, Dict
 
 
-@dataclass
 class DeviceMode:
+    """Where index and search run.  Only ``CUDA_ONLY`` is served by this package: PyTorch-ROCm
+    names the MI355X "cuda", and the string is what configurations of the reference carry."""
+
     CPU_ONLY = "cpu_only"
-    CUDA_ONLY = "cuda_only"  # the HIP backend: PyTorch-ROCm names the MI355X "cuda"
+    CUDA_ONLY = "cuda_only"
     CPU_CUDA = "cpu-cuda"
+    ALL = (CPU_ONLY, CUDA_ONLY, CPU_CUDA)
 
 
-@dataclass
+_THRESHOLD_METHODS = ("sample_max", "sample_mean_topk", "exact_topk", "none")
+
+
+@dataclasses.dataclass
 class HiraConfig:
-    # cache
-    device_mode: str = DeviceMode.CUDA_ONLY
-    update_every: int = 1
-    # indexers
-    num_levels: int = 5
-    max_iterations: int = 1
-    branching_factor: int = 10
-    # threshold
-    threshold_method: str = "sample_mean_topk"  # "sample_max" | "sample_mean_topk" | "exact_topk"
-    sample_size: int = 1000
-    threshold_topk: int = 10  # k of "sample_mean_topk" (the reference passes k at the call)
-    # searcher
-    chunk_size = 8 * 1024
+    device_mode: str = DeviceMode.CUDA_ONLY   # cache: which backend a layer's index lives on
+    update_every: int = 1                     # cache: queued tokens that trigger an index update
+    num_levels: int = 5                       # index: levels of the tree, keys included
+    max_iterations: int = 1                   # index: Lloyd rounds per level at build
+    branching_factor: int = 10                # index: children per node
+    threshold_method: str = "sample_mean_topk"  # thresholds: one of _THRESHOLD_METHODS
+    sample_size: int = 1000                   # thresholds: keys sampled per KV head
+    threshold_topk: int = 10                  # thresholds: k of "sample_mean_topk" (not in the
+    #                                           reference, whose stub takes k at the call)
+    chunk_size = 8 * 1024                     # host searcher only (a class attribute, as in the
+    #                                           reference: not a dataclass field)
 
+    def __post_init__(self):
+        if self.device_mode not in DeviceMode.ALL:
+            raise ValueError(f"device_mode {self.device_mode!r}: one of {DeviceMode.ALL}")
+        for name in ("update_every", "num_levels", "branching_factor", "sample_size",
+                     "threshold_topk"):
+            if int(getattr(self, name)) < 1:
+                raise ValueError(f"{name} must be at least 1, got {getattr(self, name)}")
+        if int(self.max_iterations) < 0:
+            raise ValueError(f"max_iterations must not be negative, got {self.max_iterations}")
+        if self.threshold_method not in _THRESHOLD_METHODS:
+            raise ValueError(f"threshold_method {self.threshold_method!r}: one of {_THRESHOLD_METHODS}")
+
+    # ------------------------------------------------------------------ loaders
     @classmethod
-    def from_dict(cls, config_dict: dict) -> "HiraConfig":
-        known = {f.name for f in fields(cls)}
-        unknown = set(config_dict) - known - {"chunk_size"}
-        if unknown:
-            raise ValueError(f"unknown HiraConfig keys: {sorted(unknown)}")
-        cfg = cls(**{k: v for k, v in config_dict.items() if k in known})
+    def from_dict(cls, config_dict: Dict[str, Any]) -> "HiraConfig":
+        names = {f.name for f in dataclasses.fields(cls)}
+        extra = sorted(k for k in config_dict if k not in names and k != "chunk_size")
+        if extra:
+            raise ValueError(f"unknown HiraConfig keys: {extra}")
+        cfg = cls(**{k: config_dict[k] for k in config_dict if k in names})
         if "chunk_size" in config_dict:
             cfg.chunk_size = int(config_dict["chunk_size"])
         return cfg
@@ -43,22 +63,19 @@ class HiraConfig:
     def from_yaml(cls, config_path: str) -> "HiraConfig":
         import yaml
 
-        with open(config_path, "r") as f:
-            return cls.from_dict(yaml.safe_load(f) or {})
+        with open(config_path, "r", encoding="utf-8") as handle:
+            return cls.from_dict(yaml.safe_load(handle) or {})
 
-    def get_indexer_kwargs(self) -> dict:
-        return {
-            "num_levels": self.num_levels,
-            "max_iterations": self.max_iterations,
-            "branching_factor": self.branching_factor,
-        }
+    # ------------------------------------------------------------------ what each part is built from
+    def get_indexer_kwargs(self) -> Dict[str, int]:
+        return {name: int(getattr(self, name))
+                for name in ("num_levels", "max_iterations", "branching_factor")}
 
-    def get_threshold_kwargs(self) -> dict:
+    def get_searcher_kwargs(self) -> Dict[str, int]:
+        on_gpu = self.device_mode == DeviceMode.CUDA_ONLY
+        return {"block_c": self.branching_factor} if on_gpu else {"chunk_size": self.chunk_size}
+
+    def get_threshold_kwargs(self) -> Dict[str, Any]:
         """What the cache layer needs to keep a key sample and turn it into thresholds."""
-        return {"method": self.threshold_method, "sample_size": self.sample_size,
-                "topk": self.threshold_topk}
-
-    def get_searcher_kwargs(self) -> dict:
-        if self.device_mode == DeviceMode.CUDA_ONLY:
-            return {"block_c": self.branching_factor}
-        return {"chunk_size": self.chunk_size}
+        return {"method": self.threshold_method, "sample_size": int(self.sample_size),
+                "topk": int(self.threshold_topk)}
