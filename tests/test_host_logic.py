@@ -193,3 +193,14 @@ def test_bench_refuses_more_than_one_gpu():
     r = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True,
                        text=True, timeout=120)
     assert r.returncode == 2 and "ONE GPU" in (r.stdout + r.stderr)
+
+
+def test_config_rejects_bad_settings():
+    for bad in (dict(device_mode="gpu"), dict(update_every=0), dict(num_levels=0),
+                dict(branching_factor=0), dict(max_iterations=-1), dict(threshold_method="median"),
+                dict(sample_size=0), dict(threshold_topk=0)):
+        with pytest.raises(ValueError):
+            hira_config.HiraConfig(**bad)
+    cfg = hira_config.HiraConfig(max_iterations=0, threshold_method="none")
+    assert cfg.get_indexer_kwargs() == {"num_levels": 5, "max_iterations": 0, "branching_factor": 10}
+    assert cfg.get_threshold_kwargs() == {"method": "none", "sample_size": 1000, "topk": 10}
