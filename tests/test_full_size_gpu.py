@@ -55,3 +55,57 @@ def test_size_independent_properties_at_full_size(cfg, gpu_device):
         scale=w.d ** -0.5).reshape(w.h_q, w.d)
     err = ((dense - ref).abs().max(dim=1).values / ref.abs().max(dim=1).values).max()
     assert float(err) <= 2e-3, float(err)
+
+
+def _check_tree_on_device(idx, keys_all):
+    """The structure check of the update tests, in torch on the GPU: every key present once and
+    in its slot, children packed from slot 0, every radius covers its subtree."""
+    t, n, d = keys_all.shape
+    bf, nl = idx.branching_factor, idx.num_levels
+    s0 = idx.size[0]
+    perm = idx.perm[:, :s0].long()
+    ok = perm >= 0
+    kr = idx.keys_rowmajor()[:, :s0].float()
+    for h in range(t):
+        assert torch.equal(perm[h][ok[h]].sort().values, torch.arange(n, device=perm.device))
+        assert torch.equal(kr[h][ok[h]], keys_all[h][perm[h][ok[h]]].float())
+    child_c, child_r, child_ok = kr, torch.zeros_like(kr[..., 0]), ok
+    for l in range(1, nl):
+        k = idx.size[l]
+        cen = idx.centers_rowmajor(l)[:, :k].float()
+        rad = idx.radii[l][:, :k]
+        cnt = idx.counts[l][:, :k]
+        short = k * bf - child_ok.shape[1]
+        if short > 0:
+            child_c = torch.cat([child_c, child_c.new_zeros((t, short, d))], 1)
+            child_r = torch.cat([child_r, child_r.new_zeros((t, short))], 1)
+            child_ok = torch.cat([child_ok, child_ok.new_zeros((t, short))], 1)
+        blk = child_ok[:, : k * bf].reshape(t, k, bf)
+        assert torch.equal(cnt.long(), blk.sum(-1)), f"counts of level {l}"
+        assert bool((blk[..., :-1] >= blk[..., 1:]).all()), f"children of level {l} not packed"
+        dist = (child_c[:, : k * bf].reshape(t, k, bf, d) - cen[:, :, None]).norm(dim=-1)
+        reach = torch.where(blk, dist + child_r[:, : k * bf].reshape(t, k, bf),
+                            torch.full_like(dist, float("-inf"))).max(dim=-1).values
+        has = cnt > 0
+        assert bool((rad[has] >= reach[has] * (1 - 1e-5) - 1e-5).all()), f"radius of level {l}"
+        child_c, child_r, child_ok = cen, torch.where(has, rad, torch.zeros_like(rad)), has
+
+
+def test_build_and_growth_keep_the_tree_valid_at_full_size(gpu_device):
+    """cfg 4's index (8 x 131072 keys, 4 levels): valid after the build, after a window that
+    is grafted, after single appends and after a subtree rebuild."""
+    from hira_amd import synth
+    from hira_amd.indexer import HIPIndexer
+
+    w = synth.WORKLOADS[4]
+    keys, values = synth.make_kv(w)
+    more, _ = synth.make_stream(w, 2048 + 40)
+    kd, vd, md = keys.cuda(), values.cuda(), more.cuda()
+    idx = HIPIndexer(w.num_levels, w.kmeans_iters, w.bf).build(kd, vd)
+    _check_tree_on_device(idx, kd[0])
+    idx.update(md[:, :, :2048], md[:, :, :2048])
+    for i in range(2048, 2088):
+        idx.update(md[:, :, i:i + 1], md[:, :, i:i + 1], sync=False)
+    idx.rebuild_subtree(3)
+    assert idx.num_keys == w.n + 2088
+    _check_tree_on_device(idx, torch.cat([kd[0], md[0]], dim=1))
