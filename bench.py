@@ -282,6 +282,9 @@ def main():
     ap.add_argument("--block-threads", type=int, default=0)
     ap.add_argument("--nodes-per-wave", type=int, default=0)
     ap.add_argument("--kernel", type=int, default=0)
+    ap.add_argument("--share", type=int, default=0,
+                    help="MFMA kernel: workgroups that gate the same tiles and split the survivors "
+                         "(0 = chosen by the library, 1 = no sharing)")
     ap.add_argument("--kmeans-iters", type=int, default=-1)
     ap.add_argument("--separate-merge", action="store_true",
                     help="fold the attention partials in a second launch")
@@ -360,7 +363,7 @@ def main():
             taus[i, hs] = exact_topk(keys_d[b], q_d[i, hs], ksel[b])
     scale = w.d ** -0.5
     searcher = HIPSearcher(block_threads=a.block_threads, nodes_per_wave=a.nodes_per_wave,
-                           kernel=a.kernel, separate_merge=a.separate_merge)
+                           kernel=a.kernel, separate_merge=a.separate_merge, share=a.share)
     h_all = w.batch * w.h_q
     plan = searcher.plan_attention(index, h_all, scaling=torch.full((h_all,), scale))
     outs = torch.empty((total, h_all, w.d), dtype=torch.float32, device=dev)

@@ -16,7 +16,7 @@ LIB_PATH = CSRC / "libhira_hip.so"
 HIRA_MAX_LEVELS = 8
 HIRA_F32, HIRA_BF16 = 0, 1
 HIRA_ROW_MAJOR, HIRA_TILE16 = 0, 1
-HIRA_ABI_VERSION = 3
+HIRA_ABI_VERSION = 4
 
 _vp = C.c_void_p
 
@@ -79,6 +79,7 @@ class HiraLaunch(C.Structure):
         ("nodes_per_wave", C.c_int32),
         ("kernel", C.c_int32),
         ("separate_merge", C.c_int32),
+        ("share", C.c_int32),
     ]
 
 
@@ -99,6 +100,12 @@ SYMBOLS = {
     "hira_build": (
         C.c_int,
         [C.POINTER(HiraTree), _vp, _vp, C.c_int32, C.c_int32, C.c_int32, C.c_uint64, _vp,
+         C.c_size_t, _vp],
+    ),
+    "hira_nearest_workspace_bytes": (C.c_size_t, [C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
+    "hira_nearest": (
+        C.c_int,
+        [_vp, C.c_int32, C.c_int32, C.c_int32, _vp, C.c_int32, C.c_int32, _vp, _vp, _vp, _vp,
          C.c_size_t, _vp],
     ),
     "hira_update": (C.c_int, [C.POINTER(HiraTree), _vp, _vp, C.c_int32, _vp, _vp]),

@@ -43,6 +43,27 @@ def _dense(query, key, value, attention_mask, scaling, is_causal):
     return out.transpose(1, 2).contiguous()
 
 
+def _hides_a_key(attention_mask) -> bool:
+    """Does the mask hide a key from the LAST query position?  Causal masking never does (the
+    last position sees every key before it), so what it hides there is padding.  Boolean masks:
+    True = attend; floating masks are additive (0 = attend); integer masks: 1 = attend."""
+    if attention_mask is None:
+        return False
+    last = attention_mask[..., -1, :] if attention_mask.ndim >= 3 else attention_mask
+    if last.dtype == torch.bool:
+        return bool((~last).any())
+    if last.is_floating_point():
+        return bool((last != 0).any())
+    return bool((last == 0).any())
+
+
+_PADDING_ERROR = (
+    "hira attention: the attention mask hides key positions (a padded batch). The index holds "
+    "every cached position and the sparse decode step attends to all it selects, so padded "
+    "prompts would silently attend to pad keys; run sequences of equal length per batch, or "
+    "one sequence per cache")
+
+
 def index_thresholds(indexer, query: torch.Tensor, topk: int) -> torch.Tensor:
     """(B*H_q,) thresholds that keep exactly the `topk` best indexed keys of every head."""
     keys = indexer.keys_rowmajor()  # (T, N_pad, D) slot order
@@ -69,12 +90,20 @@ def hira_attention_forward(module, query, key, value, attention_mask=None, dropo
         return _dense(query, key, value, attention_mask, scaling, True), None
     cache = key
     if cache.prefill_keys is not None:
+        if _hides_a_key(attention_mask):
+            raise ValueError(_PADDING_ERROR)
         return _dense(query, cache.prefill_keys, cache.prefill_values, attention_mask, scaling,
                       True), None
     if query.shape[2] != 1:
         raise ValueError("sparse decode expects one query position per step")
     indexer, searcher = cache.indexer, cache.searcher
     b, h_q = query.shape[0], query.shape[1]
+    # a mask that hides keys cannot be honoured by the decode step: looked at once per index
+    # (padding does not move between steps, and the look costs a host synchronisation)
+    if attention_mask is not None and not getattr(indexer, "_decode_mask_checked", False):
+        if _hides_a_key(attention_mask):
+            raise ValueError(_PADDING_ERROR)
+        indexer._decode_mask_checked = True
     if hira_threshold is None:
         hira_threshold = getattr(module, "hira_threshold", None)
     if hira_topk is None:

@@ -121,7 +121,9 @@ class HiraCacheLayer(CacheLayerMixin):
         self._sample_gen = torch.Generator().manual_seed(12345)
         pick = torch.randperm(n, generator=self._sample_gen)[:s].sort().values
         k4 = key_states if key_states.ndim == 4 else key_states[None]
-        self.samples = k4[:, :, pick.to(k4.device)].reshape(-1, s, self.dim).contiguous()
+        # (in the index's storage dtype: the threshold kernel reads samples and queries alike)
+        store = getattr(self.indexer, "dtype", None) or k4.dtype
+        self.samples = k4[:, :, pick.to(k4.device)].reshape(-1, s, self.dim).to(store).contiguous()
 
     def _refresh_samples(self, new_keys, seen: int):
         """Keep the sample uniform over all indexed keys as the index grows (reservoir
@@ -146,6 +148,11 @@ class HiraCacheLayer(CacheLayerMixin):
         if bool(join.any()):
             who = join.nonzero().squeeze(1)
             slots = torch.randint(0, s, (who.numel(),), generator=self._sample_gen)
+            # a slot drawn twice keeps its last arrival (an indexed assignment with repeated
+            # targets has no defined order)
+            last = {int(sl): int(wh) for sl, wh in zip(slots.tolist(), who.tolist())}
+            slots = torch.tensor(list(last.keys()), dtype=torch.long)
+            who = torch.tensor(list(last.values()), dtype=torch.long)
             self.samples[:, slots.to(self.samples.device)] = rows[:, who.to(rows.device)]
 
     def _output(self, prefill_keys=None, prefill_values=None):
@@ -164,7 +171,16 @@ class HiraCacheLayer(CacheLayerMixin):
         )
 
     def update_index(self):
-        self.indexer.update(self.queued_keys, self.queued_values)
+        # no read-back of the level sizes: the host carries their bounds (HIPIndexer.update,
+        # sync=False), so folding the queue into the index does not wait for the GPU; a
+        # one-level index has no node counts to bound with and keeps the synchronous form
+        import inspect
+
+        if "sync" in inspect.signature(self.indexer.update).parameters:
+            self.indexer.update(self.queued_keys, self.queued_values,
+                                sync=getattr(self.indexer, "num_levels", 1) < 2)
+        else:  # an indexer with the reference's two-argument update
+            self.indexer.update(self.queued_keys, self.queued_values)
         self._refresh_samples(self.queued_keys, self.indexed_len)
         self.queued_keys = self._empty_queue()
         self.queued_values = self._empty_queue()

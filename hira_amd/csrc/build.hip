@@ -786,3 +786,91 @@ extern "C" int hira_build(const HiraTree* tree, const void* keys_in, const void*
                ? build_impl<float>(tree, keys_in, values_in, n, niter, pack_rounds, seed, b, s)
                : build_impl<bf16_t>(tree, keys_in, values_in, n, niter, pack_rounds, seed, b, s);
 }
+
+// ---- nearest centre as a call of its own -------------------------------------------------
+namespace hira {
+
+__global__ void k_valid_to_fill(const int32_t* valid, size_t n, int32_t* fill) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) fill[i] = valid[i] != 0 ? 0 : 1;  // "full" (>= 1 of 1 slots) = not usable
+}
+
+struct NearestWs {
+    void* tiles;
+    float* n2;
+    int32_t* fill;
+    size_t total;
+};
+
+static void carve_nearest(int dtype, int T, int m, int D, bool masked, void* ws, NearestWs* b) {
+    Carver c{reinterpret_cast<char*>(ws), 0};
+    b->tiles = nullptr;
+    b->n2 = nullptr;
+    if (dtype == HIRA_BF16 && (D == 64 || D == 128 || D == 256)) {
+        const size_t kpad = (size_t)assign_tiles(m) * 16;
+        b->tiles = c.take<char>((size_t)T * kpad * D * 4);
+        b->n2 = c.take<float>((size_t)T * kpad);
+    }
+    b->fill = masked ? c.take<int32_t>((size_t)T * m) : nullptr;
+    b->total = (c.used + 255) & ~(size_t)255;
+}
+
+static int check_nearest_args(int dtype, int T, int n, int m, int D) {
+    HIRA_CHECK_ARG(dtype == HIRA_F32 || dtype == HIRA_BF16, "dtype %d", dtype);
+    const int epl = dtype == HIRA_F32 ? 4 : 8;
+    HIRA_CHECK_ARG(T >= 1 && T <= 65535, "num_trees %d", T);
+    HIRA_CHECK_ARG(n >= 1 && m >= 1, "n = %d rows, m = %d centres", n, m);
+    HIRA_CHECK_ARG(D >= epl && D % epl == 0 && D <= 64 * epl,
+                   "dim %d: rows must be a multiple of 16 bytes", D);
+    return HIRA_OK;
+}
+
+}  // namespace hira
+
+extern "C" size_t hira_nearest_workspace_bytes(int32_t dtype, int32_t num_trees, int32_t m,
+                                               int32_t dim) {
+    if (check_nearest_args(dtype, num_trees, 1, m, dim) != HIRA_OK) return 0;
+    NearestWs b;
+    carve_nearest(dtype, num_trees, m, dim, true, nullptr, &b);
+    return b.total > 0 ? b.total : 256;
+}
+
+extern "C" int hira_nearest(const void* x, int32_t dtype, int32_t num_trees, int32_t n,
+                            const float* centers, int32_t m, int32_t dim, const int32_t* valid,
+                            int32_t* idx, float* dist2, void* workspace, size_t workspace_bytes,
+                            void* stream) {
+    int rc = check_nearest_args(dtype, num_trees, n, m, dim);
+    if (rc != HIRA_OK) return rc;
+    HIRA_CHECK_ARG(x && centers && idx && dist2, "x / centers / idx / dist2 missing");
+    NearestWs b;
+    carve_nearest(dtype, num_trees, m, dim, valid != nullptr, workspace, &b);
+    if (b.total > 0 && (workspace == nullptr || workspace_bytes < b.total))
+        return fail(HIRA_EWORKSPACE, "workspace %zu bytes, need %zu", workspace_bytes, b.total);
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const size_t nm = (size_t)num_trees * m;
+    if (valid != nullptr)
+        hipLaunchKernelGGL(k_valid_to_fill, dim3((unsigned)((nm + 255) / 256)), dim3(256), 0, s,
+                           valid, nm, b.fill);
+    // a row without any usable centre keeps idx -1 and an infinite distance
+    fill_i32(idx, (size_t)num_trees * n, -1, s);
+    fill_i32(reinterpret_cast<int32_t*>(dist2), (size_t)num_trees * n, 0x7f800000, s);
+    if (b.tiles != nullptr) {
+        rc = launch_cent_prep(dim, centers, m, num_trees, b.fill, 1, b.tiles, b.n2, s);
+        if (rc == HIRA_OK)
+            rc = launch_assign_mfma(dim, x, n, (size_t)n, b.tiles, b.n2, m, num_trees, nullptr,
+                                    nullptr, 0, idx, dist2, s);
+    } else {
+        const int epl = dtype == HIRA_F32 ? 4 : 8;
+        int lpr = 2;
+        while (lpr * epl < dim) lpr <<= 1;
+        const dim3 grid(ceil_div(n, 4 * (64 / lpr) * kPPG), num_trees);
+        rc = dtype == HIRA_F32
+                 ? launch_assign<float>(lpr, grid, s, x, n, (size_t)n, centers, m, dim, b.fill, 1,
+                                        nullptr, nullptr, 0, idx, dist2)
+                 : launch_assign<bf16_t>(lpr, grid, s, x, n, (size_t)n, centers, m, dim, b.fill, 1,
+                                         nullptr, nullptr, 0, idx, dist2);
+    }
+    if (rc != HIRA_OK) return rc;
+    HIRA_CHECK_LAUNCH("nearest-centre kernel");
+    return HIRA_OK;
+}

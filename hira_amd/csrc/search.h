@@ -34,6 +34,8 @@ struct SearchParams {
     // work split
     int32_t nodes_per_wave;  // level-1 nodes (or pseudo blocks) per wave; MFMA kernel: tiles per workgroup
     int32_t tree_blocks;     // workgroups that walk the tree; the rest scan the queue
+    int32_t share;           // MFMA kernel: workgroups that gate the same tiles and split what
+                             // survives (tree_blocks is a multiple of it)
     int32_t num_nodes;       // level-1 nodes (or pseudo blocks over the keys when L == 1)
     int32_t num_queue_blocks;
     // outputs
@@ -63,6 +65,7 @@ struct SearchPlan {
     int nodes_per_wave;
     int num_nodes, num_queue_blocks;
     int tree_blocks, queue_blocks, head_chunks;
+    int share;        // MFMA kernel: see SearchParams
     size_t smem;
 };
 
@@ -71,6 +74,23 @@ bool mfma_search_supported(const HiraTree* t, const HiraQueue* queue);
 constexpr int kMfmaThreads = 512;       // workgroup size of the MFMA kernel (8 waves), at most
 constexpr int kMfmaMaxTilesPerWg = 16;  // tiles of 16 level-1 nodes one workgroup walks, at most
 int launch_search_mfma(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
+
+// Hand-off of the attention partials from the workgroups of a tree to the one that folds them
+// (maybe behind another L2).  The partials are written with device-scope atomic stores: they
+// are written through to the level at which every compute unit of the device sees them, and
+// such a store only counts as complete (leaves the wave's count of outstanding memory
+// operations) once it is visible at that level.  Every thread therefore waits here for its own
+// stores to complete; the caller's barrier follows, then ONE thread takes a ticket with a
+// device-scope atomic add, so every ticket is drawn after all partials of its workgroup are
+// visible.  The workgroup that draws the last ticket reads the partials with device-scope
+// atomic loads (which do not take a stale copy from its own L2) after a barrier that depends
+// on the ticket.  A release fence at device scope would also order the stores but writes the
+// whole L2 back first (measured: the decode step takes 36 instead of 20 microseconds);
+// nothing but these atomic stores has to be handed over, so the wait is enough.
+__device__ __forceinline__ void hand_off_release() {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+}
 
 // Element index of (row, column j) inside one tree's (cap, D) matrix.
 //   row-major: row*D + j

@@ -384,7 +384,7 @@ __global__ __launch_bounds__(256) void search_kernel(const SearchParams p) {
     // ---- the last workgroup of this tree (and head pass) to arrive folds its partials ----
     __shared__ int s_last;
     __shared__ float s_fold_red[4];
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // my stores have completed
+    hand_off_release();
     __syncthreads();
     if (threadIdx.x == 0) {
         int* ctr = p.done + (size_t)tree * gridDim.z + blockIdx.z;
@@ -515,9 +515,20 @@ static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* que
             // more work than one workgroup per CU can take: several rounds of smaller ones
             if (tpw > kMfmaMaxTilesPerWg) tpw = kMfmaMaxTilesPerWg / 2;
         }
+        // groups of `share` workgroups may gate the same share*tpw tiles (at most 16: two a wave)
+        // and split the survivors evenly.  Off unless asked for: measured at the benchmark's
+        // shapes the spread between workgroups comes from the burst of key reads draining
+        // through the memory system, not from uneven node counts, and the longer gate costs
+        // more than the even deal gains.
+        int share = launch ? launch->share : 0;
+        HIRA_CHECK_ARG(share >= 0 && share * tpw <= kMfmaMaxTilesPerWg,
+                       "MFMA kernel: share %d x %d tiles per workgroup (at most %d tiles gated)",
+                       share, tpw, kMfmaMaxTilesPerWg);
+        if (share == 0) share = 1;
+        plan->share = share;
         plan->nodes_per_wave = tpw;
         plan->num_nodes = t->size[1];
-        plan->tree_blocks = (tiles + tpw - 1) / tpw;
+        plan->tree_blocks = (tiles + tpw * share - 1) / (tpw * share) * share;
         plan->queue_blocks = plan->num_queue_blocks > 0 ? 1 : 0;  // one workgroup takes the whole queue
         plan->smem = 0;
         return HIRA_OK;
@@ -604,9 +615,13 @@ extern "C" size_t hira_search_workspace_bytes(const HiraTree* tree, const HiraQu
     return workspace_need(query->num_q_heads, P, tree->vdim, tree->num_trees, plan.head_chunks);
 }
 
-extern "C" int hira_search(const HiraTree* tree, const HiraQuery* query, const HiraQueue* queue,
-                           const HiraSearchOut* out, const HiraLaunch* launch, void* workspace,
-                           size_t workspace_bytes, void* stream) {
+// The search behind both entry points.  Attention needs arrival counters (one int32 per tree
+// and head pass, zero between calls) and room for the partials; `fixed_counters` > 0: the
+// counters live in a region of that many entries of their own (the entry point that allocates
+// nothing), else at the start of the caller's workspace, the partials right after them.
+static int search_impl(const HiraTree* tree, const HiraQuery* query, const HiraQueue* queue,
+                       const HiraSearchOut* out, const HiraLaunch* launch, void* workspace,
+                       size_t workspace_bytes, size_t fixed_counters, void* stream) {
     SearchPlan plan;
     int rc = make_plan(tree, query, queue, launch, &plan);
     if (rc != HIRA_OK) return rc;
@@ -661,6 +676,7 @@ extern "C" int hira_search(const HiraTree* tree, const HiraQuery* query, const H
     }
     p.nodes_per_wave = plan.nodes_per_wave;
     p.tree_blocks = plan.tree_blocks;
+    p.share = plan.kernel == 2 ? plan.share : 1;
     p.num_nodes = plan.num_nodes;
     p.num_queue_blocks = use_queue ? plan.num_queue_blocks : 0;
     p.dense = out->dense;
@@ -676,12 +692,20 @@ extern "C" int hira_search(const HiraTree* tree, const HiraQuery* query, const H
     if (P == 0) return HIRA_OK;
     p.num_parts = P;
     if (attn) {
-        const size_t need = workspace_need(query->num_q_heads, (size_t)P, tree->vdim,
-                                           tree->num_trees, plan.head_chunks);
+        size_t ctr_bytes = counter_bytes(tree->num_trees, plan.head_chunks);
+        if (fixed_counters > 0) {
+            if ((size_t)tree->num_trees * plan.head_chunks > fixed_counters)
+                return fail(HIRA_EWORKSPACE, "%d trees x %d head passes: more than the %zu arrival "
+                            "counters of the built-in scratch buffer", tree->num_trees,
+                            plan.head_chunks, fixed_counters);
+            ctr_bytes = fixed_counters * sizeof(int32_t);
+        }
+        const size_t need = ctr_bytes + workspace_need(query->num_q_heads, (size_t)P, tree->vdim, 0, 0);
         if (workspace == nullptr || workspace_bytes < need)
-            return fail(HIRA_EWORKSPACE, "workspace %zu bytes, need %zu", workspace_bytes, need);
-        float* w = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) +
-                                            counter_bytes(tree->num_trees, plan.head_chunks));
+            return fail(HIRA_EWORKSPACE, fixed_counters > 0
+                            ? "the built-in scratch buffer holds %zu bytes, this search needs %zu"
+                            : "workspace %zu bytes, need %zu", workspace_bytes, need);
+        float* w = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + ctr_bytes);
         p.part_acc = w;
         p.part_m = w + (size_t)query->num_q_heads * P * tree->vdim;
         p.part_l = p.part_m + (size_t)query->num_q_heads * P;
@@ -724,4 +748,10 @@ extern "C" int hira_search(const HiraTree* tree, const HiraQuery* query, const H
         HIRA_CHECK_LAUNCH("merge kernel");
     }
     return HIRA_OK;
+}
+
+extern "C" int hira_search(const HiraTree* tree, const HiraQuery* query, const HiraQueue* queue,
+                           const HiraSearchOut* out, const HiraLaunch* launch, void* workspace,
+                           size_t workspace_bytes, void* stream) {
+    return search_impl(tree, query, queue, out, launch, workspace, workspace_bytes, 0, stream);
 }

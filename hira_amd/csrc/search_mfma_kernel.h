@@ -219,14 +219,20 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     const int tree = blockIdx.x;
     const int L = p.num_levels, bf = p.bf;
     const bool want_attn = p.part_acc != nullptr;
-    // my tiles: blockIdx.y, blockIdx.y + (tree workgroups), ...  Neighbouring tiles hold
-    // sibling nodes, which tend to survive (and be selected from) together: striding deals
-    // the busy stretches of the tree out over the workgroups.
-    const int wg_tiles = (p.size[1] + 15) >> 4, wg_stride = p.tree_blocks;
-    const int ntile = (int)blockIdx.y < wg_stride
-                          ? min(p.nodes_per_wave, (wg_tiles - (int)blockIdx.y + wg_stride - 1) / wg_stride)
+    // The tree's workgroups come in groups of `share`.  The workgroups of a group gate the same
+    // tiles -- grp, grp + (groups), ... : a stride apart, since neighbouring tiles hold sibling
+    // nodes, which tend to survive (and be selected from) together -- so each of them knows the
+    // group's whole ordered list of surviving nodes without a word exchanged, and member `rep`
+    // takes entries rep, rep + share, ... of it.  Gating a tile costs a wave one 16 x D read
+    // that the L2 serves; what it buys is that the keys to scan are dealt out evenly however
+    // unevenly the query's hits are spread over the tree.
+    const int wg_tiles = (p.size[1] + 15) >> 4;
+    const int share = p.share, n_groups = p.tree_blocks / share;
+    const int grp = (int)blockIdx.y % n_groups, rep = (int)blockIdx.y / n_groups;
+    const int ntile = (int)blockIdx.y < p.tree_blocks
+                          ? min(p.nodes_per_wave * share, (wg_tiles - grp + n_groups - 1) / n_groups)
                           : 0;
-    auto tile_of = [&](int tl) { return (int)blockIdx.y + tl * wg_stride; };
+    auto tile_of = [&](int tl) { return grp + tl * n_groups; };
     // level-1 node behind entry n (tile n / 16 of mine, node n % 16 of the tile)
     auto node_of = [&](int n) { return tile_of(n >> 4) * 16 + (n & 15); };
     const bool is_queue = (int)blockIdx.y >= p.tree_blocks;  // the workgroup after the tree's
@@ -367,7 +373,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         // ---- gate: one tile per wave at a time ------------------------------------------------
         while (tl_mine < ntile) {  // uniform in the wave
             const int t1 = tile_of(tl_mine);
-            const bool count_nodes = stats != nullptr && lane == 0;
+            const bool count_nodes = stats != nullptr && lane == 0 && rep == 0;  // once per group
             size_t span = 1;  // level-1 nodes under one node of the current level
             for (int l = 2; l < L; ++l) span *= (size_t)bf;
             int lcur = L - 1;
@@ -438,7 +444,8 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         __syncthreads();
         HIRA_TL(1);
 
-        // ---- the surviving nodes of my tiles, dealt round-robin to the waves ----------------------
+        // ---- the surviving nodes of the group's tiles in order; mine are entries rep, rep +
+        // share, ... of them, dealt round-robin to the waves ----------------------------------------
         int rounds, alive = 0;
         {
             const int NT = ntile * 16;
@@ -454,7 +461,8 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                         (uint32_t)(64 * i + lane) | ((info >> 16) << 8) | (info << 16);
                 alive += __popcll(all);
             }
-            rounds = ((alive + nw - 1) / nw + NB - 1) / NB;
+            const int mine = alive > rep ? (alive - rep + share - 1) / share : 0;
+            rounds = ((mine + nw - 1) / nw + NB - 1) / NB;
         }
 
         const float sc2 = sc * kLog2e;
@@ -470,12 +478,13 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         uint32_t nx_mask[NB];
         uint4 a[NB][MT][KS];
         auto fetch = [&](int round, int u_only) {  // u_only < 0: all NB nodes of the round
-            // my nodes of the round: entries (round*NB + u) * nw + wave of the survivors
+            // my nodes of the round: entries ((round*NB + u) * nw + wave) * share + rep of the
+            // group's survivors
             uint32_t ent[NB];
 #pragma unroll
             for (int u = 0; u < NB; ++u) {
                 if (u_only >= 0 && u != u_only) continue;
-                const int k = (round * NB + u) * nw + wave;
+                const int k = ((round * NB + u) * nw + wave) * share + rep;
                 ent[u] = k < alive ? s_order[wave][k] : 0xFFu;
             }
 #pragma unroll
@@ -802,7 +811,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     if (p.done == nullptr) return;  // the caller folds the partials in a second launch
 
     // ---- the last workgroup of this tree (and pass) to arrive folds the tree's partials ----
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // my stores have completed
+    hand_off_release();
     __syncthreads();
     if (threadIdx.x == 0) {
         int* ctr = p.done + (size_t)tree * gridDim.z + blockIdx.z;

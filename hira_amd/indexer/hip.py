@@ -392,6 +392,22 @@ class HIPIndexer(BaseIndexer):
         self._tree_struct = None
         return self
 
+    @staticmethod
+    def storage_dtype(dtype: torch.dtype) -> torch.dtype:
+        """The dtype an index over keys of `dtype` stores: bf16 and fp32 as they are; fp16
+        becomes bf16 (same size, the kernels' 16-bit type; a warning says so, since bf16 has
+        three bits less of mantissa); anything else is up-cast to fp32 as the reference does
+        for every input (indexer/cuda.py:365-368)."""
+        if dtype in _DTYPES:
+            return dtype
+        if dtype == torch.float16:
+            import warnings
+
+            warnings.warn("HIPIndexer stores float16 keys/values as bfloat16 (8 bits of mantissa "
+                          "instead of 11); pass float32 tensors to keep every bit", stacklevel=3)
+            return torch.bfloat16
+        return torch.float32
+
     # ------------------------------------------------------------------ build / update
     @torch.no_grad()
     def build(self, keys: torch.Tensor, values: Optional[torch.Tensor] = None):
@@ -403,7 +419,7 @@ class HIPIndexer(BaseIndexer):
         if values is not None and values.shape[:3] != keys.shape[:3]:
             raise ValueError("values must be aligned with keys: (B,H,L,Dv)")
         b, h, n, d = keys.shape
-        dtype = keys.dtype if keys.dtype in _DTYPES else torch.float32
+        dtype = self.storage_dtype(keys.dtype)
         vdim = 0 if values is None else int(values.shape[-1])
         self._allocate(b, h, n, d, vdim, dtype)
         kin = keys.to(device=self.device, dtype=dtype).reshape(b * h, n, d).contiguous()
@@ -435,7 +451,8 @@ class HIPIndexer(BaseIndexer):
             return [self.num_keys + m]
         # (new nodes appear only once every node of a level is full, so the bound holds for
         # the total of several calls: count from the last sizes that were read back)
-        base = self._exact_size if self._pending else self.size
+        # (while an unsynced stretch is open self.size holds bounds, not sizes)
+        base = self._exact_size if self._exact_size is not None else self.size
         need = [0] * nl
         new = m + self._pending
         for l in range(1, nl):
@@ -454,6 +471,12 @@ class HIPIndexer(BaseIndexer):
             caps.append(-(-c2 // 16) * 16 if self.tiled else c2)
         if caps == self.cap:
             return
+        if getattr(self, "_unsynced_room", 0) > 0:
+            # a launch captured by begin_unsynced holds the current pointers
+            raise RuntimeError(
+                "the index would have to re-allocate while a stretch of unsynced updates is open "
+                "(a captured decode step holds its pointers): call sync_sizes() first, or "
+                "reserve() more room before begin_unsynced()")
 
         def grown(old, cap, fill):
             new = torch.full((old.shape[0], cap) + tuple(old.shape[2:]), fill, dtype=old.dtype,
@@ -602,6 +625,7 @@ class HIPIndexer(BaseIndexer):
         if self.num_levels < 2:
             raise ValueError("needs a tree of at least two levels")
         self.sync_sizes()
+        self._unsynced_room = 0  # (the stretch before this one is over: pointers may move now)
         need = self._needed_caps(int(appends))
         self._grow(need)
         if self._state is None:
@@ -709,6 +733,7 @@ class HIPIndexer(BaseIndexer):
         self.num_keys += m
         if sync:
             self._adopt_state(self._state.cpu())
+            self._unsynced_room = 0
             return self
         if self._pending == 0:
             self._exact_size = list(self.size)
@@ -734,6 +759,9 @@ class HIPIndexer(BaseIndexer):
         if self.num_levels < 3:
             raise ValueError("rebuild_subtree needs at least three levels")
         bf = self.branching_factor
+        if self.tiled and bf % 16:
+            raise ValueError("rebuild_subtree on a tiled index needs a fan-out that is a multiple "
+                             "of 16 (a subtree's slots must start on a tile)")
         self.sync_sizes()
         if not 0 <= node < self.size[2]:
             raise ValueError(f"level-2 node {node} not in 0..{self.size[2] - 1}")

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define HIRA_ABI_VERSION 3
+#define HIRA_ABI_VERSION 4
 #define HIRA_MAX_LEVELS 8
 
 enum { HIRA_F32 = 0, HIRA_BF16 = 1 };
@@ -133,6 +133,9 @@ typedef struct HiraLaunch {
     int32_t kernel;         /* 0 = auto, 1 = vector-ALU kernel, 2 = MFMA kernel (bf16) */
     int32_t separate_merge; /* != 0: fold the attention partials in a second launch even
                                where the search kernel could do it itself */
+    int32_t share;          /* MFMA kernel: workgroups of a tree that gate the same tiles and
+                               split the surviving nodes among them (share * nodes_per_wave at
+                               most 16); 0 or 1 = every workgroup keeps to its own tiles */
 } HiraLaunch;
 
 int hira_abi_version(void);
@@ -182,6 +185,27 @@ size_t hira_build_workspace_bytes(const HiraTree* tree, int32_t n);
 int hira_build(const HiraTree* tree, const void* keys_in, const void* values_in, int32_t n,
                int32_t niter, int32_t pack_rounds, uint64_t seed, void* workspace,
                size_t workspace_bytes, void* stream);
+
+/*
+ * Nearest centre of every row, the distance step of the build (every Lloyd round and every
+ * packing round of hira_build runs these kernels) as a call of its own:
+ *   idx[t][i] = argmin_k ||x[t][i] - centers[t][k]||^2 over the centres with valid[t][k] != 0,
+ * the lowest k on ties, -1 (and dist2 = +inf) when no centre is valid.
+ * Replaces nearest_l2_triton_batched (kernels/triton_update_kernels.py:6-123, 329-418:
+ * argmin of ||c||^2 - 2 x.c over valid centres in blocks of 128, then across the blocks) and
+ * the cdist + argmin of the reference's GPU build (indexer/cuda.py:244-264).
+ *   x        (T, n, D) rows in `dtype`; centers (T, m, D) fp32 (k-means centroids are fp32
+ *            means); valid (T, m) int32 or NULL (all valid)
+ *   idx      (T, n) int32; dist2 (T, n) fp32 squared distance to the chosen centre
+ * bf16 rows of 64, 128 or 256 columns run on the matrix cores (centres split into two bf16
+ * halves so that the choice is as good as with fp32 products), everything else on the vector
+ * ALUs with fp32 differences.
+ */
+size_t hira_nearest_workspace_bytes(int32_t dtype, int32_t num_trees, int32_t m, int32_t dim);
+int hira_nearest(const void* x, int32_t dtype, int32_t num_trees, int32_t n,
+                 const float* centers, int32_t m, int32_t dim, const int32_t* valid,
+                 int32_t* idx, float* dist2, void* workspace, size_t workspace_bytes,
+                 void* stream);
 
 /*
  * Append m new keys (and values) per tree to an existing index, in insertion order.

@@ -1,7 +1,7 @@
 """Turn rocprofv3 CSV output into the short text summaries kept under profiles/.
 
-    python -m hira_amd.profile_summary kernels <kernel_trace.csv>      # per-kernel time
-    python -m hira_amd.profile_summary counters <fetch.csv> <write.csv> \
+    python profile_summary.py kernels <kernel_trace.csv>      # per-kernel time
+    python profile_summary.py counters <fetch.csv> <write.csv> \
         --calib-read BYTES --calib-write BYTES [--json OUT.json]
 
 `counters` scales FETCH_SIZE / WRITE_SIZE of the search kernel by what the same counters

@@ -204,3 +204,59 @@ def test_config_rejects_bad_settings():
     cfg = hira_config.HiraConfig(max_iterations=0, threshold_method="none")
     assert cfg.get_indexer_kwargs() == {"num_levels": 5, "max_iterations": 0, "branching_factor": 10}
     assert cfg.get_threshold_kwargs() == {"method": "none", "sample_size": 1000, "topk": 10}
+
+
+def test_attention_refuses_masks_that_hide_keys():
+    """A padded batch cannot be honoured by the sparse decode step (the index holds every cached
+    position): the attention function raises instead of attending to pad keys."""
+    from types import SimpleNamespace
+
+    from hira_amd.attention.hira_attention import _hides_a_key, hira_attention_forward
+
+    b, h, l, d = 2, 2, 5, 16
+    q = torch.randn(b, h, l, d)
+    cache = SimpleNamespace(indexer=object(), prefill_keys=torch.randn(b, h, l, d),
+                            prefill_values=torch.randn(b, h, l, d))
+    causal = torch.tril(torch.ones(l, l, dtype=torch.bool))[None, None].expand(b, 1, l, l)
+    out, _ = hira_attention_forward(None, q, cache, None, attention_mask=causal)
+    assert out.shape == (b, l, h, d)
+    padded = causal.clone()
+    padded[1, :, :, 0] = False                      # sequence 1 is left-padded by one position
+    with pytest.raises(ValueError, match="padded"):
+        hira_attention_forward(None, q, cache, None, attention_mask=padded)
+    additive = torch.zeros(b, 1, l, l).masked_fill(~padded, float("-inf"))
+    with pytest.raises(ValueError, match="padded"):
+        hira_attention_forward(None, q, cache, None, attention_mask=additive)
+    assert not _hides_a_key(None)
+    assert not _hides_a_key(torch.ones(b, l, dtype=torch.long))
+    assert _hides_a_key(torch.tensor([[0, 1, 1], [1, 1, 1]]))
+    # decode: looked at on the first step of an index
+    idx = SimpleNamespace()
+    dec = SimpleNamespace(indexer=idx, searcher=None, prefill_keys=None)
+    with pytest.raises(ValueError, match="padded"):
+        hira_attention_forward(None, q[:, :, :1], dec, None, attention_mask=padded[:, :, -1:, :])
+
+
+def test_unsynced_stretch_guards_the_pointers():
+    """While a stretch of updates without read-back is open (a captured decode step holds the
+    pointers) the index refuses to re-allocate, and the capacity bound counts from the exact
+    sizes, not from the bound that stands in for them."""
+    idx = HIPIndexer(3, 1, 4, device="cpu")
+    idx.num_trees, idx.num_keys = 1, 64
+    idx.size, idx.cap = [64, 16, 4], [64, 16, 4]
+    idx._exact_size, idx._pending = [64, 16, 4], 0
+    idx.size = [96, 24, 8]                      # bounds, as begin_unsynced leaves them
+    assert idx._needed_caps(4)[2] == 4 + 2      # from the exact size 4, not from the bound 8
+    idx._unsynced_room = 8
+    idx.tiled = False
+    with pytest.raises(RuntimeError, match="re-allocate"):
+        idx._grow([128, 32, 8])
+    idx._grow([64, 16, 4])                      # nothing to do: fine
+
+
+def test_storage_dtype_policy():
+    assert HIPIndexer.storage_dtype(torch.bfloat16) == torch.bfloat16
+    assert HIPIndexer.storage_dtype(torch.float32) == torch.float32
+    with pytest.warns(UserWarning, match="bfloat16"):
+        assert HIPIndexer.storage_dtype(torch.float16) == torch.bfloat16
+    assert HIPIndexer.storage_dtype(torch.float64) == torch.float32
