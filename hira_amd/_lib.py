@@ -96,6 +96,11 @@ SYMBOLS = {
         [C.POINTER(HiraTree), C.POINTER(HiraQuery), C.POINTER(HiraQueue),
          C.POINTER(HiraSearchOut), C.POINTER(HiraLaunch), _vp, C.c_size_t, _vp],
     ),
+    "hira_search_noalloc": (
+        C.c_int,
+        [C.POINTER(HiraTree), C.POINTER(HiraQuery), C.POINTER(HiraQueue),
+         C.POINTER(HiraSearchOut), C.POINTER(HiraLaunch), _vp],
+    ),
     "hira_build_workspace_bytes": (C.c_size_t, [C.POINTER(HiraTree), C.c_int32]),
     "hira_build": (
         C.c_int,

@@ -755,3 +755,42 @@ extern "C" int hira_search(const HiraTree* tree, const HiraQuery* query, const H
                            size_t workspace_bytes, void* stream) {
     return search_impl(tree, query, queue, out, launch, workspace, workspace_bytes, 0, stream);
 }
+
+// ---- the same search for callers that cannot allocate ----------------------------------------
+// Its scratch (arrival counters, then attention partials) is this array in the library's own
+// device image: every GPU the library runs on holds a copy until the process ends.  Host code
+// never touches `scratch` by name (the name is a host-side stand-in, not a device address): the
+// device address is asked for once per device, with that device current, and kept.
+namespace hira {
+constexpr size_t kScratchBytes = (size_t)8 << 20;
+constexpr size_t kScratchCounters = 16384;  // int32 arrival counters at the start (64 KiB)
+constexpr int kMaxDevices = 64;
+}  // namespace hira
+static __device__ __align__(256) unsigned char scratch[hira::kScratchBytes];
+static void* g_scratch_ptr[hira::kMaxDevices];  // per device; written once (same value from any thread)
+
+static int scratch_for_current_device(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(HIRA_ELAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+    HIRA_CHECK_ARG(dev >= 0 && dev < kMaxDevices, "device %d: at most %d devices", dev, kMaxDevices);
+    void* ptr = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+    if (ptr == nullptr) {
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr)
+            return fail(HIRA_ELAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", dev,
+                        hipGetErrorString(e));
+        __atomic_store_n(&g_scratch_ptr[dev], ptr, __ATOMIC_RELEASE);
+    }
+    *out = ptr;
+    return HIRA_OK;
+}
+
+extern "C" int hira_search_noalloc(const HiraTree* tree, const HiraQuery* query,
+                                   const HiraQueue* queue, const HiraSearchOut* out,
+                                   const HiraLaunch* launch, void* stream) {
+    void* ptr = nullptr;
+    const int rc = scratch_for_current_device(&ptr);
+    if (rc != HIRA_OK) return rc;
+    return search_impl(tree, query, queue, out, launch, ptr, kScratchBytes, kScratchCounters, stream);
+}

@@ -166,6 +166,25 @@ int hira_search(const HiraTree* tree, const HiraQuery* query, const HiraQueue* q
                 size_t workspace_bytes, void* stream);
 
 /*
+ * hira_search for callers that cannot allocate device memory and have no workspace to pass:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has
+ * no counterpart in the reference.  Same arguments and results as hira_search; the arrival
+ * counters and attention partials live in a buffer inside the library's own device image
+ * (8 MiB per GPU the library runs on, held until the process ends), so the call allocates
+ * nothing and asks the caller for nothing.  Limits: at most 16384 trees x head passes, and
+ * H_q * P * (Dv + 2) * 4 bytes of partials (P = workgroups per tree, as
+ * hira_search_workspace_bytes counts them) must fit in 8 MiB - 64 KiB; larger searches are
+ * refused with HIRA_EWORKSPACE and a message naming both sizes.  The device that `stream`
+ * belongs to must be the current device.  Every call on a GPU shares that GPU's buffer: calls
+ * that may overlap on one GPU (different streams) race -- order them, or give the others a
+ * workspace of their own through hira_search.  The counters are left at zero by every
+ * completed call; the partials keep the last call's contents and are overwritten before they
+ * are read.
+ */
+int hira_search_noalloc(const HiraTree* tree, const HiraQuery* query, const HiraQueue* queue,
+                        const HiraSearchOut* out, const HiraLaunch* launch, void* stream);
+
+/*
  * Index build.  Replaces CUDAIndexer.build and its helpers (indexer/cuda.py:56-108,
  * 200-336, 338-538: centroid choice, nearest-centroid assignment, closest-first packing into
  * blocks of bf, layout of the levels, radii from the layout, indexer/cuda.py:114-198) and,
