@@ -33,9 +33,13 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def algorithmic_bytes(stats, w, num_levels, steps):
+def algorithmic_bytes(stats, w, num_levels, steps, shadow=False):
     """Mean algorithmic bytes per step from the device counters summed over `steps` steps.
-    stats: (T, MAX_LEVELS+2) int64."""
+    stats: (T, HIRA_STATS_COLS) int64.  Scan of the bf16 keys: every candidate key costs its row
+    (d*e bytes).  Scan of the 8-bit shadow (`shadow`): a candidate costs d bytes, and the rows
+    that the shadow cannot rule out (counted by the kernel) cost their bf16 row on top; a node
+    costs four more bytes (its error bound).  Returns (bytes of the path that ran, bytes by the
+    bf16-scan formula for the same walk, counts)."""
     import numpy as np
     from hira_amd import _lib
 
@@ -44,12 +48,17 @@ def algorithmic_bytes(stats, w, num_levels, steps):
     nodes = sum(s[l] for l in range(1, num_levels))
     cand = s[0]
     sel_any = s[_lib.HIRA_MAX_LEVELS]
+    fetched = s[_lib.HIRA_MAX_LEVELS + 2]
     h_q = w.h_q * w.batch
-    b_search = nodes * (w.d * e + 4) + cand * w.d * e
     b_attn = sel_any * w.d * e + h_q * w.d * 4 + h_q * w.d * e
-    return b_search + b_attn, dict(nodes_per_step=nodes, candidates_per_step=cand,
-                                   selected_union_per_step=sel_any,
-                                   selected_pairs_per_step=s[_lib.HIRA_MAX_LEVELS + 1])
+    b_bf16 = nodes * (w.d * e + 4) + cand * w.d * e + b_attn
+    b_ran = b_bf16
+    if shadow:
+        b_ran = nodes * (w.d * e + 8) + cand * w.d + fetched * w.d * e + b_attn
+    return b_ran, b_bf16, dict(nodes_per_step=nodes, candidates_per_step=cand,
+                               selected_union_per_step=sel_any,
+                               selected_pairs_per_step=s[_lib.HIRA_MAX_LEVELS + 1],
+                               exact_rows_per_step=fetched)
 
 
 def measured_traffic(workload_name):
@@ -286,6 +295,8 @@ def main():
                     help="MFMA kernel: workgroups that gate the same tiles and split the survivors "
                          "(0 = chosen by the library, 1 = no sharing)")
     ap.add_argument("--kmeans-iters", type=int, default=-1)
+    ap.add_argument("--layout", default="auto", choices=["auto", "tiled", "q8", "row_major"],
+                    help="index layout (q8: an 8-bit shadow of the keys is scanned first)")
     ap.add_argument("--separate-merge", action="store_true",
                     help="fold the attention partials in a second launch")
     ap.add_argument("--profile", action="store_true",
@@ -341,12 +352,12 @@ def main():
     keys_d, values_d = keys.to(dev), values.to(dev)
     niter = w.kmeans_iters if a.kmeans_iters < 0 else a.kmeans_iters
     t0 = time.perf_counter()
-    index = HIPIndexer(w.num_levels, niter, w.bf, device="cuda:0").build(keys_d, values_d)
+    index = HIPIndexer(w.num_levels, niter, w.bf, device="cuda:0", layout=a.layout).build(keys_d, values_d)
     torch.cuda.synchronize()
     build_ms = (time.perf_counter() - t0) * 1e3
     # (the first build of a process also loads the library and its code objects)
     t0 = time.perf_counter()
-    again = HIPIndexer(w.num_levels, niter, w.bf, device="cuda:0").build(keys_d, values_d)
+    again = HIPIndexer(w.num_levels, niter, w.bf, device="cuda:0", layout=a.layout).build(keys_d, values_d)
     torch.cuda.synchronize()
     build_again_ms = (time.perf_counter() - t0) * 1e3
     del again
@@ -390,14 +401,15 @@ def main():
         return
 
     # ---- counters: algorithmic bytes of the K timed steps ---------------------------
-    stats = torch.zeros((index.num_trees, _lib.HIRA_MAX_LEVELS + 2), dtype=torch.int64, device=dev)
+    stats = torch.zeros((index.num_trees, _lib.HIRA_STATS_COLS), dtype=torch.int64, device=dev)
     splan = searcher.plan_attention(index, h_all, scaling=torch.full((h_all,), scale), stats=stats)
     scratch = torch.empty((h_all, w.d), dtype=torch.float32, device=dev)
     if not a.profile:
         for i in range(W, total):
             splan.run(q_d[i], taus[i], scratch)
         torch.cuda.synchronize()
-    alg_bytes, counts = algorithmic_bytes(stats.cpu().numpy(), w, index.num_levels, K)
+    alg_bytes, alg_bytes_bf16, counts = algorithmic_bytes(stats.cpu().numpy(), w, index.num_levels, K,
+                                                          shadow=index.q8)
     want_pairs = sum(ksel[b] * w.h_q for b in range(w.batch))
     if abs(counts["selected_pairs_per_step"] - want_pairs) > 1e-6 * want_pairs:
         log(f"[bench] WARNING: selected {counts['selected_pairs_per_step']} pairs/step, "
@@ -468,7 +480,7 @@ def main():
         one_index = 2 * keys_d.numel() * keys_d.element_size()
         a.layers = 8 if one_index <= 256 * 1024 * 1024 else 0
     if a.layers > 1 and not a.profile:
-        copies = [index] + [HIPIndexer(w.num_levels, niter, w.bf, device="cuda:0").build(keys_d, values_d)
+        copies = [index] + [HIPIndexer(w.num_levels, niter, w.bf, device="cuda:0", layout=a.layout).build(keys_d, values_d)
                             for _ in range(a.layers - 1)]
         plans = [plan] + [searcher.plan_attention(c, h_all, scaling=torch.full((h_all,), scale))
                           for c in copies[1:]]
@@ -487,7 +499,8 @@ def main():
             stream.synchronize()
         same = bool(torch.equal(outs2[W:], outs[W:]))
         rot = {"indexes": a.layers, "us_per_step": round(r0.elapsed_time(r1) * 1e3 / K, 3),
-               "bytes_of_all_indexes": int(a.layers * 2 * keys_d.numel() * keys_d.element_size()),
+               "bytes_of_all_indexes": int(a.layers * (2 * keys_d.numel() * keys_d.element_size()
+                                                        + (keys_d.numel() if index.q8 else 0))),
                "same_outputs": same}
         del copies, plans, g3
 
@@ -520,17 +533,25 @@ def main():
     except Exception as ex:  # noqa: BLE001
         log(f"[bench] dense SDPA comparator failed: {ex}")
     # our kernel with every key selected (threshold -inf): a dense decode attention
+    # (always over bf16 keys in the tiled layout: with every key selected an 8-bit scan ahead of
+    # the exact test would only add work, and the comparator should be the best dense path)
     ninf = torch.full((h_all,), -3.0e38, dtype=torch.float32, device=dev)
+    dplan = plan
+    if index.q8:
+        dindex = HIPIndexer(w.num_levels, niter, w.bf, device="cuda:0").build(keys_d, values_d)
+        dplan = searcher.plan_attention(dindex, h_all, scaling=torch.full((h_all,), scale))
     for _ in range(3):
-        plan.run(q_d[0], ninf, scratch)
+        dplan.run(q_d[0], ninf, scratch)
     torch.cuda.synchronize()
     d0, d1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     d0.record()
     for i in range(16):
-        plan.run(q_d[W + i % K], ninf, scratch)
+        dplan.run(q_d[W + i % K], ninf, scratch)
     d1.record()
     torch.cuda.synchronize()
     dense_us["ours_all_selected"] = d0.elapsed_time(d1) * 1e3 / 16
+    if index.q8:
+        del dplan, dindex
 
     # thresholds from a key sample (1000 keys per tree, mean of the 10 best): the launch a
     # deployment puts ahead of every search; K of them in one graph
@@ -573,11 +594,12 @@ def main():
         "data": "captured keys/queries, synthetic values" if a.npz else "synthetic",
         "config": {"workload": w.name, "h_q": w.h_q, "h_kv": w.h_kv, "context": w.n,
                    "head_dim": w.d, "batch": w.batch, "levels": w.num_levels, "bf": w.bf,
-                   "select_per_head": ksel, "kmeans_iters": niter},
+                   "select_per_head": ksel, "kmeans_iters": niter, "layout": index.layout_name},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": measured_traffic(w.name)},
+                     "traffic": measured_traffic(w.name + ("_q8" if index.q8 else ""))},
         "algorithmic_bytes_per_step": round(alg_bytes),
+        "algorithmic_bytes_per_step_bf16_scan": round(alg_bytes_bf16),
         "gpu_us_per_step_events": round(kernel_us, 3),
         "eager_us_per_step": round(eager_ms * 1e3 / K, 3),
         "eager_step_us": {"mean": round(float(per_step.mean()), 2),

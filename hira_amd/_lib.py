@@ -14,8 +14,9 @@ CSRC = HERE / "csrc"
 LIB_PATH = CSRC / "libhira_hip.so"
 
 HIRA_MAX_LEVELS = 8
+HIRA_STATS_COLS = HIRA_MAX_LEVELS + 3  # counters per tree a search can fill in
 HIRA_F32, HIRA_BF16 = 0, 1
-HIRA_ROW_MAJOR, HIRA_TILE16 = 0, 1
+HIRA_ROW_MAJOR, HIRA_TILE16, HIRA_TILE16_Q8 = 0, 1, 2
 HIRA_ABI_VERSION = 4
 
 _vp = C.c_void_p
@@ -39,6 +40,9 @@ class HiraTree(C.Structure):
         ("centers", _vp * HIRA_MAX_LEVELS),
         ("radii", _vp * HIRA_MAX_LEVELS),
         ("counts", _vp * HIRA_MAX_LEVELS),
+        ("keys8", _vp),
+        ("kscale", _vp),
+        ("keps", _vp),
     ]
 
 
@@ -113,6 +117,7 @@ SYMBOLS = {
         [_vp, C.c_int32, C.c_int32, C.c_int32, _vp, C.c_int32, C.c_int32, _vp, _vp, _vp, _vp,
          C.c_size_t, _vp],
     ),
+    "hira_quantize": (C.c_int, [C.POINTER(HiraTree), C.c_int32, C.c_int32, C.c_int32, _vp]),
     "hira_update": (C.c_int, [C.POINTER(HiraTree), _vp, _vp, C.c_int32, _vp, _vp]),
     "hira_sparse_attention": (
         C.c_int,

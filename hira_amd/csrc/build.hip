@@ -439,8 +439,9 @@ __global__ __launch_bounds__(64) void k_radii(const void* child, size_t child_tr
                                               size_t child_radii_stride,
                                               const int32_t* child_order, int size_child,
                                               const void* centers, size_t center_tree_stride,
-                                              int size, int bf, int D, int layout, float* radii,
-                                              int32_t* counts, size_t out_stride) {
+                                              int size, int bf, int D, int child_layout,
+                                              int layout, float* radii, int32_t* counts,
+                                              size_t out_stride) {
     const int p = blockIdx.x, t = blockIdx.y;
     const int lane = threadIdx.x;
     float r = -INFINITY;
@@ -453,7 +454,7 @@ __global__ __launch_bounds__(64) void k_radii(const void* child, size_t child_tr
         float ss = 0.0f;
         for (int e = lane; e < D; e += 64) {
             const float df =
-                load_elem<T>(child, (size_t)t * child_tree_stride * D + elem_index(layout, D, (size_t)s, e)) -
+                load_elem<T>(child, (size_t)t * child_tree_stride * D + elem_index(child_layout, D, (size_t)s, e)) -
                 load_elem<T>(centers, (size_t)t * center_tree_stride * D + elem_index(layout, D, (size_t)p, e));
             ss += df * df;
         }
@@ -696,7 +697,7 @@ static int build_impl(const HiraTree* t, const void* keys_in, const void* values
         const size_t tot = (size_t)t->size[0] * D;
         hipLaunchKernelGGL((k_gather_rows<T>), dim3((unsigned)((tot + 255) / 256), NT), dim3(256),
                            0, s, keys_in, (size_t)n, w.order[0], t->size[0], D, t->keys,
-                           (size_t)t->cap[0], t->layout, t->perm, (size_t)t->cap[0]);
+                           (size_t)t->cap[0], key_layout_of(t->layout), t->perm, (size_t)t->cap[0]);
         if (values_in && t->values) {
             const size_t totv = (size_t)t->size[0] * t->vdim;
             hipLaunchKernelGGL((k_gather_rows<T>), dim3((unsigned)((totv + 255) / 256), NT),
@@ -707,7 +708,7 @@ static int build_impl(const HiraTree* t, const void* keys_in, const void* values
             const size_t totc = (size_t)t->size[l] * D;
             hipLaunchKernelGGL((k_gather_rows<T>), dim3((unsigned)((totc + 255) / 256), NT),
                                dim3(256), 0, s, w.cent_t[l], (size_t)K[l], w.order[l], t->size[l], D,
-                               t->centers[l], (size_t)t->cap[l], t->layout, nullptr, (size_t)0);
+                               t->centers[l], (size_t)t->cap[l], center_layout_of(t->layout), nullptr, (size_t)0);
         }
     }
     // radii and counts, bottom-up
@@ -717,9 +718,12 @@ static int build_impl(const HiraTree* t, const void* keys_in, const void* values
         hipLaunchKernelGGL((k_radii<T>), dim3(t->size[l], NT), dim3(64), 0, s, child,
                            (size_t)t->cap[l - 1], crad, (size_t)t->cap[l - 1], w.order[l - 1],
                            t->size[l - 1], t->centers[l], (size_t)t->cap[l], t->size[l], bf, D,
-                           t->layout, t->radii[l], t->counts[l], (size_t)t->cap[l]);
+                           l == 1 ? key_layout_of(t->layout) : center_layout_of(t->layout),
+                           center_layout_of(t->layout), t->radii[l], t->counts[l], (size_t)t->cap[l]);
     }
     HIRA_CHECK_LAUNCH("build layout");
+    if (t->layout == HIRA_TILE16_Q8)  // steps from all keys, then the 8-bit shadow
+        return hira_quantize(t, 0, t->size[0], 1, s);
     return HIRA_OK;
 }
 
@@ -734,8 +738,13 @@ static int check_build_args(const HiraTree* t, int n) {
     HIRA_CHECK_ARG(t->dim >= epl && t->dim % epl == 0 && t->dim <= 64 * epl,
                    "dim %d: rows must be a multiple of 16 bytes", t->dim);
     HIRA_CHECK_ARG(n >= 1, "need at least one key, got %d", n);
-    HIRA_CHECK_ARG(t->layout == HIRA_ROW_MAJOR || t->layout == HIRA_TILE16, "layout %d", t->layout);
-    if (t->layout == HIRA_TILE16) {
+    HIRA_CHECK_ARG(t->layout == HIRA_ROW_MAJOR || t->layout == HIRA_TILE16 ||
+                       t->layout == HIRA_TILE16_Q8, "layout %d", t->layout);
+    if (t->layout == HIRA_TILE16_Q8)
+        HIRA_CHECK_ARG(t->dim % 64 == 0 && t->num_levels >= 2 && t->keys8 && t->kscale && t->keps,
+                       "the layout with an 8-bit shadow needs rows of a multiple of 64 columns, at "
+                       "least two levels, and the keys8 / kscale / keps arrays");
+    if (t->layout != HIRA_ROW_MAJOR) {
         HIRA_CHECK_ARG(t->dtype == HIRA_BF16 && t->dim % 32 == 0,
                        "the tiled layout needs bf16 rows of a multiple of 32 columns");
         for (int l = 0; l < t->num_levels; ++l)

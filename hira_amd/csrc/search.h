@@ -19,7 +19,11 @@ struct SearchParams {
     int32_t size[HIRA_MAX_LEVELS];
     int32_t cap[HIRA_MAX_LEVELS];
     int32_t num_levels, bf, dim, vdim;
-    int32_t layout;  // HIRA_ROW_MAJOR or HIRA_TILE16 (keys and centers)
+    int32_t layout;  // of the centers: HIRA_ROW_MAJOR or HIRA_TILE16
+    int32_t key_layout;  // of the keys
+    const int8_t* keys8;  // HIRA_TILE16_Q8: the 8-bit shadow, its steps and error bounds
+    const float* kscale;
+    const float* keps;
     // queries
     const void* q;
     const float* tau;
@@ -90,6 +94,20 @@ int launch_search_mfma(const SearchPlan& plan, const SearchParams& p, dim3 grid,
 __device__ __forceinline__ void hand_off_release() {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+}
+
+// Where the keys / the centers of a tree layout sit (HIRA_TILE16_Q8: tiled centers, row-major
+// keys beside their 8-bit shadow).
+__device__ __host__ __forceinline__ int key_layout_of(int layout) {
+    return layout == HIRA_TILE16 ? HIRA_TILE16 : HIRA_ROW_MAJOR;
+}
+__device__ __host__ __forceinline__ int center_layout_of(int layout) {
+    return layout == HIRA_ROW_MAJOR ? HIRA_ROW_MAJOR : HIRA_TILE16;
+}
+// Byte index of column j of row `row` inside one tree's 8-bit shadow (tiles of 16 x 64).
+__device__ __host__ __forceinline__ size_t shadow_index(int D, size_t row, int j) {
+    const size_t chunk = ((row / 16) * (size_t)(D / 64) + (size_t)(j / 64)) * 64 + (size_t)((j % 64) / 16) * 16 + row % 16;
+    return chunk * 16 + (size_t)(j % 16);
 }
 
 // Element index of (row, column j) inside one tree's (cap, D) matrix.

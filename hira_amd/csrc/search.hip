@@ -147,7 +147,7 @@ __global__ __launch_bounds__(256) void search_kernel(const SearchParams p) {
     const size_t krow0 = (size_t)tree * (is_queue ? p.queue_cap : p.cap[0]);
     const int n_rows = is_queue ? p.queue_len : p.size[0];
     const int block_rows = real_nodes ? p.bf : kPseudoBlock;
-    const int klayout = is_queue ? HIRA_ROW_MAJOR : p.layout;
+    const int klayout = is_queue ? HIRA_ROW_MAJOR : p.key_layout;
 
     for (int n0 = node_first; n0 < node_last; n0 += RPW) {
         // -------- gates: lane group rg owns node n0 + rg -----------------------------
@@ -328,7 +328,7 @@ __global__ __launch_bounds__(256) void search_kernel(const SearchParams p) {
     }
 
     if (p.stats) {
-        unsigned long long* st = p.stats + (size_t)tree * (HIRA_MAX_LEVELS + 2);
+        unsigned long long* st = p.stats + (size_t)tree * HIRA_STATS_COLS;
 #pragma unroll
         for (int l = 0; l < HIRA_MAX_LEVELS; ++l)
             if (st_nodes[l]) atomicAdd(&st[l], st_nodes[l]);
@@ -468,9 +468,13 @@ static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* que
                        q->tree_q_heads,
                    "query arrays missing");
     HIRA_CHECK_ARG(q->max_group >= 1, "max_group %d", q->max_group);
-    HIRA_CHECK_ARG(t->layout == HIRA_ROW_MAJOR || t->layout == HIRA_TILE16, "layout %d",
-                   t->layout);
-    if (t->layout == HIRA_TILE16) {
+    HIRA_CHECK_ARG(t->layout == HIRA_ROW_MAJOR || t->layout == HIRA_TILE16 ||
+                       t->layout == HIRA_TILE16_Q8, "layout %d", t->layout);
+    if (t->layout == HIRA_TILE16_Q8)
+        HIRA_CHECK_ARG(t->dim % 64 == 0 && t->num_levels >= 2 && t->keys8 && t->kscale && t->keps,
+                       "the layout with an 8-bit shadow needs rows of a multiple of 64 columns, at "
+                       "least two levels, and the keys8 / kscale / keps arrays");
+    if (t->layout != HIRA_ROW_MAJOR) {
         HIRA_CHECK_ARG(t->dtype == HIRA_BF16 && t->dim % 32 == 0,
                        "the tiled layout needs bf16 rows of a multiple of 32 columns");
         for (int l = 0; l < t->num_levels; ++l)
@@ -661,7 +665,13 @@ static int search_impl(const HiraTree* tree, const HiraQuery* query, const HiraQ
     p.bf = tree->bf;
     p.dim = tree->dim;
     p.vdim = tree->vdim;
-    p.layout = tree->layout;
+    p.layout = center_layout_of(tree->layout);
+    p.key_layout = key_layout_of(tree->layout);
+    if (tree->layout == HIRA_TILE16_Q8) {
+        p.keys8 = tree->keys8;
+        p.kscale = tree->kscale;
+        p.keps = tree->keps;
+    }
     p.q = query->q;
     p.tau = query->tau;
     p.scaling = query->scaling;

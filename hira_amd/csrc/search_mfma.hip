@@ -4,7 +4,7 @@
 namespace hira {
 
 bool mfma_search_supported(const HiraTree* t, const HiraQueue* queue) {
-    if (t->dtype != HIRA_BF16 || t->layout != HIRA_TILE16) return false;
+    if (t->dtype != HIRA_BF16 || (t->layout != HIRA_TILE16 && t->layout != HIRA_TILE16_Q8)) return false;
     if (t->num_levels < 2) return false;
     if (t->bf % 16 != 0 || t->bf > 16 * kMaxTiles) return false;
     if (!(t->dim == 64 || t->dim == 128 || t->dim == 256)) return false;
@@ -17,10 +17,11 @@ bool mfma_search_supported(const HiraTree* t, const HiraQueue* queue) {
 
 // grid: x = tree, y = tile of 16 level-1 nodes, z = pass of 16 heads
 int launch_search_mfma(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s) {
+    const bool q8 = p.keys8 != nullptr;  // the scan reads the keys' 8-bit shadow
     switch (p.dim) {
-        case 64: launch_mfma_d64(plan, p, grid, s); return HIRA_OK;
-        case 128: launch_mfma_d128(plan, p, grid, s); return HIRA_OK;
-        case 256: launch_mfma_d256(plan, p, grid, s); return HIRA_OK;
+        case 64: (q8 ? launch_mfma_q8_d64 : launch_mfma_d64)(plan, p, grid, s); return HIRA_OK;
+        case 128: (q8 ? launch_mfma_q8_d128 : launch_mfma_d128)(plan, p, grid, s); return HIRA_OK;
+        case 256: (q8 ? launch_mfma_q8_d256 : launch_mfma_d256)(plan, p, grid, s); return HIRA_OK;
         default: return fail(HIRA_EINVAL, "MFMA kernel: dim %d", p.dim);
     }
 }

@@ -43,6 +43,7 @@ namespace hira {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(4))) int i32x4_t;
 
 constexpr int kHeadsPerPass = 16;   // MFMA N
 constexpr int kMaxTiles = 4;        // key tiles per block: bf <= 64
@@ -119,6 +120,32 @@ __device__ __forceinline__ f32x4_t tile_scores_lds(const uint4 (&a)[KS], const u
     return acc;
 }
 
+// A 16 x 64 tile of the keys' 8-bit shadow against the 16-bit query steps of up to 16 heads,
+// split into a high and a low byte (two v_mfma_i32_16x16x64_i8 per 64 columns): exact integers
+//   sum_j (256 hi_j + lo_j) k8_j
+// for (row 4*(lane/16) + j, head lane % 16).  Lane (kb, i) of the A operand and lane (kb, head)
+// of the B operands both hold columns [64 s + 16 kb, +16): the order of the columns inside the
+// instruction does not matter as long as both sides agree.
+template <int KS8>
+__device__ __forceinline__ i32x4_t tile_scores_i8(const uint4 (&a)[KS8], const uint4 (&bhi)[KS8],
+                                                  const uint4 (&blo)[KS8]) {
+    i32x4_t hi = {0, 0, 0, 0}, lo = {0, 0, 0, 0};
+#pragma unroll
+    for (int s = 0; s < KS8; ++s) {
+        hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4_t, a[s]),
+                                                   __builtin_bit_cast(i32x4_t, bhi[s]), hi, 0, 0, 0);
+        lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4_t, a[s]),
+                                                   __builtin_bit_cast(i32x4_t, blo[s]), lo, 0, 0, 0);
+    }
+    return hi * 256 + lo;
+}
+
+constexpr float kQ8Steps = 32000.0f;   // the largest |q_j kscale_j| of a head, in its 16-bit steps
+constexpr float kQ8KeySlack = 4e-3f;   // added to a node's error bound (in steps of the shadow):
+                                       // rounding in the bound itself, in sum |q_j kscale_j| and
+                                       // in the fp32 scores of the exact test (D <= 256)
+constexpr float kQ8QuerySlack = 0.51f; // a query component is at most this many steps off
+
 __device__ __forceinline__ float pick4(const f32x4_t& v, int j) {
     return j == 0 ? v[0] : (j == 1 ? v[1] : (j == 2 ? v[2] : v[3]));
 }
@@ -133,18 +160,21 @@ __device__ __forceinline__ void stat_add(unsigned long long* st, int slot, unsig
 }
 
 // Compile-time shape of one instantiation.
-template <int KS, int MT, int GS>
+template <int KS, int MT, int GS, bool Q8 = false>
 struct MfmaShape {
     static constexpr int D = 32 * KS;
     static constexpr int ROWS = MT * 16;  // key slots of one node
+    static constexpr int KA = Q8 ? KS / 2 : KS;  // 16-byte chunks a lane holds of a scanned tile
     // nodes whose key tiles one wave keeps in flight: what the budget of 256 registers leaves
-    // after twice the accumulators (GS x D/64) and some seventy registers of everything else,
-    // and what keeps the round's list under 48 KiB of LDS
-    static constexpr int KEY_REGS = 256 - 72 - 2 * GS * (KS / 2);
-    static constexpr int NB_REGS = KEY_REGS / (MT * KS * 4);
+    // after twice the accumulators (GS x D/64) and some seventy registers of everything else
+    // (with the 8-bit shadow: also its B operands, one batch of key rows of the exact test and
+    // the value rows asked for ahead of it), and what keeps the round's list under 48 KiB of LDS
+    static constexpr int KEY_REGS = 256 - 72 - 2 * GS * (KS / 2) - (Q8 ? 4 * KS + 4 * KS + 32 : 0);
+    static constexpr int NB_REGS = KEY_REGS / (MT * KA * 4);
     static constexpr int NB_LDS = (12000 / (GS + 1)) / (kMfmaWaves * ROWS);
     static constexpr int NB_MIN = NB_REGS < NB_LDS ? NB_REGS : NB_LDS;
-    static constexpr int NB = NB_MIN < 1 ? 1 : (NB_MIN > 4 ? 4 : NB_MIN);
+    static constexpr int NB_MAX = Q8 ? 8 : 4;
+    static constexpr int NB = NB_MIN < 1 ? 1 : (NB_MIN > NB_MAX ? NB_MAX : NB_MIN);
     static constexpr int LIST = kMfmaWaves * NB * ROWS;  // rows of the list of one round
     static constexpr int SCAN_WORDS = LIST * (GS + 1) + LIST / 16;  // row list, tile slots, GS scores per row
     static constexpr int MERGE_WORDS = kMfmaWaves * 4 * D;  // four heads of every wave
@@ -157,12 +187,13 @@ struct GateLoads {
     uint4 a1[KS];      // the tile of level-1 centres
     float4 r4;         // radii of rows 4*kb .. 4*kb+3
     int4 c4;           // child counts of the same rows
+    float4 e4;         // (8-bit shadow) error bounds of the same rows
     uint4 anc[2][KS];  // tiles holding the ancestors at levels min(L-1,3) and the one below
     float arad[2];
     size_t aid[2];
 };
 
-template <int KS>
+template <int KS, bool Q8>
 __device__ __forceinline__ void gate_issue(const SearchParams& p, int tree, int t1, int lane,
                                            int kb, GateLoads<KS>& g) {
     const int L = p.num_levels;
@@ -170,6 +201,7 @@ __device__ __forceinline__ void gate_issue(const SearchParams& p, int tree, int 
     load_tile<KS>(tile_ptr<KS>(p.centers[1], row1, (size_t)t1, lane), g.a1);
     g.r4 = *reinterpret_cast<const float4*>(p.radii[1] + row1 + (size_t)t1 * 16 + 4 * kb);
     g.c4 = *reinterpret_cast<const int4*>(p.counts[1] + row1 + (size_t)t1 * 16 + 4 * kb);
+    if (Q8) g.e4 = *reinterpret_cast<const float4*>(p.keps + row1 + (size_t)t1 * 16 + 4 * kb);
     size_t sp = 1;  // level-1 nodes under one node of level min(L-1, 3)
     for (int l = 2; l <= min(L - 1, 3); ++l) sp *= (size_t)p.bf;
     const int n_par = min(max(L - 2, 0), 2);
@@ -190,11 +222,18 @@ __device__ __forceinline__ void gate_issue(const SearchParams& p, int tree, int 
 
 // OUT: the launch also wants dense scores or selection lists (kept out of the attention-only
 // instantiation, whose registers are all spoken for).
-template <int KS, int MT, int GS, bool OUT>
+// Q8: the index keeps an 8-bit shadow of its keys (HIRA_TILE16_Q8).  The scan then reads the
+// shadow's tiles (half the bytes) and lists the rows that the shadow cannot rule out for some
+// head; their bf16 rows (row-major) are fetched, 16 at a time as one MFMA operand, and take the
+// exact test -- with the very products of the other layout, so the selected set and the scores
+// are the same bit for bit.
+template <int KS, int MT, int GS, bool OUT, bool Q8>
 __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const SearchParams p) {
-    using S = MfmaShape<KS, MT, GS>;
+    using S = MfmaShape<KS, MT, GS, Q8>;
     constexpr int D = S::D;
     constexpr int NB = S::NB;
+    constexpr int KA = S::KA;          // 16-byte chunks per lane of a scanned tile
+    constexpr int KS8 = Q8 ? KS / 2 : 1;
     constexpr int VPL = KS / 2;        // value elements per lane: Dv = D = 64 * VPL
     constexpr int VW = (VPL + 1) / 2;  // dwords of a value row per lane
     __shared__ uint32_t s_words[S::WORDS];  // the round's list; the merge; the fold
@@ -210,6 +249,11 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     __shared__ int s_nc[kHeadsPerPass];
     __shared__ int s_last;
     __shared__ uint4 s_bq[KS * 64];  // the B operand (queries) of the scan
+    // 8-bit shadow: the queries in steps of the shadow, high and low bytes, as B operands; the
+    // step and sum_j |q_j kscale_j| of every head; the error bounds of my nodes
+    __shared__ uint4 s_bq8[Q8 ? 2 * KS8 * 64 : 1];
+    __shared__ float s_qc[Q8 ? 2 * kHeadsPerPass : 1];
+    __shared__ float s_keps[Q8 ? kMfmaMaxTilesPerWg * 16 : 1];
 
     const int lane = lane_id();
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -242,7 +286,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         p.stats + (((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 16;
 #define HIRA_TL(k) do { if (threadIdx.x == 0) tl[k] = wall_clock64(); } while (0)
 #else
-    unsigned long long* stats = p.stats ? p.stats + (size_t)tree * (HIRA_MAX_LEVELS + 2) : nullptr;
+    unsigned long long* stats = p.stats ? p.stats + (size_t)tree * HIRA_STATS_COLS : nullptr;
 #define HIRA_TL(k) do { } while (0)
 #endif
     HIRA_TL(0);
@@ -349,7 +393,78 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         const float tau = head_ok ? p.tau[qh] : INFINITY;
         const float sc = head_ok ? p.scaling[qh] : 0.0f;
         GateLoads<KS> gl;
-        if (tl_mine < ntile) gate_issue<KS>(p, tree, tile_of(tl_mine), lane, kb, gl);
+        if (tl_mine < ntile) gate_issue<KS, Q8>(p, tree, tile_of(tl_mine), lane, kb, gl);
+        if constexpr (Q8) {
+            // ---- the queries in steps of the shadow (wave 0, for all): lane (kb, head) takes
+            // columns [64 s + 16 kb, +16) as the shadow's tiles hold them: u_j = q_j kscale_j,
+            // the head's step su = max_j |u_j| / kQ8Steps, U_j = round(u_j / su) in two bytes -------
+            if (wave == 0) {
+                float uf[KS8][16];
+                float umax = 0.0f, asum = 0.0f;
+#pragma unroll
+                for (int s = 0; s < KS8; ++s) {
+                    const int c0 = 64 * s + 16 * kb;
+                    uint4 qa = make_uint4(0, 0, 0, 0), qb = make_uint4(0, 0, 0, 0);
+                    if (head_ok) {
+                        const uint16_t* qp = reinterpret_cast<const uint16_t*>(p.q) + (size_t)qh * D + c0;
+                        qa = *reinterpret_cast<const uint4*>(qp);
+                        qb = *reinterpret_cast<const uint4*>(qp + 8);
+                    }
+                    float qf[16];
+                    {
+                        float f[8];
+                        unpack<bf16_t>(qa, f);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) qf[e] = f[e];
+                        unpack<bf16_t>(qb, f);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) qf[8 + e] = f[e];
+                    }
+                    const float4* kp = reinterpret_cast<const float4*>(p.kscale + (size_t)tree * D + c0);
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const float4 k4 = kp[c];
+                        uf[s][4 * c + 0] = qf[4 * c + 0] * k4.x;
+                        uf[s][4 * c + 1] = qf[4 * c + 1] * k4.y;
+                        uf[s][4 * c + 2] = qf[4 * c + 2] * k4.z;
+                        uf[s][4 * c + 3] = qf[4 * c + 3] * k4.w;
+                    }
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        umax = fmaxf(umax, fabsf(uf[s][e]));
+                        asum += fabsf(uf[s][e]);
+                    }
+                }
+                umax = fmaxf(umax, __shfl_xor(umax, 16, 64));
+                umax = fmaxf(umax, __shfl_xor(umax, 32, 64));
+                asum += __shfl_xor(asum, 16, 64);
+                asum += __shfl_xor(asum, 32, 64);
+                const float su = fmaxf(umax, 1e-30f) / kQ8Steps;
+#pragma unroll
+                for (int s = 0; s < KS8; ++s) {
+                    uint32_t hi[4], lo[4];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        hi[c] = 0u;
+                        lo[c] = 0u;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const int U = (int)rintf(uf[s][4 * c + e] / su);
+                            const int h = (U + 128) >> 8;  // U = 256 h + l, l in [-128, 127]
+                            const int l = U - (h << 8);
+                            hi[c] |= ((uint32_t)h & 0xFFu) << (8 * e);
+                            lo[c] |= ((uint32_t)l & 0xFFu) << (8 * e);
+                        }
+                    }
+                    s_bq8[s * 64 + lane] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+                    s_bq8[(KS8 + s) * 64 + lane] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+                }
+                if (kb == 0) {
+                    s_qc[col] = su;
+                    s_qc[kHeadsPerPass + col] = asum;
+                }
+            }
+        }
 
         // ---- B operand and ||q|| -----------------------------------------------------------
         bf16x8_t bq[KS];
@@ -437,8 +552,18 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 s_ninfo[tl_mine * 16 + lane] =
                     (uint32_t)((bits >> (16 * (lane >> 2))) & 0xFFFFull) | ((uint32_t)cnt_n << 16);
             }
+            if constexpr (Q8) {  // the error bounds of the tile's nodes travel like the counts
+                const float ee[4] = {gl.e4.x, gl.e4.y, gl.e4.z, gl.e4.w};
+                float eps_n = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float e = __shfl(ee[j], 16 * ((lane >> 2) & 3), 64);
+                    if ((lane & 3) == j) eps_n = e;
+                }
+                if (lane < 16) s_keps[tl_mine * 16 + lane] = eps_n;
+            }
             tl_mine += nw;
-            if (tl_mine < ntile) gate_issue<KS>(p, tree, tile_of(tl_mine), lane, kb, gl);
+            if (tl_mine < ntile) gate_issue<KS, Q8>(p, tree, tile_of(tl_mine), lane, kb, gl);
         }
         HIRA_TL(7);
         __syncthreads();
@@ -468,15 +593,31 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         const float sc2 = sc * kLog2e;
         const size_t row0 = (size_t)tree * p.cap[0];
 
+        // (8-bit shadow: krsrc = the bf16 rows of the exact test, row-major; k8rsrc = the tiles
+        // of the shadow, which the scan reads)
         const __amdgpu_buffer_rsrc_t krsrc = make_rsrc(
             reinterpret_cast<const uint16_t*>(p.keys) + row0 * (size_t)D, (size_t)p.cap[0] * D * 2);
+        const __amdgpu_buffer_rsrc_t k8rsrc =
+            Q8 ? make_rsrc(p.keys8 + row0 * (size_t)D, (size_t)p.cap[0] * D) : krsrc;
+        uint4 bq8h[KS8], bq8l[KS8];
+        float su = 0.0f, asum = 0.0f;
+        if constexpr (Q8) {
+#pragma unroll
+            for (int s = 0; s < KS8; ++s) {
+                bq8h[s] = s_bq8[s * 64 + lane];
+                bq8l[s] = s_bq8[(KS8 + s) * 64 + lane];
+            }
+            su = s_qc[col];
+            asum = s_qc[kHeadsPerPass + col];
+        }
         const __amdgpu_buffer_rsrc_t vrsrc = make_rsrc(
             reinterpret_cast<const uint16_t*>(p.values) + row0 * (size_t)D, (size_t)p.cap[0] * D * 2);
         // The nodes a wave takes in a round (up to NB of its share), what LDS says about them,
         // and the loads of their key tiles.
         int nx_node[NB], nx_cnt[NB];
         uint32_t nx_mask[NB];
-        uint4 a[NB][MT][KS];
+        float nx_eps[Q8 ? NB : 1];
+        uint4 a[NB][MT][KA];
         auto fetch = [&](int round, int u_only) {  // u_only < 0: all NB nodes of the round
             // my nodes of the round: entries ((round*NB + u) * nw + wave) * share + rep of the
             // group's survivors
@@ -495,12 +636,13 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 nx_node[u] = n;
                 nx_cnt[u] = (int)((e >> 8) & 0xFFu);
                 nx_mask[u] = e >> 16;
+                if constexpr (Q8) nx_eps[u] = s_keps[max(n, 0)];
                 const unsigned tile_first = (unsigned)(node_of(max(n, 0)) * bf) / 16u;
 #pragma unroll
                 for (int tt = 0; tt < MT; ++tt)
                     if (tt * 16 < nx_cnt[u])
-                        load_tile_buf<KS>(krsrc, (unsigned)lane * 16u,
-                                          (tile_first + tt) * (unsigned)(KS * 1024), a[u][tt]);
+                        load_tile_buf<KA>(Q8 ? k8rsrc : krsrc, (unsigned)lane * 16u,
+                                          (tile_first + tt) * (unsigned)(KA * 1024), a[u][tt]);
             }
         };
         if (rounds > 0) fetch(0, -1);
@@ -528,11 +670,118 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
             const int zrow0 = wave * (NB * S::ROWS);  // my stretch of the round's rows
             int node[NB], cnt[NB];
             uint32_t nmask[NB];
+            // dense scores / compact lists of the selected rows among 16 scored ones: lane
+            // (kb, head) holds rows 4*kb + j, whose key slots are slot4[j]
+            auto emit = [&](unsigned sel4, const f32x4_t& sco, const unsigned (&slot4)[4]) {
+                unsigned long long sb[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) sb[j] = __ballot((sel4 >> j) & 1u);
+                int base = 0;
+                if (p.sel_count != nullptr) {  // one atomic per head of the tile (kb = 0)
+                    int mine = 0;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        mine += __popcll(sb[j] & (0x0001000100010001ull << col));
+                    int b0 = 0;
+                    if (kb == 0 && mine > 0) b0 = atomicAdd(&p.sel_count[qh], mine);
+                    base = __shfl(b0, col, 64);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if ((sel4 >> j) & 1u) {
+                        const unsigned slot = slot4[j];
+                        int idx = (int)slot;
+                        if (p.dense_by_position) idx = p.perm[row0 + slot];
+                        if (p.dense != nullptr)
+                            p.dense[(int64_t)qh * p.dense_stride + idx] = sco[j] * sc;
+                        if (p.sel_count != nullptr) {
+                            // hits of my head ordered before (kb, j): rows j' < j of any
+                            // kb, then row j of lower kb
+                            int before = 0;
+#pragma unroll
+                            for (int j2 = 0; j2 < 4; ++j2) {
+                                unsigned long long bits = sb[j2] & (0x0001000100010001ull << col);
+                                if (j2 == j) bits &= (1ull << (16 * kb)) - 1ull;
+                                if (j2 <= j) before += __popcll(bits);
+                            }
+                            const int pos = base + before;
+                            if (pos < p.sel_cap) {
+                                p.sel_index[(int64_t)qh * p.sel_cap + pos] = idx;
+                                p.sel_score[(int64_t)qh * p.sel_cap + pos] = sco[j];
+                            }
+                        }
+                    }
+                }
+            };
+            // rows (of 16) for which some head's bit is set: OR over the 16 lanes (heads) of my
+            // row group by rotating inside the group, then the four groups side by side
+            auto rows_of = [&](unsigned sel4) {
+                unsigned any4 = sel4;
+                any4 |= (unsigned)__builtin_amdgcn_update_dpp(0, (int)any4, 0x121, 0xF, 0xF, false);
+                any4 |= (unsigned)__builtin_amdgcn_update_dpp(0, (int)any4, 0x122, 0xF, 0xF, false);
+                any4 |= (unsigned)__builtin_amdgcn_update_dpp(0, (int)any4, 0x124, 0xF, 0xF, false);
+                any4 |= (unsigned)__builtin_amdgcn_update_dpp(0, (int)any4, 0x128, 0xF, 0xF, false);
+                return (unsigned)__builtin_amdgcn_readlane((int)any4, 0) |
+                       ((unsigned)__builtin_amdgcn_readlane((int)any4, 16) << 4) |
+                       ((unsigned)__builtin_amdgcn_readlane((int)any4, 32) << 8) |
+                       ((unsigned)__builtin_amdgcn_readlane((int)any4, 48) << 12);
+            };
+            auto count_selected = [&](unsigned sel4, unsigned rowmask) {
+                const unsigned pairs = (unsigned)__popcll(__ballot(sel4 & 1u)) +
+                                       (unsigned)__popcll(__ballot(sel4 & 2u)) +
+                                       (unsigned)__popcll(__ballot(sel4 & 4u)) +
+                                       (unsigned)__popcll(__ballot(sel4 & 8u));
+                if (lane == 0) {
+                    stat_add(stats, HIRA_MAX_LEVELS, (unsigned)__popc(rowmask));
+                    stat_add(stats, HIRA_MAX_LEVELS + 1, pairs);
+                }
+            };
 #pragma unroll
             for (int u = 0; u < NB; ++u) {
                 node[u] = nx_node[u];
                 cnt[u] = nx_cnt[u];
                 nmask[u] = nx_mask[u];
+                const unsigned slot0 = (unsigned)(node_of(max(node[u], 0)) * bf);
+                if constexpr (Q8) {
+                    // ---- the shadow's tiles: which rows can it not rule out, for which heads? ----
+                    const float eps_u = nx_eps[u];
+                    i32x4_t est_u[MT];
+#pragma unroll
+                    for (int tt = 0; tt < MT; ++tt)
+                        if (tt * 16 < cnt[u]) est_u[tt] = tile_scores_i8<KS8>(a[u][tt], bq8h, bq8l);
+                    if (r + 1 < rounds) fetch(r + 1, u);
+                    // the score q.k lies within `marg` of su * (the integer): the keys' rounding
+                    // (eps_u steps a component at most) and the query's (kQ8QuerySlack steps of su)
+                    const float marg = (eps_u + kQ8KeySlack) * asum + su * (kQ8QuerySlack * 127.0f * (float)D);
+                    const bool head_on = head_ok && ((nmask[u] >> col) & 1u);
+                    const float thr_u = head_on ? tau - marg - 1e-6f * (fabsf(tau) + marg) : INFINITY;
+                    if (stats && lane == 0) stat_add(stats, 0, (unsigned)cnt[u]);
+#pragma unroll
+                    for (int tt = 0; tt < MT; ++tt) {
+                        if (tt * 16 >= cnt[u]) continue;  // uniform
+                        const int lim = cnt[u] - tt * 16 - 4 * kb;  // my rows j < lim hold keys
+                        unsigned pass4 = 0u;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            if (su * (float)est_u[tt][j] >= thr_u && j < lim) pass4 |= 1u << j;
+                        if (__ballot(pass4 != 0u) == 0ull) continue;  // uniform
+                        const unsigned rowmask = rows_of(pass4);
+                        if (stats && lane == 0) stat_add(stats, HIRA_MAX_LEVELS + 2, (unsigned)__popc(rowmask));
+                        const unsigned tslot = slot0 + tt * 16;
+                        // the tile's rows in the table say, for now, which heads a row passed for
+                        // (0 / -inf); the rows that passed for some head join my list
+                        const int trow = zrow0 + (u * MT + tt) * 16;
+                        if (col < GS) {
+                            float* zp = lst_z + (trow + 4 * kb) * GS + col;
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) zp[j * GS] = ((pass4 >> j) & 1u) ? 0.0f : -INFINITY;
+                        }
+                        if (lane_o < 16 && ((rowmask >> lane_o) & 1u))
+                            lst_row[zrow0 + nsel + __popc(rowmask & ((1u << lane_o) - 1u))] = (uint32_t)(trow + lane_o);
+                        if (lane_o == 0) lst_tslot[trow >> 4] = tslot;
+                        nsel += __popc(rowmask);
+                    }
+                } else {
                 f32x4_t sco_u[MT];
 #pragma unroll
                 for (int tt = 0; tt < MT; ++tt)  // (only read where it is written: under this condition)
@@ -540,7 +789,6 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 if (r + 1 < rounds) fetch(r + 1, u);
                 // a head for which the node did not survive selects nothing
                 const float tau_u = ((nmask[u] >> col) & 1u) ? tau : INFINITY;
-                const unsigned slot0 = (unsigned)(node_of(max(node[u], 0)) * bf);
                 if (stats && lane == 0) stat_add(stats, 0, (unsigned)cnt[u]);
 #pragma unroll
                 for (int tt = 0; tt < MT; ++tt) {
@@ -552,70 +800,15 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                     for (int j = 0; j < 4; ++j)
                         if (sco[j] >= tau_u && j < lim) sel4 |= 1u << j;
                     if (__ballot(sel4 != 0u) == 0ull) continue;  // uniform
-                    // rows selected by some head: OR over the 16 lanes (heads) of my row group by
-                    // rotating inside the group, then the four groups side by side
-                    unsigned any4 = sel4;
-                    any4 |= (unsigned)__builtin_amdgcn_update_dpp(0, (int)any4, 0x121, 0xF, 0xF, false);
-                    any4 |= (unsigned)__builtin_amdgcn_update_dpp(0, (int)any4, 0x122, 0xF, 0xF, false);
-                    any4 |= (unsigned)__builtin_amdgcn_update_dpp(0, (int)any4, 0x124, 0xF, 0xF, false);
-                    any4 |= (unsigned)__builtin_amdgcn_update_dpp(0, (int)any4, 0x128, 0xF, 0xF, false);
-                    const unsigned rowmask = (unsigned)__builtin_amdgcn_readlane((int)any4, 0) |
-                                             ((unsigned)__builtin_amdgcn_readlane((int)any4, 16) << 4) |
-                                             ((unsigned)__builtin_amdgcn_readlane((int)any4, 32) << 8) |
-                                             ((unsigned)__builtin_amdgcn_readlane((int)any4, 48) << 12);
-                    if (stats) {
-                        const unsigned pairs = (unsigned)__popcll(__ballot(sel4 & 1u)) +
-                                               (unsigned)__popcll(__ballot(sel4 & 2u)) +
-                                               (unsigned)__popcll(__ballot(sel4 & 4u)) +
-                                               (unsigned)__popcll(__ballot(sel4 & 8u));
-                        if (lane == 0) {
-                            stat_add(stats, HIRA_MAX_LEVELS, (unsigned)__popc(rowmask));
-                            stat_add(stats, HIRA_MAX_LEVELS + 1, pairs);
-                        }
-                    }
+                    const unsigned rowmask = rows_of(sel4);  // rows selected by some head
+                    if (stats) count_selected(sel4, rowmask);
                     const unsigned tslot = slot0 + tt * 16;
 
                     // ---- dense scores / compact lists ------------------------------------------
                     if (OUT && (p.dense != nullptr || p.sel_count != nullptr)) {
-                        unsigned long long sb[4];
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) sb[j] = __ballot((sel4 >> j) & 1u);
-                        int base = 0;
-                        if (p.sel_count != nullptr) {  // one atomic per head of the tile (kb = 0)
-                            int mine = 0;
-#pragma unroll
-                            for (int j = 0; j < 4; ++j)
-                                mine += __popcll(sb[j] & (0x0001000100010001ull << col));
-                            int b0 = 0;
-                            if (kb == 0 && mine > 0) b0 = atomicAdd(&p.sel_count[qh], mine);
-                            base = __shfl(b0, col, 64);
-                        }
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            if ((sel4 >> j) & 1u) {
-                                const unsigned slot = tslot + 4 * kb + j;
-                                int idx = (int)slot;
-                                if (p.dense_by_position) idx = p.perm[row0 + slot];
-                                if (p.dense != nullptr)
-                                    p.dense[(int64_t)qh * p.dense_stride + idx] = sco[j] * sc;
-                                if (p.sel_count != nullptr) {
-                                    // hits of my head ordered before (kb, j): rows j' < j of any
-                                    // kb, then row j of lower kb
-                                    int before = 0;
-#pragma unroll
-                                    for (int j2 = 0; j2 < 4; ++j2) {
-                                        unsigned long long bits = sb[j2] & (0x0001000100010001ull << col);
-                                        if (j2 == j) bits &= (1ull << (16 * kb)) - 1ull;
-                                        if (j2 <= j) before += __popcll(bits);
-                                    }
-                                    const int pos = base + before;
-                                    if (pos < p.sel_cap) {
-                                        p.sel_index[(int64_t)qh * p.sel_cap + pos] = idx;
-                                        p.sel_score[(int64_t)qh * p.sel_cap + pos] = sco[j];
-                                    }
-                                }
-                            }
-                        }
+                        const unsigned slot4[4] = {tslot + 4 * kb, tslot + 4 * kb + 1, tslot + 4 * kb + 2,
+                                                   tslot + 4 * kb + 3};
+                        emit(sel4, sco, slot4);
                     }
 
                     // ---- the tile's scores go to the table, its selected rows join my list -----------
@@ -638,42 +831,14 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                     }
                     nsel += __popc(rowmask);
                 }
+                }  // shadow or bf16 tiles
             }
-            if (!want_attn) continue;  // uniform in the launch
+            const int tot = nsel;  // rows on my list
 
-            // ---- the best selected score of every head in my rows of this round --------------------
-            zmax = fmaxf(zmax, __shfl_xor(zmax, 16, 64));
-            zmax = fmaxf(zmax, __shfl_xor(zmax, 32, 64));
-            const float rmax = zmax;
-            const int tot = nsel;
-#ifdef HIRA_TIMELINE
-            if (r == 0) HIRA_TL(9);
-            if (threadIdx.x == 0 && r == 0) { tl[6] = (unsigned long long)tot; tl[12] = (unsigned long long)rounds; }
-#endif
-            if (tot == 0) continue;  // uniform in the wave: nothing selected in my rows
-
-            // the new maximum of every head, and what it does to the sums so far; head g lives in
-            // lane g; the weights below are computed with lane = (row, head), head = lane % GS
-            const float mnew = fmaxf(m_run, rmax);
-            const float f = (m_run == mnew) ? 1.0f : exp2f(m_run - mnew);
-            m_run = mnew;
-            // a head without a selected key has m = -inf and only z = -inf: any finite stand-in
-            const float m_lane = __shfl(mnew == -INFINITY ? 0.0f : mnew, lane_o & (GS - 1), 64);
-            if (__ballot(f != 1.0f) != 0ull) {  // uniform
-                l_mine *= __shfl(f, lane_o & (GS - 1), 64);
-#pragma unroll
-                for (int g = 0; g < GS; ++g) {
-                    const float fg = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), g));
-#pragma unroll
-                    for (int e = 0; e < VPL; ++e) acc[g][e] *= fg;
-                }
-            }
-
-            // ---- gather my listed rows: kVBatch value rows in flight -------------------------------
+            // ---- value rows: kVBatch in flight; the rows of a batch in the score table (lane =
+            // (row of the pass, head)), their key slots, and the loads ---------------------------------
             constexpr int RP = 64 / GS;          // rows whose weights one pass over the lanes computes
             constexpr int NPASS = kVBatch / RP;  // GS = 4: 2, GS = 8: 4, GS = 16: 8
-            // the rows of a batch in the score table (lane = (row of the pass, head)), their key
-            // slots, and the loads of their value rows
             auto issue = [&](int e0, int (&at_v)[NPASS], uint32_t (&vraw)[kVBatch][VW]) {
 #pragma unroll
                 for (int ps = 0; ps < NPASS; ++ps) {
@@ -703,6 +868,78 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                     }
                 }
             };
+            int at_v0[Q8 ? NPASS : 1];
+            uint32_t vraw0[Q8 ? kVBatch : 1][VW];
+            if constexpr (Q8) {
+                // the value rows of the first batch are asked for ahead of the key rows: most rows
+                // that the shadow lets through are selected
+                if (want_attn && tot > 0) issue(0, at_v0, vraw0);
+                // ---- the exact test: the listed rows' bf16 keys, 16 at a time as one A operand
+                // (lane (kb, i): columns [32 s + 8 kb, +8) of the i-th of them) -----------------------
+                for (int e0 = 0; e0 < tot; e0 += 16) {  // uniform in the wave
+                    const int le = e0 + (lane_o & 15);
+                    const int at = le < tot ? (int)lst_row[zrow0 + le] : -1;  // (-1: past the end)
+                    const unsigned slot = at >= 0 ? lst_tslot[at >> 4] + (unsigned)(at & 15) : 0u;
+                    uint4 kr[KS];
+#pragma unroll
+                    for (int s = 0; s < KS; ++s)
+                        kr[s] = __builtin_bit_cast(
+                            uint4, __builtin_amdgcn_raw_buffer_load_b128(
+                                       krsrc, slot * (unsigned)(D * 2) + (unsigned)(kb * 16 + s * 64), 0, 0));
+                    const f32x4_t sco = tile_scores_lds<KS>(kr, s_bq, lane_o);
+                    unsigned sel4 = 0u;
+                    int at4[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        at4[j] = __shfl(at, 4 * kb + j, 64);
+                        const bool mine = col < GS && at4[j] >= 0;
+                        // (the table holds 0 where the shadow let the row pass for my head)
+                        const float pz = mine ? lst_z[at4[j] * GS + col] : -INFINITY;
+                        const bool sel = pz == 0.0f && sco[j] >= tau;
+                        if (sel) sel4 |= 1u << j;
+                        const float z = sel ? sco[j] * sc2 : -INFINITY;
+                        zmax = fmaxf(zmax, z);
+                        if (mine) lst_z[at4[j] * GS + col] = z;
+                    }
+                    if (stats) count_selected(sel4, rows_of(sel4));
+                    if (OUT && (p.dense != nullptr || p.sel_count != nullptr)) {
+                        unsigned slot4[4];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) slot4[j] = (unsigned)__shfl((int)slot, 4 * kb + j, 64);
+                        emit(sel4, sco, slot4);
+                    }
+                }
+            }
+            if (!want_attn) continue;  // uniform in the launch
+
+            // ---- the best selected score of every head in my rows of this round --------------------
+            zmax = fmaxf(zmax, __shfl_xor(zmax, 16, 64));
+            zmax = fmaxf(zmax, __shfl_xor(zmax, 32, 64));
+            const float rmax = zmax;
+#ifdef HIRA_TIMELINE
+            if (r == 0) HIRA_TL(9);
+            if (threadIdx.x == 0 && r == 0) { tl[6] = (unsigned long long)tot; tl[12] = (unsigned long long)rounds; }
+#endif
+            if (tot == 0) continue;  // uniform in the wave: nothing selected in my rows
+
+            // the new maximum of every head, and what it does to the sums so far; head g lives in
+            // lane g; the weights below are computed with lane = (row, head), head = lane % GS
+            const float mnew = fmaxf(m_run, rmax);
+            const float f = (m_run == mnew) ? 1.0f : exp2f(m_run - mnew);
+            m_run = mnew;
+            // a head without a selected key has m = -inf and only z = -inf: any finite stand-in
+            const float m_lane = __shfl(mnew == -INFINITY ? 0.0f : mnew, lane_o & (GS - 1), 64);
+            if (__ballot(f != 1.0f) != 0ull) {  // uniform
+                l_mine *= __shfl(f, lane_o & (GS - 1), 64);
+#pragma unroll
+                for (int g = 0; g < GS; ++g) {
+                    const float fg = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), g));
+#pragma unroll
+                    for (int e = 0; e < VPL; ++e) acc[g][e] *= fg;
+                }
+            }
+
+            // ---- gather my listed rows ------------------------------------------------------------
             auto consume = [&](int e0, const int (&at_v)[NPASS], const uint32_t (&vraw)[kVBatch][VW]) {
                 // (nothing of what follows may be scheduled ahead of loads issued before this point)
                 __builtin_amdgcn_sched_barrier(0);
@@ -739,7 +976,8 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                     }
                 }
             };
-            for (int e0 = 0; e0 < tot; e0 += kVBatch) {  // uniform in the wave
+            if constexpr (Q8) consume(0, at_v0, vraw0);
+            for (int e0 = Q8 ? kVBatch : 0; e0 < tot; e0 += kVBatch) {  // uniform in the wave
                 int at_v[NPASS];
                 uint32_t vraw[kVBatch][VW];
                 issue(e0, at_v, vraw);
@@ -903,36 +1141,40 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     HIRA_TL(5);
 }
 
-template <int KS, int MT>
+template <int KS, int MT, bool Q8>
 void launch_mfma_gs(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s) {
     const dim3 block(plan.threads);
     const bool out = p.dense != nullptr || p.sel_count != nullptr;
     if (plan.gmax <= 4) {
-        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 4, true>), grid, block, 0, s, p);
-        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 4, false>), grid, block, 0, s, p);
+        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 4, true, Q8>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 4, false, Q8>), grid, block, 0, s, p);
     } else if (plan.gmax <= 8) {
-        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 8, true>), grid, block, 0, s, p);
-        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 8, false>), grid, block, 0, s, p);
+        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 8, true, Q8>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 8, false, Q8>), grid, block, 0, s, p);
     } else {
-        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 16, true>), grid, block, 0, s, p);
-        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 16, false>), grid, block, 0, s, p);
+        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 16, true, Q8>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 16, false, Q8>), grid, block, 0, s, p);
     }
 }
 
-template <int KS>
+template <int KS, bool Q8>
 void launch_mfma_mt(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s) {
     const int mt = p.bf / 16;
     if (mt <= 1)
-        launch_mfma_gs<KS, 1>(plan, p, grid, s);
+        launch_mfma_gs<KS, 1, Q8>(plan, p, grid, s);
     else if (mt == 2)
-        launch_mfma_gs<KS, 2>(plan, p, grid, s);
+        launch_mfma_gs<KS, 2, Q8>(plan, p, grid, s);
     else
-        launch_mfma_gs<KS, 4>(plan, p, grid, s);
+        launch_mfma_gs<KS, 4, Q8>(plan, p, grid, s);
 }
 
-// one translation unit per key width keeps the build parallel
+// one translation unit per key width (and per kind of scan: bf16 tiles, 8-bit shadow) keeps the
+// build parallel
 void launch_mfma_d64(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
 void launch_mfma_d128(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
 void launch_mfma_d256(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
+void launch_mfma_q8_d64(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
+void launch_mfma_q8_d128(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
+void launch_mfma_q8_d256(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
 
 }  // namespace hira

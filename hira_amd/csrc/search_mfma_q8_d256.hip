@@ -1,0 +1,8 @@
+// MFMA search kernel instantiations for D = 256, keys scanned through their 8-bit shadow.
+#include "search_mfma_kernel.h"
+
+namespace hira {
+void launch_mfma_q8_d256(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s) {
+    launch_mfma_mt<8, true>(plan, p, grid, s);
+}
+}  // namespace hira

@@ -35,7 +35,11 @@ struct UpdateParams {
     float* radii[HIRA_MAX_LEVELS];
     int32_t* counts[HIRA_MAX_LEVELS];
     int32_t cap[HIRA_MAX_LEVELS];
-    int32_t num_levels, bf, dim, vdim, layout;
+    int32_t num_levels, bf, dim, vdim, layout;  // layout: of the centers
+    int32_t key_layout;
+    int8_t* keys8;        // HIRA_TILE16_Q8: the 8-bit shadow of the keys
+    const float* kscale;  //   its step per tree and channel
+    float* keps;          //   largest error, in steps, among the keys of each level-1 node
     const void* new_keys;    // (T, m, D)
     const void* new_values;  // (T, m, Dv) or NULL
     int32_t m;
@@ -206,7 +210,29 @@ __global__ __launch_bounds__(kUpdThreads) void k_update(const UpdateParams p) {
             const T* dummy = nullptr;
             (void)dummy;
             for (int j = t; j < D; j += kUpdThreads)
-                store_elem<T>(p.keys, base0 * D + elem_index(p.layout, D, (size_t)slot, j), x[j]);
+                store_elem<T>(p.keys, base0 * D + elem_index(p.key_layout, D, (size_t)slot, j), x[j]);
+            if (p.keys8 != nullptr) {
+                // the key's 8-bit shadow with the tree's steps; a component beyond +-127 steps
+                // clips, and the node's error bound then covers it
+                float worst = 0.0f;
+                for (int j = t; j < D; j += kUpdThreads) {
+                    const float u = x[j] / p.kscale[(size_t)tree * D + j];
+                    const float r = fminf(fmaxf(rintf(u), -127.0f), 127.0f);
+                    worst = fmaxf(worst, fabsf(u - r));
+                    p.keys8[base0 * D + shadow_index(D, (size_t)slot, j)] = (int8_t)(int)r;
+                }
+                worst = wave_max(worst);
+                if ((t & 63) == 0) red_f[t >> 6] = worst;
+                __syncthreads();
+                if (t == 0) {
+                    float* e = p.keps + (size_t)tree * p.cap[1] + node1;
+                    const float w = fmaxf(fmaxf(red_f[0], red_f[1]), fmaxf(red_f[2], red_f[3]));
+                    // a node that just opened holds no other key: its bound starts here
+                    const bool fresh = p.counts[1][(size_t)tree * p.cap[1] + node1] == 1;
+                    *e = fresh ? w : fmaxf(*e, w);
+                }
+                __syncthreads();
+            }
             if (p.new_values && p.values) {
                 const size_t vs = ((size_t)tree * p.m + i) * Dv;
                 for (int j = t; j < Dv; j += kUpdThreads)
@@ -294,7 +320,15 @@ extern "C" int hira_update(const HiraTree* tree, const void* new_keys, const voi
     p.bf = tree->bf;
     p.dim = tree->dim;
     p.vdim = tree->vdim;
-    p.layout = tree->layout;
+    p.layout = center_layout_of(tree->layout);
+    p.key_layout = key_layout_of(tree->layout);
+    if (tree->layout == HIRA_TILE16_Q8) {
+        HIRA_CHECK_ARG(tree->keys8 && tree->kscale && tree->keps && tree->num_levels >= 2,
+                       "keys8 / kscale / keps missing");
+        p.keys8 = tree->keys8;
+        p.kscale = tree->kscale;
+        p.keps = tree->keps;
+    }
     p.new_keys = new_keys;
     p.new_values = new_values;
     p.m = m;

@@ -104,10 +104,18 @@ class HIPIndexer(BaseIndexer):
         self.pad_value = pad_value
         self.seed = int(seed)
         self.pack_rounds = int(pack_rounds)
-        if layout not in ("auto", "row_major", "tiled"):
-            raise ValueError("layout must be 'auto', 'row_major' or 'tiled'")
+        if layout not in ("auto", "row_major", "tiled", "q8"):
+            raise ValueError("layout must be 'auto', 'row_major', 'tiled' or 'q8'")
         self.layout_request = layout
-        self.tiled = False  # keys / centers stored in the MFMA tile arrangement
+        self.tiled = False  # centers (and, unless q8, keys) stored in the MFMA tile arrangement
+        # q8: tiled centers, row-major keys and beside them an 8-bit shadow copy of the keys
+        # (keys8, one step per tree and channel in kscale, error bounds per level-1 node in
+        # keps) that the search scans first; bf16 rows are then fetched only for the keys the
+        # shadow cannot rule out
+        self.q8 = False
+        self.keys8: Optional[torch.Tensor] = None
+        self.kscale: Optional[torch.Tensor] = None
+        self.keps: Optional[torch.Tensor] = None
         self.capacity = capacity  # key slots to reserve per tree (room for appends)
         # update() calls with at least this many keys per tree build a sub-tree over the new
         # keys and graft it at the tail instead of placing the keys one by one
@@ -148,10 +156,18 @@ class HIPIndexer(BaseIndexer):
     def _head_view(self, t: torch.Tensor, n: int, rows: bool = False) -> torch.Tensor:
         """(T, cap, ...) -> (H, n, ...) for batch 1, (B, H, n, ...) otherwise.  `rows`: t is
         a key / centre matrix; it is returned row-major (a copy when the index is tiled)."""
-        if rows and self.tiled:
+        if rows and (self.keys_tiled if t is self.keys_buf else self.tiled):
             t = from_tiled(t)
         v = t[:, :n]
         return v if self.batch == 1 else v.reshape(self.batch, self.num_heads, *v.shape[1:])
+
+    @property
+    def keys_tiled(self) -> bool:
+        return self.tiled and not self.q8
+
+    @property
+    def layout_name(self) -> str:
+        return "q8" if self.q8 else ("tiled" if self.tiled else "row_major")
 
     @property
     def children(self):
@@ -159,7 +175,7 @@ class HIPIndexer(BaseIndexer):
 
     def keys_rowmajor(self) -> torch.Tensor:
         """(T, N_pad, D) keys in slot order, row-major (a copy when the index is tiled)."""
-        k = from_tiled(self.keys_buf) if self.tiled else self.keys_buf
+        k = from_tiled(self.keys_buf) if self.keys_tiled else self.keys_buf
         return k[:, : self.size[0]]
 
     def centers_rowmajor(self, l: int) -> torch.Tensor:
@@ -225,8 +241,13 @@ class HIPIndexer(BaseIndexer):
         tile_ok = (dtype == torch.bfloat16 and dim % 32 == 0)
         if self.layout_request == "tiled" and not tile_ok:
             raise ValueError("the tiled layout needs bfloat16 keys with dim a multiple of 32")
+        q8_ok = tile_ok and dim % 64 == 0 and dim <= 256 and nl >= 2
+        if self.layout_request == "q8" and not q8_ok:
+            raise ValueError("the q8 layout needs bfloat16 keys with dim 64, 128, 192 or 256 and at "
+                             "least two levels")
+        self.q8 = self.layout_request == "q8"
         self.tiled = tile_ok and (
-            self.layout_request == "tiled"
+            self.layout_request in ("tiled", "q8")
             or (self.layout_request == "auto" and nl >= 2 and bf % 16 == 0
                 and dim in (64, 128, 256) and vdim in (0, dim)))
         if self.tiled:
@@ -236,6 +257,11 @@ class HIPIndexer(BaseIndexer):
         self.values_buf = (
             torch.zeros((t, self.cap[0], vdim), dtype=dtype, device=dev) if vdim else None)
         self.perm = torch.full((t, self.cap[0]), -1, dtype=torch.int32, device=dev)
+        self.keys8 = self.kscale = self.keps = None
+        if self.q8:
+            self.keys8 = torch.zeros((t, self.cap[0], dim), dtype=torch.int8, device=dev)
+            self.kscale = torch.ones((t, dim), dtype=torch.float32, device=dev)
+            self.keps = torch.zeros((t, self.cap[1]), dtype=torch.float32, device=dev)
         self.centers, self.radii, self.counts = [None], [None], [None]
         for l in range(1, nl):
             self.centers.append(torch.zeros((t, self.cap[l], dim), dtype=dtype, device=dev))
@@ -256,7 +282,11 @@ class HIPIndexer(BaseIndexer):
             t.bf = self.branching_factor
             t.dim, t.vdim = self.dim, self.vdim
             t.dtype = _DTYPES[self.dtype]
-            t.layout = _lib.HIRA_TILE16 if self.tiled else _lib.HIRA_ROW_MAJOR
+            t.layout = (_lib.HIRA_TILE16_Q8 if self.q8 else
+                        _lib.HIRA_TILE16 if self.tiled else _lib.HIRA_ROW_MAJOR)
+            if self.q8:
+                t.keys8, t.kscale = self.keys8.data_ptr(), self.kscale.data_ptr()
+                t.keps = self.keps.data_ptr()
             for l in range(self.num_levels):
                 t.size[l], t.cap[l] = self.size[l], self.cap[l]
             t.keys = self.keys_buf.data_ptr()
@@ -288,7 +318,7 @@ class HIPIndexer(BaseIndexer):
         if self.size[0] != n_pad:
             raise ValueError(f"keys have {n_pad} slots, layout needs {self.size[0]}")
         self.keys_buf[:, :n_pad] = keys.to(device=self.device, dtype=dtype)
-        if self.tiled:
+        if self.keys_tiled:
             self.keys_buf.copy_(to_tiled(self.keys_buf))
         if values is not None:
             self.values_buf[:, :n_pad] = torch.as_tensor(values).to(device=self.device,
@@ -303,6 +333,26 @@ class HIPIndexer(BaseIndexer):
             self.radii[l][:, :k] = torch.as_tensor(radii[l]).to(self.device, torch.float32)
             self.counts[l][:, :k] = torch.as_tensor(counts[l]).to(self.device, torch.int32)
         self.num_keys = int(num_keys if num_keys is not None else (perm[0] >= 0).sum().item())
+        if self.q8:
+            self.quantize(new_steps=True)
+        return self
+
+    def quantize(self, slot_first: int = 0, slot_count: Optional[int] = None,
+                 new_steps: bool = False) -> "HIPIndexer":
+        """(Re)make the 8-bit shadow of the keys in slots [slot_first, +slot_count) of every tree
+        (whole level-1 nodes; default: all slots in use) from the bf16 keys as they stand;
+        ``new_steps`` first derives the step of every channel from all keys (then the whole
+        shadow must be remade).  A q8 index only; one or four small launches."""
+        if not self.q8:
+            return self
+        bf = self.branching_factor
+        if slot_count is None:
+            slot_count = self.size[0] - slot_first
+        slot_count = -(-slot_count // bf) * bf
+        tree = self.tree_struct()
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        _lib.check(_lib.lib().hira_quantize(C.byref(tree), int(slot_first), int(slot_count),
+                                            1 if new_steps else 0, stream))
         return self
 
     # ------------------------------------------------------------------ persistence
@@ -329,11 +379,15 @@ class HIPIndexer(BaseIndexer):
             tensors[f"counts.{l}"] = self.counts[l][:, : rows[l]]
         if self._state is not None:
             tensors["update_state"] = self._state
+        if self.q8:
+            tensors["keys8"] = self.keys8[:, : rows[0]]
+            tensors["kscale"] = self.kscale
+            tensors["keps"] = self.keps[:, : rows[1]]
         meta = {
             "format": "hira_amd.index.v1", "num_levels": self.num_levels,
             "branching_factor": self.branching_factor, "max_iterations": self.max_iterations,
             "pack_rounds": self.pack_rounds, "seed": self.seed, "pad_value": self.pad_value,
-            "layout_request": self.layout_request, "tiled": self.tiled, "batch": self.batch,
+            "layout_request": self.layout_request, "tiled": self.tiled, "q8": self.q8, "batch": self.batch,
             "num_heads": self.num_heads, "dim": self.dim, "vdim": self.vdim,
             "dtype": "bfloat16" if self.dtype == torch.bfloat16 else "float32",
             "size": list(self.size), "rows": rows, "num_keys": self.num_keys,
@@ -365,7 +419,7 @@ class HIPIndexer(BaseIndexer):
         # room for what the file holds (and for `capacity`), then the saved sizes
         self._allocate(meta["batch"], meta["num_heads"], max(rows[0], 1), meta["dim"],
                        meta["vdim"], dtype)
-        if self.tiled != bool(meta["tiled"]):
+        if self.tiled != bool(meta["tiled"]) or self.q8 != bool(meta.get("q8", False)):
             raise ValueError(f"{path}: stored layout does not match what this build would choose")
         self.size = list(rows)
         self._grow(rows)
@@ -388,6 +442,10 @@ class HIPIndexer(BaseIndexer):
             put(self.counts[l], f"counts.{l}")
         if "update_state" in tensors:
             self._state = tensors["update_state"].to(self.device)
+        if self.q8:
+            put(self.keys8, "keys8")
+            self.kscale.copy_(tensors["kscale"].to(self.device))
+            put(self.keps, "keps")
         self.num_keys = int(meta["num_keys"])
         self._tree_struct = None
         return self
@@ -488,6 +546,9 @@ class HIPIndexer(BaseIndexer):
         if self.values_buf is not None:
             self.values_buf = grown(self.values_buf, caps[0], 0)
         self.perm = grown(self.perm, caps[0], -1)
+        if self.q8:
+            self.keys8 = grown(self.keys8, caps[0], 0)
+            self.keps = grown(self.keps, caps[1], 0)
         for l in range(1, self.num_levels):
             self.centers[l] = grown(self.centers[l], caps[l], 0)
             self.radii[l] = grown(self.radii[l], caps[l], float("-inf"))
@@ -533,10 +594,10 @@ class HIPIndexer(BaseIndexer):
         bf, nl = self.branching_factor, self.num_levels
         sub = HIPIndexer(sub_levels, self.max_iterations, bf, seed=self.seed + self.num_keys,
                          device=str(self.device), pack_rounds=self.pack_rounds,
-                         layout="tiled" if self.tiled else "row_major", graft_min=1 << 62)
+                         layout=self.layout_name, graft_min=1 << 62)
         sub.build(new_keys.to(self.device, self.dtype),
                   None if new_values is None else new_values.to(self.device, self.dtype))
-        if sub.tiled != self.tiled:
+        if sub.tiled != self.tiled or sub.q8 != self.q8:
             raise RuntimeError("sub-tree layout differs from the index's")
         stop = sub_levels - 1  # the sub-tree's top level, as a level of the index
         r16 = (lambda n: -(-n // 16) * 16) if self.tiled else (lambda n: n)
@@ -566,10 +627,12 @@ class HIPIndexer(BaseIndexer):
         n0 = sub.size[0]
         sp = sub.perm[:, :n0]
         sp = torch.where(sp >= 0, sp + self.num_keys, torch.full_like(sp, -1))
+        quant = []  # key slot ranges whose 8-bit shadow has to be remade (q8)
         for (trees, _), off in zip(groups, offs):
             # level 0 and the inner levels start at multiples of bf (of 16 where tiled): whole
             # tiles copy as they are
             self.keys_buf[trees, off[0]:off[0] + r16(n0)] = sub.keys_buf[trees, : r16(n0)]
+            quant.append((off[0], n0))
             if self.values_buf is not None:
                 self.values_buf[trees, off[0]:off[0] + n0] = sub.values_buf[trees, :n0]
             self.perm[trees, off[0]:off[0] + n0] = sp[trees]
@@ -607,6 +670,8 @@ class HIPIndexer(BaseIndexer):
         self._state[:, _lib.HIRA_MAX_LEVELS] += m
         self.num_keys += m
         self._tree_struct = None
+        for first, count in quant:  # with the index's own steps (a sub-tree has others)
+            self.quantize(first, count)
         return self
 
     def reserve(self, appends: int) -> "HIPIndexer":
@@ -774,11 +839,11 @@ class HIPIndexer(BaseIndexer):
             if n == 0:
                 continue
             rows = self.keys_buf[t:t + 1, s0:s1]
-            rows = (from_tiled(rows) if self.tiled else rows)[0, live]
+            rows = (from_tiled(rows) if self.keys_tiled else rows)[0, live]
             vals = None if self.values_buf is None else self.values_buf[t, s0:s1][live]
             sub = HIPIndexer(2, self.max_iterations, bf, seed=self.seed + node,
                              device=str(self.device), pack_rounds=self.pack_rounds,
-                             layout="tiled" if self.tiled else "row_major")
+                             layout=self.layout_name)
             sub.build(rows[None, None], None if vals is None else vals[None, None])
             k, m = sub.size[1], sub.size[0]  # level-1 nodes and key slots the subtree uses now
             # keys, values, positions: the rebuilt slots first, the rest of the subtree empty
@@ -816,4 +881,5 @@ class HIPIndexer(BaseIndexer):
                 self.radii[l][t, child] = r
                 c_child, r_child, child = cl, r, child // bf
         self._tree_struct = None
+        self.quantize(s0, s1 - s0)
         return self

@@ -33,6 +33,7 @@ extern "C" {
 
 #define HIRA_ABI_VERSION 4
 #define HIRA_MAX_LEVELS 8
+#define HIRA_STATS_COLS (HIRA_MAX_LEVELS + 3) /* counters per tree a search can fill in */
 
 enum { HIRA_F32 = 0, HIRA_BF16 = 1 };
 
@@ -42,7 +43,18 @@ enum { HIRA_F32 = 0, HIRA_BF16 = 1 };
  * [32 s + 8 kb, +8) of row 16 tile + i sits at chunk index (tile*(D/32) + s)*64 + kb*16 + i,
  * i.e. one wave-wide 128-bit load fetches a complete 16x32 MFMA operand tile from 1 KiB of
  * contiguous memory.  Values, radii, counts and perm are never tiled. */
-enum { HIRA_ROW_MAJOR = 0, HIRA_TILE16 = 1 };
+enum { HIRA_ROW_MAJOR = 0, HIRA_TILE16 = 1, HIRA_TILE16_Q8 = 2 };
+/* HIRA_TILE16_Q8 (bf16 only, D a multiple of 64, every cap a multiple of 16): the centers of
+ * every level are tiled as in HIRA_TILE16, the keys are ROW-MAJOR, and beside them sits an
+ * 8-bit shadow copy `keys8` that the search scans first: k8 = round(k / kscale[channel]),
+ * clipped to [-127, 127], with one step `kscale` per tree and channel, in tiles of 16 rows x
+ * 64 columns -- the 16-byte chunk holding columns [64 s + 16 kb, +16) of row 16 tile + i sits
+ * at chunk index (tile*(D/64) + s)*64 + kb*16 + i, one wave-wide 128-bit load per 16x64 tile.
+ * keps[node] bounds |k/kscale - k8| over all channels of all keys of level-1 node `node`
+ * (0.5 unless a key appended later clipped).  A key whose 8-bit score plus the error bound
+ * these numbers give stays below the threshold cannot be selected; only the others have
+ * their bf16 row fetched and tested exactly, so the selected set is that of the other
+ * layouts bit for bit. */
 
 enum {
     HIRA_OK = 0,
@@ -58,7 +70,7 @@ typedef struct HiraTree {
     int32_t dim;        /* key / query / center dim D; D*elem_size a multiple of 16 B */
     int32_t vdim;       /* value dim Dv (0 if there are no values) */
     int32_t dtype;
-    int32_t layout;     /* HIRA_ROW_MAJOR or HIRA_TILE16 */
+    int32_t layout;     /* HIRA_ROW_MAJOR, HIRA_TILE16 or HIRA_TILE16_Q8 */
     int32_t reserved_;  /* keeps the arrays below 8-byte aligned; must be 0 */
     int32_t size[HIRA_MAX_LEVELS];
     int32_t cap[HIRA_MAX_LEVELS];
@@ -68,6 +80,11 @@ typedef struct HiraTree {
     void* centers[HIRA_MAX_LEVELS];  /* [l >= 1] (T, cap[l], D), stored as `layout` says */
     float* radii[HIRA_MAX_LEVELS];   /* [l >= 1] (T, cap[l]) */
     int32_t* counts[HIRA_MAX_LEVELS];/* [l >= 1] (T, cap[l]) */
+    /* HIRA_TILE16_Q8 only (NULL otherwise): */
+    int8_t* keys8;                   /* (T, cap[0], D) 8-bit shadow of the keys, tiled 16 x 64 */
+    float* kscale;                   /* (T, D) step of the shadow per tree and channel */
+    float* keps;                     /* (T, cap[1]) largest rounding/clipping error, in steps,
+                                        among the keys of each level-1 node */
 } HiraTree;
 
 /* One decode step's queries.  Query head h belongs to tree q2tree order given as CSR:
@@ -117,10 +134,11 @@ typedef struct HiraSearchOut {
     /* (3) attention over the selected keys (+ the queue): out (H_q, Dv) fp32.
      *     Heads with an empty selection get zeros. */
     float* attn_out;
-    /* optional counters, zeroed by the caller: (T, HIRA_MAX_LEVELS+2) uint64:
+    /* optional counters, zeroed by the caller: (T, HIRA_STATS_COLS) uint64:
      *     [l] nodes of level l evaluated by at least one head of the tree's group
      *     (l = 0: candidate keys), [HIRA_MAX_LEVELS] keys selected by at least one head,
-     *     [HIRA_MAX_LEVELS+1] (key, head) selections. */
+     *     [HIRA_MAX_LEVELS+1] (key, head) selections, [HIRA_MAX_LEVELS+2] keys whose bf16 row
+     *     was fetched for the exact test after the 8-bit scan (HIRA_TILE16_Q8; else 0). */
     unsigned long long* stats;
 } HiraSearchOut;
 
@@ -245,6 +263,19 @@ int hira_nearest(const void* x, int32_t dtype, int32_t num_trees, int32_t n,
  */
 int hira_update(const HiraTree* tree, const void* new_keys, const void* new_values, int32_t m,
                 int32_t* state, void* stream);
+
+/*
+ * (Re)compute the 8-bit shadow of a HIRA_TILE16_Q8 index from its bf16 keys, for the key slots
+ * [slot_first, slot_first + slot_count) of every tree (whole level-1 nodes: both multiples of
+ * bf): keys8 for those slots and keps for their nodes.  recompute_scale != 0 first derives
+ * kscale from ALL key slots [0, size[0]) (largest magnitude per channel / 127) and then needs
+ * the whole range.  hira_build calls this itself; callers that move keys around afterwards
+ * (grafting a sub-tree, re-clustering a subtree, restoring a file) call it for what they
+ * touched.  Empty slots (perm < 0) hold zeros and do not count.  No counterpart in the
+ * reference, which keeps fp32 keys only (indexer/cuda.py:365-368).
+ */
+int hira_quantize(const HiraTree* tree, int32_t slot_first, int32_t slot_count,
+                  int32_t recompute_scale, void* stream);
 
 /*
  * Per-head thresholds from a sample of each tree's keys, in one launch ahead of hira_search

@@ -129,7 +129,7 @@ def test_mfma_kernel_matches_oracle_and_vector_kernel(case, gpu_device):
     stats = {}
     for kernel in (2, 1):
         se = HIPSearcher(kernel=kernel)
-        st = torch.zeros((h_kv, _lib.HIRA_MAX_LEVELS + 2), dtype=torch.int64, device="cuda")
+        st = torch.zeros((h_kv, _lib.HIRA_STATS_COLS), dtype=torch.int64, device="cuda")
         out = se.search(q, th, c["idx"], scaling=sc, stats=st).cpu().numpy()
         assert_same_selection(out != 0, s, c["th"])
         m = out != 0
@@ -200,7 +200,7 @@ def test_device_counters_match_oracle_traffic(gpu_device):
     from hira_amd import _lib
 
     c = _setup(2, 8, 4096, 64, 16, 3, torch.float32, seed=8, keep=40)
-    stats = torch.zeros((2, _lib.HIRA_MAX_LEVELS + 2), dtype=torch.int64, device="cuda")
+    stats = torch.zeros((2, _lib.HIRA_STATS_COLS), dtype=torch.int64, device="cuda")
     HIPSearcher().search(torch.from_numpy(c["q"]), torch.from_numpy(c["th"]), c["idx"], stats=stats)
     tree, csr = ho.fixed_fanout_as_cpu_tree(c["ff"])
     tr = ho.group_traffic(tree, c["q"], c["th"], q2kv=c["q2kv"], csr=csr,
