@@ -169,7 +169,8 @@ struct MfmaShape {
     // after twice the accumulators (GS x D/64) and some seventy registers of everything else
     // (with the 8-bit shadow: also its B operands, one batch of key rows of the exact test and
     // the value rows asked for ahead of it), and what keeps the round's list under 48 KiB of LDS
-    static constexpr int KEY_REGS = 256 - 72 - 2 * GS * (KS / 2) - (Q8 ? 4 * KS + 4 * KS + 32 : 0);
+    static constexpr int KEY_REGS =
+        256 - 72 - 2 * GS * (KS / 2) - (Q8 ? 4 * KS + (KS <= 4 ? 8 : 4) * KS + 32 : 0);
     static constexpr int NB_REGS = KEY_REGS / (MT * KA * 4);
     static constexpr int NB_LDS = (12000 / (GS + 1)) / (kMfmaWaves * ROWS);
     static constexpr int NB_MIN = NB_REGS < NB_LDS ? NB_REGS : NB_LDS;
@@ -395,10 +396,11 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         GateLoads<KS> gl;
         if (tl_mine < ntile) gate_issue<KS, Q8>(p, tree, tile_of(tl_mine), lane, kb, gl);
         if constexpr (Q8) {
-            // ---- the queries in steps of the shadow (wave 0, for all): lane (kb, head) takes
+            // ---- the queries in steps of the shadow (the last wave, which has the fewest tiles to
+            // gate, for all): lane (kb, head) takes
             // columns [64 s + 16 kb, +16) as the shadow's tiles hold them: u_j = q_j kscale_j,
             // the head's step su = max_j |u_j| / kQ8Steps, U_j = round(u_j / su) in two bytes -------
-            if (wave == 0) {
+            if (wave == nw - 1) {
                 float uf[KS8][16];
                 float umax = 0.0f, asum = 0.0f;
 #pragma unroll
@@ -440,6 +442,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 asum += __shfl_xor(asum, 16, 64);
                 asum += __shfl_xor(asum, 32, 64);
                 const float su = fmaxf(umax, 1e-30f) / kQ8Steps;
+                const float inv = kQ8Steps / fmaxf(umax, 1e-30f);  // (u * inv: within 0.004 of u / su)
 #pragma unroll
                 for (int s = 0; s < KS8; ++s) {
                     uint32_t hi[4], lo[4];
@@ -449,7 +452,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                         lo[c] = 0u;
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
-                            const int U = (int)rintf(uf[s][4 * c + e] / su);
+                            const int U = (int)rintf(uf[s][4 * c + e] * inv);
                             const int h = (U + 128) >> 8;  // U = 256 h + l, l in [-128, 127]
                             const int l = U - (h << 8);
                             hi[c] |= ((uint32_t)h & 0xFFu) << (8 * e);
@@ -639,14 +642,26 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 if constexpr (Q8) nx_eps[u] = s_keps[max(n, 0)];
                 const unsigned tile_first = (unsigned)(node_of(max(n, 0)) * bf) / 16u;
 #pragma unroll
-                for (int tt = 0; tt < MT; ++tt)
-                    if (tt * 16 < nx_cnt[u])
-                        load_tile_buf<KA>(Q8 ? k8rsrc : krsrc, (unsigned)lane * 16u,
+                for (int tt = 0; tt < MT; ++tt) {
+                    if constexpr (Q8) {
+                        // every load is issued, whatever the node (straight-line code, so that the
+                        // waits further down can count the loads behind them); a tile that is not
+                        // there is asked for beyond the end of the buffer: zeros, no memory access
+                        load_tile_buf<KA>(k8rsrc, (unsigned)lane * 16u + (tt * 16 < nx_cnt[u] ? 0u : 0x80000000u),
                                           (tile_first + tt) * (unsigned)(KA * 1024), a[u][tt]);
+                    } else {
+                        if (tt * 16 < nx_cnt[u])
+                            load_tile_buf<KA>(krsrc, (unsigned)lane * 16u,
+                                              (tile_first + tt) * (unsigned)(KA * 1024), a[u][tt]);
+                    }
+                }
             }
         };
         if (rounds > 0) fetch(0, -1);
 
+        constexpr int KB0 = KS <= 4 ? 2 : 1;      // batches of 16 key rows asked for ahead
+        constexpr int RP = 64 / GS;               // rows whose weights one pass over the lanes computes
+        constexpr int NPASS = kVBatch / RP;       // GS = 4: 2, GS = 8: 4, GS = 16: 8
         for (int r = 0; r < rounds; ++r) {  // uniform in the workgroup
             // the round's score table and row list; every wave has a stretch of ROWS * NB rows of
             // its own and nobody else looks at it: no barrier inside the rounds
@@ -747,9 +762,8 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                     const float eps_u = nx_eps[u];
                     i32x4_t est_u[MT];
 #pragma unroll
-                    for (int tt = 0; tt < MT; ++tt)
-                        if (tt * 16 < cnt[u]) est_u[tt] = tile_scores_i8<KS8>(a[u][tt], bq8h, bq8l);
-                    if (r + 1 < rounds) fetch(r + 1, u);
+                    for (int tt = 0; tt < MT; ++tt)  // (every tile: one that is not there came as zeros)
+                        est_u[tt] = tile_scores_i8<KS8>(a[u][tt], bq8h, bq8l);
                     // the score q.k lies within `marg` of su * (the integer): the keys' rounding
                     // (eps_u steps a component at most) and the query's (kQ8QuerySlack steps of su)
                     const float marg = (eps_u + kQ8KeySlack) * asum + su * (kQ8QuerySlack * 127.0f * (float)D);
@@ -834,11 +848,10 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 }  // shadow or bf16 tiles
             }
             const int tot = nsel;  // rows on my list
+            if (r == 0) HIRA_TL(10);
 
             // ---- value rows: kVBatch in flight; the rows of a batch in the score table (lane =
             // (row of the pass, head)), their key slots, and the loads ---------------------------------
-            constexpr int RP = 64 / GS;          // rows whose weights one pass over the lanes computes
-            constexpr int NPASS = kVBatch / RP;  // GS = 4: 2, GS = 8: 4, GS = 16: 8
             auto issue = [&](int e0, int (&at_v)[NPASS], uint32_t (&vraw)[kVBatch][VW]) {
 #pragma unroll
                 for (int ps = 0; ps < NPASS; ++ps) {
@@ -868,59 +881,57 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                     }
                 }
             };
-            int at_v0[Q8 ? NPASS : 1];
-            uint32_t vraw0[Q8 ? kVBatch : 1][VW];
-            if constexpr (Q8) {
-                // the value rows of the first batch are asked for ahead of the key rows: most rows
-                // that the shadow lets through are selected
-                if (want_attn && tot > 0) issue(0, at_v0, vraw0);
-                // ---- the exact test: the listed rows' bf16 keys, 16 at a time as one A operand
-                // (lane (kb, i): columns [32 s + 8 kb, +8) of the i-th of them) -----------------------
-                for (int e0 = 0; e0 < tot; e0 += 16) {  // uniform in the wave
-                    const int le = e0 + (lane_o & 15);
-                    const int at = le < tot ? (int)lst_row[zrow0 + le] : -1;  // (-1: past the end)
-                    const unsigned slot = at >= 0 ? lst_tslot[at >> 4] + (unsigned)(at & 15) : 0u;
-                    uint4 kr[KS];
+            // ---- the exact test (8-bit shadow): the listed rows' bf16 keys, 16 at a time as one A
+            // operand (lane (kb, i): columns [32 s + 8 kb, +8) of the i-th of them) ---------------------
+            auto rows16 = [&](int e0, int& at, unsigned& slot, uint4 (&kr)[KS]) {
+                const int le = e0 + (lane_o & 15);
+                at = le < tot ? (int)lst_row[zrow0 + le] : -1;  // (-1: past the end)
+                slot = at >= 0 ? lst_tslot[at >> 4] + (unsigned)(at & 15) : 0u;
 #pragma unroll
-                    for (int s = 0; s < KS; ++s)
-                        kr[s] = __builtin_bit_cast(
-                            uint4, __builtin_amdgcn_raw_buffer_load_b128(
-                                       krsrc, slot * (unsigned)(D * 2) + (unsigned)(kb * 16 + s * 64), 0, 0));
-                    const f32x4_t sco = tile_scores_lds<KS>(kr, s_bq, lane_o);
-                    unsigned sel4 = 0u;
-                    int at4[4];
+                for (int s = 0; s < KS; ++s)
+                    kr[s] = __builtin_bit_cast(
+                        uint4, __builtin_amdgcn_raw_buffer_load_b128(
+                                   krsrc, slot * (unsigned)(D * 2) + (unsigned)(kb * 16 + s * 64), 0, 0));
+            };
+            auto exact16 = [&](int at, unsigned slot, const uint4 (&kr)[KS]) {
+                const f32x4_t sco = tile_scores_lds<KS>(kr, s_bq, lane_o);
+                unsigned sel4 = 0u;
+                int at4[4];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        at4[j] = __shfl(at, 4 * kb + j, 64);
-                        const bool mine = col < GS && at4[j] >= 0;
-                        // (the table holds 0 where the shadow let the row pass for my head)
-                        const float pz = mine ? lst_z[at4[j] * GS + col] : -INFINITY;
-                        const bool sel = pz == 0.0f && sco[j] >= tau;
-                        if (sel) sel4 |= 1u << j;
-                        const float z = sel ? sco[j] * sc2 : -INFINITY;
-                        zmax = fmaxf(zmax, z);
-                        if (mine) lst_z[at4[j] * GS + col] = z;
-                    }
-                    if (stats) count_selected(sel4, rows_of(sel4));
-                    if (OUT && (p.dense != nullptr || p.sel_count != nullptr)) {
-                        unsigned slot4[4];
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) slot4[j] = (unsigned)__shfl((int)slot, 4 * kb + j, 64);
-                        emit(sel4, sco, slot4);
-                    }
+                for (int j = 0; j < 4; ++j) {
+                    at4[j] = __shfl(at, 4 * kb + j, 64);
+                    const bool mine = col < GS && at4[j] >= 0;
+                    // (the table holds 0 where the shadow let the row pass for my head)
+                    const float pz = mine ? lst_z[at4[j] * GS + col] : -INFINITY;
+                    const bool sel = pz == 0.0f && sco[j] >= tau;
+                    if (sel) sel4 |= 1u << j;
+                    const float z = sel ? sco[j] * sc2 : -INFINITY;
+                    zmax = fmaxf(zmax, z);
+                    if (mine) lst_z[at4[j] * GS + col] = z;
                 }
-            }
-            if (!want_attn) continue;  // uniform in the launch
+                if (stats) count_selected(sel4, rows_of(sel4));
+                if (OUT && (p.dense != nullptr || p.sel_count != nullptr)) {
+                    unsigned slot4[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) slot4[j] = (unsigned)__shfl((int)slot, 4 * kb + j, 64);
+                    emit(sel4, sco, slot4);
+                }
+            };
+            // ---- what is left to do with the rows of a round (`pr`; the lists and `tot` are its):
+            // the best selected score of every head, the sums rescaled to it, the value rows ----------
+            auto finish = [&](int pr, const int (&at_v0)[NPASS], const uint32_t (&vraw0)[kVBatch][VW]) {
+                (void)pr;
+            if (!want_attn) return;  // uniform in the launch
 
             // ---- the best selected score of every head in my rows of this round --------------------
             zmax = fmaxf(zmax, __shfl_xor(zmax, 16, 64));
             zmax = fmaxf(zmax, __shfl_xor(zmax, 32, 64));
             const float rmax = zmax;
 #ifdef HIRA_TIMELINE
-            if (r == 0) HIRA_TL(9);
-            if (threadIdx.x == 0 && r == 0) { tl[6] = (unsigned long long)tot; tl[12] = (unsigned long long)rounds; }
+            if (pr == 0) HIRA_TL(9);
+            if (threadIdx.x == 0 && pr == 0) { tl[6] = (unsigned long long)tot; tl[12] = (unsigned long long)rounds; }
 #endif
-            if (tot == 0) continue;  // uniform in the wave: nothing selected in my rows
+            if (tot == 0) return;  // uniform in the wave: nothing selected in my rows
 
             // the new maximum of every head, and what it does to the sums so far; head g lives in
             // lane g; the weights below are computed with lane = (row, head), head = lane % GS
@@ -983,7 +994,45 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 issue(e0, at_v, vraw);
                 consume(e0, at_v, vraw);
             }
-            if (r == 0) HIRA_TL(11);
+            if (pr == 0) HIRA_TL(11);
+            if (pr == 1) HIRA_TL(13);
+            if (pr == 2) HIRA_TL(14);
+            };
+            if constexpr (Q8) {
+                // Order of the requests: the value rows of the first batch (most rows that the shadow
+                // lets through are selected), the key rows of the first KB0 * 16 listed rows, and only
+                // then the tiles of the next round -- loads come back in the order they were asked
+                // for, so the exact test and the gather wait for the rows alone and run while the
+                // next round's tiles are on their way.
+                int at_v0[NPASS], at_k[KB0];
+                uint32_t vraw0[kVBatch][VW];
+                unsigned slot_k[KB0];
+                uint4 kr0[KB0][KS];
+                __builtin_amdgcn_sched_barrier(0);
+                if (want_attn) issue(0, at_v0, vraw0);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int b = 0; b < KB0; ++b) rows16(16 * b, at_k[b], slot_k[b], kr0[b]);
+                __builtin_amdgcn_sched_barrier(0);
+                fetch(r + 1, -1);  // (past the last round: no node, nothing read)
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int b = 0; b < KB0; ++b)
+                    if (16 * b < tot) exact16(at_k[b], slot_k[b], kr0[b]);  // uniform
+                for (int e0 = 16 * KB0; e0 < tot; e0 += 16) {  // uniform in the wave; seldom
+                    int at;
+                    unsigned slot;
+                    uint4 kr[KS];
+                    rows16(e0, at, slot, kr);
+                    exact16(at, slot, kr);
+                }
+                finish(r, at_v0, vraw0);
+            } else {
+                int none_at[NPASS];
+                uint32_t none_v[kVBatch][VW];
+                finish(r, none_at, none_v);
+            }
+            if (r == 3) HIRA_TL(15);
         }
     }  // tree or queue
     if (!want_attn) return;  // uniform
