@@ -11,7 +11,8 @@ HBM bandwidth using the ALGORITHMIC bytes of the walk (nodes evaluated x (d*e + 
 candidate keys x d*e + selected values x d*e + queries + output; counted by the kernel's
 own counters, which the tests tie to the CPU oracle); `cpu_baseline` times the reference's
 own C++ search kernel (compiled into oracle/_ref) -- or, if that is absent, the C
-restatement in oracle/ -- plus a host softmax-V, on a bounded sample of the same steps.
+restatement in oracle/ -- plus a host softmax-V, on a bounded sample of the same steps, and
+the CPU index build (the oracle's restatement of the reference's CPU indexer) of one tree.
 """
 from __future__ import annotations
 
@@ -74,6 +75,26 @@ def measured_traffic(workload_name):
         return None
 
 
+def cpu_index_build(w, keys_slots, perm):
+    """The reference's CPU indexer (indexer/cpu.py:48-122: bottom-up k-means levels, radii from
+    the assignment) on ONE tree of the workload -- a bounded sample: the trees are independent
+    and alike -- restated in oracle/ with a plain Lloyd k-means where the reference calls faiss
+    (not installed here): kind "port", one thread."""
+    import numpy as np
+    from oracle import hira_oracle as ho
+
+    live = perm[0] >= 0
+    keys = np.ascontiguousarray(keys_slots[0][live][np.argsort(perm[0][live])])[None]  # insertion order
+    t0 = time.perf_counter()
+    tree = ho.build_cpu_tree(keys, w.num_levels, w.bf, max_iterations=w.kmeans_iters)
+    dt = time.perf_counter() - t0
+    trees = w.batch * w.h_kv
+    return {"build_ms_one_tree": round(dt * 1e3, 1), "trees": trees, "kind": "port", "cores": 1,
+            "build_ms_all_trees_one_core": round(dt * 1e3 * trees, 1),
+            "levels": [int(l.size) for l in tree.levels], "kmeans_iters": w.kmeans_iters,
+            "sample": "tree 0 of the workload (keys of KV head 0 of sequence 0), built once"}
+
+
 def cpu_baseline(w, index, queries, taus, scale, budget_s=20.0, gpu_out=None, gpu_sel=None):
     """Reference CPU search (+ host softmax-V) on the same trees, first steps of the same
     queries, for about `budget_s` seconds of CPU work; one sequence after the other when the
@@ -85,7 +106,14 @@ def cpu_baseline(w, index, queries, taus, scale, budget_s=20.0, gpu_out=None, gp
     from oracle import hira_oracle as ho
     from oracle.build_ref import load_ref
 
-    threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")), w.h_q)
+    # threads: the host cores this process may use (the box's share of a shared machine is what
+    # OMP_NUM_THREADS says), at most one per query head -- the reference kernel's parallel loop
+    # is over the heads (kernels/cpp/torch_ext_v3.cpp:149)
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count() or 1
+    threads = max(1, min(usable, int(os.environ.get("OMP_NUM_THREADS", "16")), w.h_q))
     torch.set_num_threads(threads)
     n0 = index.size[0]
     keys_all = index.keys_rowmajor().float().cpu().numpy()
@@ -193,6 +221,7 @@ def cpu_baseline(w, index, queries, taus, scale, budget_s=20.0, gpu_out=None, gp
                       f"thresholds); median; p99 {float(np.percentile(times, 99) * 1e6):.0f} us; "
                       f"search = reference v3 C++ kernel, attention = numpy fp32",
                one_thread_us=float(np.median(times1) * 1e6), one_thread_steps=len(times1))
+    res["index_build"] = cpu_index_build(w, keys_all, perm_all)
     if gpu_out is not None:
         res["gpu_vs_cpu"] = {"steps_compared": compared, "attn_max_rel_err": attn_err,
                              "selected_set_mismatches": set_diff if gpu_sel is not None else None,
