@@ -111,6 +111,11 @@ SYMBOLS = {
         [C.POINTER(HiraTree), _vp, _vp, C.c_int32, C.c_int32, C.c_int32, C.c_uint64, _vp,
          C.c_size_t, _vp],
     ),
+    "hira_build_ragged": (
+        C.c_int,
+        [C.POINTER(HiraTree), _vp, _vp, C.c_int32, _vp, C.c_int32, C.c_int32, C.c_uint64, _vp,
+         C.c_size_t, _vp],
+    ),
     "hira_nearest_workspace_bytes": (C.c_size_t, [C.c_int32, C.c_int32, C.c_int32, C.c_int32]),
     "hira_nearest": (
         C.c_int,

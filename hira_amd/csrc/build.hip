@@ -40,14 +40,18 @@ __global__ void k_fill_i32(int32_t* p, size_t n, int32_t v) {
 // ------------------------------------------------------------------------------------
 // 1. initial centroids: item floor((k + u_k) * n_c / K), u_k in [0,1) from the seed
 // ------------------------------------------------------------------------------------
+//    (n_live != NULL: tree t holds n_live[t] <= n_c items, the first ones of its rows)
 template <typename T>
 __global__ void k_init_centroids(const void* x, int n_c, size_t x_tree_stride, int K, int D,
-                                 uint64_t seed, float* cent) {
+                                 uint64_t seed, float* cent, const int32_t* n_live, int bf) {
     const int k = blockIdx.x, t = blockIdx.y;
     const uint64_t h = mix64(seed ^ mix64((uint64_t)t * 0x100000001b3ull + (uint64_t)k));
     const double u = (double)(h >> 11) * (1.0 / 9007199254740992.0);
-    long long idx = (long long)(((double)k + u) * (double)n_c / (double)K);
-    if (idx >= n_c) idx = n_c - 1;
+    const int n_t = n_live ? max(min(n_live[t], n_c), 1) : n_c;
+    // (a tree with fewer items uses the first K_t = ceil(n_t / bf) centroids only)
+    const int K_t = n_live ? min(max((n_t + bf - 1) / bf, 1), K) : K;
+    long long idx = (long long)(((double)min(k, K_t - 1) + u) * (double)n_t / (double)K_t);
+    if (idx >= n_t) idx = n_t - 1;
     const size_t src = ((size_t)t * x_tree_stride + (size_t)idx) * D;
     float* dst = cent + ((size_t)t * K + k) * D;
     for (int j = threadIdx.x; j < D; j += blockDim.x) dst[j] = load_elem<T>(x, src + j);
@@ -306,6 +310,17 @@ __global__ __launch_bounds__(64) void k_accept(const int32_t* sorted, const int3
     }
     __syncthreads();
     if (lane == 0) fill[(size_t)t * K + k] = f + take;
+}
+
+// items a tree does not hold count as placed from the start: no phase ever touches them; and
+// a tree with n_t items uses its first ceil(n_t / bf) centroids only: the others count as full
+__global__ void k_mark_absent(const int32_t* n_live, int n_c, int K, int bf, int32_t* placed,
+                              int32_t* fill) {
+    const int t = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    const int n_t = min(max(n_live[t], 0), n_c);
+    if (i < n_c) placed[(size_t)t * n_c + i] = i >= n_t ? 1 : 0;
+    if (i < K) fill[(size_t)t * K + i] = i >= max((n_t + bf - 1) / bf, 1) ? bf : 0;
 }
 
 __global__ void k_collect_unplaced(const int32_t* placed, int n_c, int32_t* list,
@@ -592,8 +607,8 @@ static void fill_i32(int32_t* p, size_t n, int32_t v, hipStream_t s) {
 
 template <typename T>
 static int build_impl(const HiraTree* t, const void* keys_in, const void* values_in, int n,
-                      int niter, int pack_rounds, uint64_t seed, const BuildWs& w,
-                      hipStream_t s) {
+                      const int32_t* n_live, int niter, int pack_rounds, uint64_t seed,
+                      const BuildWs& w, hipStream_t s) {
     const int L = t->num_levels, NT = t->num_trees, D = t->dim, bf = t->bf;
     constexpr int EPL = Elem<T>::kPerChunk;
     int lpr = 2;
@@ -611,38 +626,58 @@ static int build_impl(const HiraTree* t, const void* keys_in, const void* values
         const dim3 g_items(ceil_div(n_c, 256), NT);
         const dim3 g_cent(Kl, NT);
 
+        // Trees with fewer items than rows (n_live): the items a tree does not hold are marked
+        // placed before anything else, and every phase walks the list of the unplaced ones.
+        const bool ragged = n_live != nullptr && l == 1;
+        const int32_t* live = nullptr;
+        const int32_t* live_cnt = nullptr;
+        const size_t live_stride = ragged ? (size_t)n_c : 0;
+        if (ragged) {
+            hipLaunchKernelGGL(k_mark_absent, dim3(ceil_div(n_c > Kl ? n_c : Kl, 256), NT), dim3(256),
+                               0, s, n_live, n_c, Kl, bf, w.placed, w.fill);
+            fill_i32(w.list_count, (size_t)NT, 0, s);
+            hipLaunchKernelGGL(k_collect_unplaced, g_items, dim3(256), 0, s, w.placed, n_c, w.list,
+                               w.list_count);
+            live = w.list;
+            live_cnt = w.list_count;
+        }
         hipLaunchKernelGGL((k_init_centroids<T>), g_cent, dim3(64), 0, s, x, n_c, xs, Kl, D,
-                           seed + 7919ull * (uint64_t)l, w.cent_f32);
+                           seed + 7919ull * (uint64_t)l, w.cent_f32, ragged ? n_live : nullptr, bf);
         for (int it = 0; it < niter; ++it) {
             int rc;
             if (w.cent_tiles != nullptr) {
-                rc = launch_cent_prep(D, w.cent_f32, Kl, NT, nullptr, bf, w.cent_tiles, w.cent_n2, s);
+                rc = launch_cent_prep(D, w.cent_f32, Kl, NT, ragged ? w.fill : nullptr, bf,
+                                      w.cent_tiles, w.cent_n2, s);
                 if (rc == HIRA_OK)
-                    rc = launch_assign_mfma(D, x, n_c, xs, w.cent_tiles, w.cent_n2, Kl, NT, nullptr,
-                                            nullptr, 0, w.assign, w.dist, s);
+                    rc = launch_assign_mfma(D, x, n_c, xs, w.cent_tiles, w.cent_n2, Kl, NT, live,
+                                            live_cnt, live_stride, w.assign, w.dist, s);
             } else {
-                rc = launch_assign<T>(lpr, g_assign, s, x, n_c, xs, w.cent_f32, Kl, D, nullptr, bf,
-                                      nullptr, nullptr, 0, w.assign, w.dist);
+                rc = launch_assign<T>(lpr, g_assign, s, x, n_c, xs, w.cent_f32, Kl, D,
+                                      ragged ? w.fill : nullptr, bf, live, live_cnt, live_stride,
+                                      w.assign, w.dist);
             }
             if (rc != HIRA_OK) return rc;
             fill_i32(w.counts, (size_t)NT * Kl, 0, s);
-            hipLaunchKernelGGL(k_bucket_count, g_items, dim3(256), 0, s, w.assign, n_c, nullptr,
-                               nullptr, (size_t)0, Kl, w.counts);
+            hipLaunchKernelGGL(k_bucket_count, g_items, dim3(256), 0, s, w.assign, n_c, live,
+                               live_cnt, live_stride, Kl, w.counts);
             hipLaunchKernelGGL(k_scan, dim3(NT), dim3(256), 0, s, w.counts, Kl, w.offsets, w.cursor);
-            hipLaunchKernelGGL(k_bucket_fill, g_items, dim3(256), 0, s, w.assign, n_c, nullptr,
-                               nullptr, (size_t)0, Kl, w.cursor, w.members);
+            hipLaunchKernelGGL(k_bucket_fill, g_items, dim3(256), 0, s, w.assign, n_c, live,
+                               live_cnt, live_stride, Kl, w.cursor, w.members);
             hipLaunchKernelGGL(k_bucket_sort, g_cent, dim3(64), 0, s, w.members, w.offsets, w.dist,
                                n_c, Kl, w.sorted);
             hipLaunchKernelGGL((k_mean<T>), g_cent, dim3(64), 0, s, x, xs, n_c, Kl, D, w.offsets,
                                w.sorted, nullptr, bf, w.cent_f32, nullptr);
         }
         // capacity packing
-        fill_i32(w.fill, (size_t)NT * Kl, 0, s);
-        fill_i32(w.placed, (size_t)NT * n_c, 0, s);
+        if (!ragged) {  // (ragged: both were set up ahead of the Lloyd rounds)
+            fill_i32(w.fill, (size_t)NT * Kl, 0, s);
+            fill_i32(w.placed, (size_t)NT * n_c, 0, s);
+        }
         fill_i32(w.slots[l], (size_t)NT * Kl * bf, -1, s);
         for (int r = 0; r < pack_rounds; ++r) {
-            const int32_t* list = r == 0 ? nullptr : w.list;
-            const int32_t* lcnt = r == 0 ? nullptr : w.list_count;
+            // (ragged: the first round walks the list of the items the trees hold, made above)
+            const int32_t* list = r == 0 && !ragged ? nullptr : w.list;
+            const int32_t* lcnt = r == 0 && !ragged ? nullptr : w.list_count;
             if (r > 0) {
                 fill_i32(w.list_count, (size_t)NT, 0, s);
                 hipLaunchKernelGGL(k_collect_unplaced, g_items, dim3(256), 0, s, w.placed, n_c,
@@ -778,8 +813,20 @@ extern "C" size_t hira_build_workspace_bytes(const HiraTree* tree, int32_t n) {
 extern "C" int hira_build(const HiraTree* tree, const void* keys_in, const void* values_in,
                           int32_t n, int32_t niter, int32_t pack_rounds, uint64_t seed,
                           void* workspace, size_t workspace_bytes, void* stream) {
+    return hira_build_ragged(tree, keys_in, values_in, n, nullptr, niter, pack_rounds, seed,
+                             workspace, workspace_bytes, stream);
+}
+
+/* see include/hira_hip.h */
+extern "C" int hira_build_ragged(const HiraTree* tree, const void* keys_in, const void* values_in,
+                                 int32_t n, const int32_t* n_live, int32_t niter,
+                                 int32_t pack_rounds, uint64_t seed, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
     int rc = check_build_args(tree, n);
     if (rc != HIRA_OK) return rc;
+    HIRA_CHECK_ARG(n_live == nullptr || tree->num_levels == 2,
+                   "per-tree key counts are taken for trees of two levels only (got %d)",
+                   tree->num_levels);
     HIRA_CHECK_ARG(keys_in != nullptr && tree->keys != nullptr && tree->perm != nullptr,
                    "keys / perm missing");
     HIRA_CHECK_ARG(niter >= 0 && pack_rounds >= 1, "niter %d, pack_rounds %d", niter, pack_rounds);
@@ -792,8 +839,8 @@ extern "C" int hira_build(const HiraTree* tree, const void* keys_in, const void*
         return fail(HIRA_EWORKSPACE, "workspace %zu bytes, need %zu", workspace_bytes, b.total);
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     return tree->dtype == HIRA_F32
-               ? build_impl<float>(tree, keys_in, values_in, n, niter, pack_rounds, seed, b, s)
-               : build_impl<bf16_t>(tree, keys_in, values_in, n, niter, pack_rounds, seed, b, s);
+               ? build_impl<float>(tree, keys_in, values_in, n, n_live, niter, pack_rounds, seed, b, s)
+               : build_impl<bf16_t>(tree, keys_in, values_in, n, n_live, niter, pack_rounds, seed, b, s);
 }
 
 // ---- nearest centre as a call of its own -------------------------------------------------

@@ -468,10 +468,15 @@ class HIPIndexer(BaseIndexer):
 
     # ------------------------------------------------------------------ build / update
     @torch.no_grad()
-    def build(self, keys: torch.Tensor, values: Optional[torch.Tensor] = None):
+    def build(self, keys: torch.Tensor, values: Optional[torch.Tensor] = None, *,
+              key_counts: Optional[torch.Tensor] = None):
         """keys (1, H, L, D) (or (B, H, L, D): one tree per sequence and KV head), values
         (1, H, L, Dv) aligned with the keys or None.  Runs on the current stream and
-        returns self without waiting (indexer/cuda.py:56-108)."""
+        returns self without waiting (indexer/cuda.py:56-108).
+
+        ``key_counts`` (B*H,) int32 on the device (two levels only): tree t holds only the first
+        key_counts[t] of its L keys; every tree still gets the layout of L keys, with emptier
+        nodes where keys are missing (``num_keys`` then says L: the bound)."""
         if keys.ndim != 4:
             raise ValueError(f"keys must be (B,H,L,D), got {tuple(keys.shape)}")
         if values is not None and values.shape[:3] != keys.shape[:3]:
@@ -491,9 +496,19 @@ class HIPIndexer(BaseIndexer):
             _lib.check(-1)
         ws = torch.empty(need, dtype=torch.uint8, device=self.device)
         stream = torch.cuda.current_stream(self.device).cuda_stream
-        rc = lib.hira_build(C.byref(tree), kin.data_ptr(), None if vin is None else vin.data_ptr(),
-                            n, self.max_iterations, self.pack_rounds, self.seed, ws.data_ptr(),
-                            need, stream)
+        if key_counts is not None:
+            if key_counts.dtype != torch.int32 or tuple(key_counts.shape) != (b * h,) \
+                    or key_counts.device.type != self.device.type or not key_counts.is_contiguous():
+                raise ValueError(f"key_counts must be a contiguous int32 tensor of {b * h} counts on "
+                                 f"{self.device}")
+            rc = lib.hira_build_ragged(C.byref(tree), kin.data_ptr(),
+                                       None if vin is None else vin.data_ptr(), n,
+                                       key_counts.data_ptr(), self.max_iterations, self.pack_rounds,
+                                       self.seed, ws.data_ptr(), need, stream)
+        else:
+            rc = lib.hira_build(C.byref(tree), kin.data_ptr(),
+                                None if vin is None else vin.data_ptr(), n, self.max_iterations,
+                                self.pack_rounds, self.seed, ws.data_ptr(), need, stream)
         _lib.check(rc)
         self.num_keys = n
         if self.verbose:
@@ -817,8 +832,9 @@ class HIPIndexer(BaseIndexer):
         keys now and then.  The keys stay in the subtree's own slots [node*bf*bf,
         (node+1)*bf*bf); its level-1 nodes get new centres, radii and counts; the level-2
         node keeps its centre, gets the radius its new children need, and its ancestors are
-        inflated where that radius grew.  One small build per tree (the trees hold different
-        numbers of keys there)."""
+        inflated where that radius grew.  One build over all trees (hira_build_ragged: the trees
+        hold different numbers of keys there) and a few batched tensor operations; nothing is
+        read back to the host."""
         if self.keys_buf is None:
             raise ValueError("Indexer is not built: call build() first.")
         if self.num_levels < 3:
@@ -830,56 +846,71 @@ class HIPIndexer(BaseIndexer):
         self.sync_sizes()
         if not 0 <= node < self.size[2]:
             raise ValueError(f"level-2 node {node} not in 0..{self.size[2] - 1}")
-        s0, n0 = node * bf * bf, node * bf
-        s1, n1 = min(s0 + bf * bf, self.cap[0]), min(n0 + bf, self.cap[1])
-        for t in range(self.num_trees):
-            perm_sub = self.perm[t, s0:s1].clone()
-            live = (perm_sub >= 0).nonzero().squeeze(1)
-            n = int(live.numel())
-            if n == 0:
-                continue
-            rows = self.keys_buf[t:t + 1, s0:s1]
-            rows = (from_tiled(rows) if self.keys_tiled else rows)[0, live]
-            vals = None if self.values_buf is None else self.values_buf[t, s0:s1][live]
-            sub = HIPIndexer(2, self.max_iterations, bf, seed=self.seed + node,
-                             device=str(self.device), pack_rounds=self.pack_rounds,
-                             layout=self.layout_name)
-            sub.build(rows[None, None], None if vals is None else vals[None, None])
-            k, m = sub.size[1], sub.size[0]  # level-1 nodes and key slots the subtree uses now
-            # keys, values, positions: the rebuilt slots first, the rest of the subtree empty
-            self.keys_buf[t, s0:s1] = 0
-            self.keys_buf[t, s0:s0 + m] = sub.keys_buf[0, :m]
-            if vals is not None:
-                self.values_buf[t, s0:s1] = 0
-                self.values_buf[t, s0:s0 + m] = sub.values_buf[0, :m]
-            sub_perm = sub.perm[0, :m].long()
-            self.perm[t, s0:s1] = -1
-            self.perm[t, s0:s0 + m] = torch.where(
-                sub_perm >= 0, perm_sub[live][sub_perm.clamp(min=0)],
-                torch.full_like(sub_perm, -1, dtype=torch.int32))
-            # level 1 (a tile of 16 centres is contiguous, so tiled rows copy as they are)
-            kc = -(-k // 16) * 16 if self.tiled else k
-            self.centers[1][t, n0:n1] = 0
-            self.centers[1][t, n0:n0 + kc] = sub.centers[1][0, :kc]
-            self.radii[1][t, n0:n1] = float("-inf")
-            self.radii[1][t, n0:n0 + k] = sub.radii[1][0, :k]
-            self.counts[1][t, n0:n1] = 0
-            self.counts[1][t, n0:n0 + k] = sub.counts[1][0, :k]
-            # level 2: same centre, the radius its children need; ancestors cover it
-            c1 = sub.centers_rowmajor(1)[0].float()
-            child, c_child, r_child = node, None, None
-            for l in range(2, self.num_levels):
-                tile0 = child // 16 * 16  # (de-tiling needs whole tiles)
-                cl = self.centers[l][t:t + 1, tile0:tile0 + 16]
-                cl = (from_tiled(cl) if self.tiled else cl)[0, child - tile0].float()
-                if l == 2:
-                    r = ((c1 - cl).norm(dim=1) + sub.radii[1][0, :k]).max() * (1 + 1e-6)
-                    self.counts[2][t, child] = k
-                else:
-                    r = torch.maximum(self.radii[l][t, child],
-                                      ((c_child - cl).norm() + r_child) * (1 + 1e-6))
-                self.radii[l][t, child] = r
-                c_child, r_child, child = cl, r, child // bf
+        T, nsub = self.num_trees, bf * bf
+        s0, n0 = node * nsub, node * bf
+        if s0 + nsub > self.cap[0] or n0 + bf > self.cap[1]:
+            raise ValueError("the subtree's slots lie beyond the capacity of the index")
+        # the subtree's keys of every tree, those it holds first (in slot order); how many each
+        # tree holds stays on the device: nothing here waits for the GPU
+        perm_sub = self.perm[:, s0:s0 + nsub]
+        live = perm_sub >= 0
+        order = torch.sort((~live).to(torch.uint8), dim=1, stable=True).indices  # (T, nsub)
+        counts = live.sum(dim=1, dtype=torch.int32).contiguous()
+        rows = self.keys_buf[:, s0:s0 + nsub]
+        rows = from_tiled(rows) if self.keys_tiled else rows
+        rows = torch.gather(rows, 1, order[:, :, None].expand(-1, -1, self.dim))
+        vals = None
+        if self.values_buf is not None:
+            vals = torch.gather(self.values_buf[:, s0:s0 + nsub], 1,
+                                order[:, :, None].expand(-1, -1, self.vdim))
+        pos = torch.gather(perm_sub, 1, order)  # insertion positions, the missing ones (-1) last
+        # one build over all trees: two levels, bf nodes of bf slots, fewer keys in some trees
+        sub = HIPIndexer(2, self.max_iterations, bf, seed=self.seed + node,
+                         device=str(self.device), pack_rounds=self.pack_rounds,
+                         layout=self.layout_name)
+        sub.build(rows.reshape(self.batch, self.num_heads, nsub, self.dim),
+                  None if vals is None else vals.reshape(self.batch, self.num_heads, nsub, self.vdim),
+                  key_counts=counts)
+        if sub.size[0] != nsub or sub.size[1] != bf or sub.tiled != self.tiled or sub.q8 != self.q8:
+            raise RuntimeError("sub-tree layout differs from the index's")
+        # a node's children fill its slots from the first one on (appends open the next child
+        # behind them): the new level-1 nodes that hold keys go first, whole nodes moving with
+        # their bf key slots (a node's rows are whole tiles, so tiled rows move as they are)
+        cnt1 = sub.counts[1][:, :bf]
+        nodes = torch.sort((cnt1 == 0).to(torch.uint8), dim=1, stable=True).indices  # (T, bf)
+
+        def by_node(x, width):  # (T, bf * bf, width) in slot order -> nodes in the new order
+            idx = nodes[:, :, None].expand(-1, -1, bf * width)
+            return torch.gather(x.reshape(T, bf, bf * width), 1, idx).reshape(T, nsub, width)
+
+        self.keys_buf[:, s0:s0 + nsub] = by_node(sub.keys_buf[:, :nsub], self.dim)
+        if vals is not None:
+            self.values_buf[:, s0:s0 + nsub] = by_node(sub.values_buf[:, :nsub], self.vdim)
+        sp = by_node(sub.perm[:, :nsub, None], 1)[:, :, 0].long()
+        self.perm[:, s0:s0 + nsub] = torch.where(
+            sp >= 0, torch.gather(pos, 1, sp.clamp(min=0)), torch.full_like(pos, -1))
+        c1 = torch.gather(sub.centers_rowmajor(1)[:, :bf], 1,
+                          nodes[:, :, None].expand(-1, -1, self.dim))     # (T, bf, D), storage type
+        r1 = torch.gather(sub.radii[1][:, :bf], 1, nodes)                  # (T, bf), -inf: empty
+        cnt1 = torch.gather(cnt1, 1, nodes)
+        self.centers[1][:, n0:n0 + bf] = to_tiled(c1) if self.tiled else c1
+        self.radii[1][:, n0:n0 + bf] = r1
+        self.counts[1][:, n0:n0 + bf] = cnt1
+        # level 2: same centre, the radius its new children need; ancestors cover it where it grew
+        c1 = c1.float()
+        child, c_child, r_child = node, None, None
+        for l in range(2, self.num_levels):
+            tile0 = child // 16 * 16  # (de-tiling needs whole tiles)
+            cl = self.centers[l][:, tile0:tile0 + 16]
+            cl = (from_tiled(cl) if self.tiled else cl)[:, child - tile0].float()  # (T, D)
+            if l == 2:
+                r = ((c1 - cl[:, None]).norm(dim=2) + r1).amax(dim=1) * (1 + 1e-6)
+                self.counts[2][:, child] = (cnt1 > 0).sum(dim=1, dtype=torch.int32)
+            else:
+                r = torch.maximum(self.radii[l][:, child],
+                                  ((c_child - cl).norm(dim=1) + r_child) * (1 + 1e-6))
+            self.radii[l][:, child] = r
+            c_child, r_child, child = cl, r, child // bf
         self._tree_struct = None
-        self.quantize(s0, s1 - s0)
+        self.quantize(s0, nsub)
         return self

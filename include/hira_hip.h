@@ -224,6 +224,20 @@ int hira_build(const HiraTree* tree, const void* keys_in, const void* values_in,
                size_t workspace_bytes, void* stream);
 
 /*
+ * hira_build for trees that hold different numbers of keys: tree t's keys are the first
+ * n_live[t] (device array of T counts, each <= n) rows of its (n, D) block of keys_in; the
+ * other rows are never read.  Every tree gets the layout of n keys (tree->size[] as for
+ * hira_build); a tree with fewer keys has emptier or empty nodes (count 0, radius -inf) and
+ * empty key slots (perm < 0).  Two levels only.  It is what re-clusters one subtree of every
+ * tree of an index in a single build (the subtrees hold different numbers of keys); the
+ * reference has no counterpart (its update never re-clusters, indexer/cuda.py:544-701).
+ * n_live == NULL: hira_build.
+ */
+int hira_build_ragged(const HiraTree* tree, const void* keys_in, const void* values_in, int32_t n,
+                      const int32_t* n_live, int32_t niter, int32_t pack_rounds, uint64_t seed,
+                      void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Nearest centre of every row, the distance step of the build (every Lloyd round and every
  * packing round of hira_build runs these kernels) as a call of its own:
  *   idx[t][i] = argmin_k ||x[t][i] - centers[t][k]||^2 over the centres with valid[t][k] != 0,

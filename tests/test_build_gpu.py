@@ -195,3 +195,54 @@ def test_build_rejects_bad_shapes(gpu_device):
         HIPIndexer(9, 1, 8)
     with pytest.raises(ValueError):
         HIPIndexer(2, 1, 65)
+
+
+@pytest.mark.parametrize("dtype,d,bf", [(torch.bfloat16, 128, 32), (torch.float32, 32, 8),
+                                        (torch.bfloat16, 64, 16)])
+def test_build_of_trees_with_different_numbers_of_keys(dtype, d, bf, gpu_device):
+    """hira_build_ragged (HIPIndexer.build(key_counts=...)): every tree gets the layout of n keys
+    but holds only its first n_t; each of those sits in exactly one slot, the others in none;
+    a tree uses ceil(n_t / bf) nodes, counts are exact, radii cover, an empty tree is all empty;
+    the search over every tree is the brute-force search over its own keys."""
+    from hira_amd.indexer.hip import HIPIndexer
+    from hira_amd.searcher.hip import HIPSearcher
+
+    n = bf * bf
+    counts = [n, n // 3 + 5, 1, 0, bf, bf + 1]
+    t = len(counts)
+    rnd = bf16_round if dtype == torch.bfloat16 else (lambda x: x)
+    keys = rnd(clustered_keys(t, n, d, seed=11, clusters=10))
+    vals = rnd(np.random.default_rng(2).normal(size=(t, n, d)).astype(np.float32))
+    kc = torch.tensor(counts, dtype=torch.int32, device="cuda")
+    idx = HIPIndexer(2, 2, bf).build(torch.from_numpy(keys)[None].to(dtype),
+                                     torch.from_numpy(vals)[None].to(dtype), key_counts=kc)
+    assert idx.size == [n, bf]
+    got = _download(idx)
+    for h, n_t in enumerate(counts):
+        perm = got["perm"][h]
+        ok = perm >= 0
+        assert np.array_equal(np.sort(perm[ok]), np.arange(n_t))
+        assert np.array_equal(got["keys"][h][ok], keys[h][perm[ok]])
+        assert np.array_equal(got["values"][h][ok], vals[h][perm[ok]])
+        blk = ok.reshape(bf, bf)
+        cnt = got["counts"][1][h]
+        assert np.array_equal(cnt, blk.sum(1))
+        assert np.all(blk[:, :-1] >= blk[:, 1:])            # a node's keys fill it from slot 0
+        used = -(-n_t // bf)
+        assert (cnt[used:] == 0).all() and (cnt[:used] > 0).all()
+        rad, cen = got["radii"][1][h], got["centers"][1][h]
+        assert np.all(rad[cnt == 0] == -np.inf)
+        need = ho.radii_from_layout(got["keys"][h], np.zeros(n, np.float32), ok, cen, bf)
+        assert np.all(rad[cnt > 0] >= need[cnt > 0] * (1 - 1e-6) - 1e-6)
+    q = rnd(random_query(t, d, seed=4))
+    s = ho.scores(keys, q, np.arange(t))
+    s = np.where(np.arange(n)[None] < np.array(counts)[:, None], s, -np.inf).astype(np.float32)
+    # thresholds that keep about a tenth of a tree's keys (its only key; nothing of an empty tree)
+    th = np.array([np.sort(s[h])[::-1][min(counts[h] // 10, counts[h] - 1)] if counts[h] else 0.0
+                   for h in range(t)], np.float32) - 1e-3
+    out = HIPSearcher(index_space="position").search(torch.from_numpy(q), torch.from_numpy(th), idx)
+    out = out.cpu().numpy()
+    assert out.shape[1] == n
+    assert_same_selection(out != 0, s, th)
+    with pytest.raises(ValueError):
+        HIPIndexer(3, 1, bf).build(torch.from_numpy(keys)[None].to(dtype), key_counts=kc)
