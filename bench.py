@@ -233,15 +233,18 @@ def streaming(a, w, index, plan, q_d, taus, out, dev):
     """Decode with a growing index: per step one key/value per tree is appended (one update
     launch), then one search + attention over the index as it stands; every
     a.rebuild_every steps one level-2 subtree is re-clustered (round-robin).  Times are GPU
-    times between events; the update also has a host part (it reads the level sizes back)."""
+    times between events.  The appends do not read the level sizes back (update(sync=False)
+    after reserve(): the host carries bounds); the sizes are re-read before every rebuild."""
     import torch
 
     from hira_amd import synth
 
     S = a.stream
     sk, sv = synth.make_stream(w, S)
-    sk, sv = sk.to(dev), sv.to(dev)
-    index._grow(index._needed_caps(S))  # room for all appends: no re-allocation while timed
+    # one contiguous (B, H, 1, D) tensor per token, as a model's decode step hands them over
+    sk = sk.to(dev).permute(2, 0, 1, 3).contiguous()[:, :, :, None, :]
+    sv = sv.to(dev).permute(2, 0, 1, 3).contiguous()[:, :, :, None, :]
+    index.reserve(S)  # room for all appends: no re-allocation while timed
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(S)]
     rb = []
     nq = q_d.shape[0]
@@ -250,7 +253,7 @@ def streaming(a, w, index, plan, q_d, taus, out, dev):
     for t in range(S):
         ev[t][0].record()
         h0 = time.perf_counter()
-        index.update(sk[:, :, t:t + 1], sv[:, :, t:t + 1])
+        index.update(sk[t], sv[t], sync=False)
         t_host_upd += time.perf_counter() - h0
         ev[t][1].record()
         plan.run(q_d[t % nq], taus[t % nq], out)

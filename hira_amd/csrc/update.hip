@@ -21,6 +21,9 @@
 // state (T, HIRA_MAX_LEVELS + 2) int32: [l] = slots of level l in use (l >= 1; the host keeps
 // the maximum over the trees as size[l]), [HIRA_MAX_LEVELS] = keys inserted so far,
 // [HIRA_MAX_LEVELS + 1] = error flag (1: a level ran out of capacity; the key was dropped).
+// [0] (trees of two or more levels): every level-1 node with a lower index is full -- a lower
+// bound that the search for a node with room starts from and raises as it learns more (0 is
+// always valid; whoever lowers a count of a level-1 node from outside must lower it too).
 #include "rows.h"
 
 namespace hira {
@@ -49,31 +52,41 @@ struct UpdateParams {
 // a bound must survive the fp32 rounding of the sums that produced it
 __device__ __forceinline__ float pad_up(float r) { return r > 0.0f ? r * (1.0f + 4.0f * 1.1920929e-7f) + 1e-30f : r; }
 
-// Nearest node of level l (among the first `used` ones) with a free child slot; -1 if none.
-// Wave w scans nodes w, w+4, ...; a full node costs one count read.  Ties go to the lowest id.
+// Nearest node of level l (among nodes first .. used - 1; the ones before `first` are known to
+// be full) with a free child slot; -1 if none.  Wave w scans nodes w, w+4, ...; a full node
+// costs one count read.  Ties go to the lowest id.  *not_full (if given) receives the lowest
+// index from `first` on whose node is not full (`used` if there is none).
+constexpr int kCountsInFlight = 16;  // reads of child counts a lane has in flight
 template <typename T>
-__device__ int nearest_with_room(const UpdateParams& p, int tree, int l, int used, const float* x,
-                                 float* red_f, int* red_i) {
+__device__ int nearest_with_room(const UpdateParams& p, int tree, int l, int first, int used,
+                                 const float* x, float* red_f, int* red_i, int* not_full,
+                                 int* count_of = nullptr) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int D = p.dim;
     const size_t base = (size_t)tree * p.cap[l];
     const int32_t* cnt = p.counts[l] + base;
     float best = INFINITY;
-    int arg = -1;
-    for (int nb = wave * 64; nb < used; nb += 4 * 4 * 64) {
-        // four reads of child counts in flight (a wave's nodes still come in increasing order)
-        int c4[4];
+    int arg = -1, argc = 0;  // the best node so far and its child count
+    int low = used;  // lowest index of a node that is not full, among those I have seen
+    for (int nb = (first & ~63) + wave * 64; nb < used; nb += kCountsInFlight * 4 * 64) {
+        // the reads of the child counts in flight together (a wave's nodes still come in
+        // increasing order): one trip to memory for 4096 nodes
+        int c4[kCountsInFlight];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < kCountsInFlight; ++u) {
             const int n = nb + u * 4 * 64 + lane;
-            c4[u] = n < used ? cnt[n] : 0;
+            c4[u] = n < used ? cnt[n] : p.bf;
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < kCountsInFlight; ++u) {
+            if (nb + u * 4 * 64 >= used) break;  // uniform
+            if (c4[u] < p.bf) low = min(low, nb + u * 4 * 64 + lane);
             // a node in use with a free slot; count 0 marks a pad slot, which is not a node yet
             unsigned long long bal = __ballot(c4[u] > 0 && c4[u] < p.bf);
             while (bal != 0ull) {  // uniform in the wave
-                const int node = nb + u * 4 * 64 + __ffsll((long long)bal) - 1;
+                const int src = __ffsll((long long)bal) - 1;
+                const int node = nb + u * 4 * 64 + src;
+                const int node_c = __shfl(c4[u], src, 64);
                 bal &= bal - 1ull;
                 float ss = 0.0f;
                 for (int j = lane; j < D; j += 64) {
@@ -85,18 +98,27 @@ __device__ int nearest_with_room(const UpdateParams& p, int tree, int l, int use
                 if (ss < best) {
                     best = ss;
                     arg = node;
+                    argc = node_c;
                 }
             }
         }
     }
     __syncthreads();
+    if (not_full != nullptr) {  // uniform
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) low = min(low, __shfl_xor(low, off, 64));
+        if (lane == 0) red_i[wave] = low;
+        __syncthreads();
+        if (threadIdx.x == 0) *not_full = max(min(min(red_i[0], red_i[1]), min(red_i[2], red_i[3])), first);
+        __syncthreads();
+    }
     if (lane == 0) {
         red_f[wave] = best;
         red_i[wave] = arg;
     }
     __syncthreads();
     float b = red_f[0];
-    int a = red_i[0];
+    int a = red_i[0], aw_of = 0;
 #pragma unroll
     for (int w = 1; w < 4; ++w) {
         const float bw = red_f[w];
@@ -104,9 +126,16 @@ __device__ int nearest_with_room(const UpdateParams& p, int tree, int l, int use
         if (aw >= 0 && (a < 0 || bw < b || (bw == b && aw < a))) {
             b = bw;
             a = aw;
+            aw_of = w;
         }
     }
     __syncthreads();
+    if (count_of != nullptr) {  // uniform: the child count of the chosen node, as the scan read it
+        if (lane == 0) red_i[wave] = argc;
+        __syncthreads();
+        *count_of = red_i[aw_of];
+        __syncthreads();
+    }
     return a;
 }
 
@@ -132,10 +161,12 @@ __global__ __launch_bounds__(kUpdThreads) void k_update(const UpdateParams p) {
 
         long long slot = -1;  // key slot
         int node1 = -1;       // level-1 node that took the key (L >= 2)
+        int count1 = 0;       // keys it held before
         if (L == 1) {
             slot = position < p.cap[0] ? position : -1;
         } else {
-            node1 = nearest_with_room<T>(p, tree, 1, st[1], x, red_f, red_i);
+            node1 = nearest_with_room<T>(p, tree, 1, min(max(st[0], 0), st[1]), st[1], x, red_f, red_i, &st[0],
+                                             &count1);
             if (node1 < 0) {
                 // ---- open a new level-1 node; attach it upwards -----------------------
                 // child_c = centre of the node being attached (the key itself at level 1)
@@ -150,7 +181,7 @@ __global__ __launch_bounds__(kUpdThreads) void k_update(const UpdateParams p) {
                         parent = -1;
                         break;
                     }
-                    parent = nearest_with_room<T>(p, tree, lvl + 1, st[lvl + 1], cbuf, red_f, red_i);
+                    parent = nearest_with_room<T>(p, tree, lvl + 1, 0, st[lvl + 1], cbuf, red_f, red_i, nullptr);
                     if (parent >= 0) break;
                     ++lvl;
                 }
@@ -192,10 +223,12 @@ __global__ __launch_bounds__(kUpdThreads) void k_update(const UpdateParams p) {
                     p.counts[opened_top + 1][(size_t)tree * p.cap[opened_top + 1] + parent] += 1;
                 __syncthreads();
                 node1 = (int)(id / bf);  // the new level-1 node (id is now its first key slot)
+                count1 = 0;
             }
             // the key takes the next slot of node1
+            // (a node found by the scan: the count the scan read; a node just opened: none)
             const size_t b1 = (size_t)tree * p.cap[1];
-            const int c = p.counts[1][b1 + node1];
+            const int c = count1;
             slot = (long long)node1 * bf + c;
             __syncthreads();
             if (t == 0) p.counts[1][b1 + node1] = c + 1;
@@ -228,7 +261,7 @@ __global__ __launch_bounds__(kUpdThreads) void k_update(const UpdateParams p) {
                     float* e = p.keps + (size_t)tree * p.cap[1] + node1;
                     const float w = fmaxf(fmaxf(red_f[0], red_f[1]), fmaxf(red_f[2], red_f[3]));
                     // a node that just opened holds no other key: its bound starts here
-                    const bool fresh = p.counts[1][(size_t)tree * p.cap[1] + node1] == 1;
+                    const bool fresh = count1 == 0;
                     *e = fresh ? w : fmaxf(*e, w);
                 }
                 __syncthreads();
@@ -254,6 +287,7 @@ __global__ __launch_bounds__(kUpdThreads) void k_update(const UpdateParams p) {
                 for (int i = 2; i < l; ++i) child /= (size_t)bf;
                 const size_t node = l == 1 ? (size_t)node1 : child / (size_t)bf;
                 const size_t bl = (size_t)tree * p.cap[l], bc = (size_t)tree * p.cap[l - 1];
+                const float rad_now = p.radii[l][bl + node];  // (asked for with the centres)
                 float ss = 0.0f;
                 for (int j = lane; j < D; j += 64) {
                     const float a =
@@ -266,7 +300,7 @@ __global__ __launch_bounds__(kUpdThreads) void k_update(const UpdateParams p) {
                 for (int off = 1; off < 64; off <<= 1) ss += __shfl_xor(ss, off, 64);
                 if (lane == 0) {
                     s_dist[l] = sqrtf(ss);
-                    s_rad[l] = p.radii[l][bl + node];
+                    s_rad[l] = rad_now;
                 }
             }
             __syncthreads();

@@ -442,6 +442,8 @@ class HIPIndexer(BaseIndexer):
             put(self.counts[l], f"counts.{l}")
         if "update_state" in tensors:
             self._state = tensors["update_state"].to(self.device)
+            if self.num_levels >= 2:
+                self._state[:, 0] = 0
         if self.q8:
             put(self.keys8, "keys8")
             self.kscale.copy_(tensors["kscale"].to(self.device))
@@ -727,6 +729,8 @@ class HIPIndexer(BaseIndexer):
         st = torch.zeros((self.num_trees, _lib.HIRA_MAX_LEVELS + 2), dtype=torch.int32)
         for l in range(self.num_levels):
             st[:, l] = self.size[l]
+        if self.num_levels >= 2:
+            st[:, 0] = 0  # "every level-1 node below this index is full": nothing known yet
         st[:, _lib.HIRA_MAX_LEVELS] = self.num_keys
         self._state = st.to(self.device)
 
@@ -911,6 +915,8 @@ class HIPIndexer(BaseIndexer):
                                   ((c_child - cl).norm(dim=1) + r_child) * (1 + 1e-6))
             self.radii[l][:, child] = r
             c_child, r_child, child = cl, r, child // bf
+        if self._state is not None:
+            self._state[:, 0] = 0  # the rebuilt nodes may have room again
         self._tree_struct = None
         self.quantize(s0, nsub)
         return self
