@@ -606,6 +606,22 @@ def main():
         t1e.record(stream)
         stream.synchronize()
     thr_us = t0e.elapsed_time(t1e) * 1e3 / K
+    # and the whole step a deployment without given thresholds runs: thresholds from the sample,
+    # then search + attention with them (two launches per step, K steps in one graph)
+    g4 = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(g4, stream=stream):
+            for i in range(W, total):
+                plan.run_sampled(q_d[i], samples, "sample_mean_topk", 10, scratch,
+                                 stream=stream.cuda_stream)
+        g4.replay()
+        stream.synchronize()
+        t0e.record(stream)
+        g4.replay()
+        t1e.record(stream)
+        stream.synchronize()
+    step_thr_us = t0e.elapsed_time(t1e) * 1e3 / K
+    del g4
     dense_best = min(dense_us.values())
 
     e = 2 if w.dtype == torch.bfloat16 else 4
@@ -640,6 +656,7 @@ def main():
         "streaming_add_GBps": round(stream_gbs, 1),
         "rotating_indexes": rot,
         "sample_threshold_us": round(thr_us, 2),
+        "step_with_sample_threshold_us": round(step_thr_us, 2),
         "dense_attention_us": {k: round(v, 2) for k, v in dense_us.items()},
         "dense_attention_bytes": dense_bytes,
         "frac_of_dense_time": round(kernel_us / dense_best, 4),

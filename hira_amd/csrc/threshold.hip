@@ -1,7 +1,11 @@
 // hira_threshold: per-head thresholds from a sample of a tree's keys, one launch.
 //   tau[h] = max_s q_h . x_s                      (HIRA_TAU_SAMPLE_MAX)
 //   tau[h] = mean of the k largest q_h . x_s      (HIRA_TAU_SAMPLE_MEAN_TOPK)
-// One workgroup of sixteen waves per query head.  Scores: 16 lanes share a sample row (16 bytes
+// One workgroup of sixteen waves per query head; with whole groups of heads per tree the
+// workgroups of a tree are a multiple of eight apart in the launch, so that they run behind the
+// same L2 (workgroups go to the eight L2s in turn) and the tree's sample is fetched from memory
+// once.  Up to 1024 samples and k <= 16: every wave sorts its 64 scores in registers, the
+// sixteen best of every wave meet in LDS, and one wave picks the k best of those 256 one by one.  Scores: 16 lanes share a sample row (16 bytes
 // each per step), eight rows per lane group in flight.  Then either a maximum, or a bitonic sort
 // by the first four waves with the scores in registers (entry e*256 + thread of the padded
 // array lives in register e of that thread: partners 256 or more apart are a register swap,
@@ -32,6 +36,48 @@ __device__ __forceinline__ float tau_block_reduce(float v, bool is_max, float* s
 }
 
 constexpr int kTauSorters = 256;  // threads that hold the scores during the sort
+
+// The value that lane ^ J holds: moves inside a row of 16 lanes (J < 16) are data-path moves,
+// only J = 16 and 32 go through the LDS crossbar.  rot4_first: which rotation by 4 brings lane ^ 4.
+template <int J>
+__device__ __forceinline__ float tau_partner(float v, bool rot4_first) {
+    if constexpr (J >= 16) {
+        return __shfl_xor(v, J, 64);
+    } else if constexpr (J == 8) {
+        return dpp_move<0x128>(v);  // row rotate by 8
+    } else if constexpr (J == 4) {
+        const float a = dpp_move<0x124>(v), b = dpp_move<0x12C>(v);  // by 4, by 12
+        return rot4_first ? a : b;
+    } else if constexpr (J == 2) {
+        return dpp_move<0x4E>(v);  // quad [2,3,0,1]
+    } else {
+        return dpp_move<0xB1>(v);  // quad [1,0,3,2]
+    }
+}
+
+// One merge stage (stretches of LEN, partners J = LEN/2 .. 1) of a wave's 64 values, one a lane,
+// largest first in the end (the last stage sorts the whole wave one way).
+template <int LEN, int J>
+__device__ __forceinline__ void tau_wave_stage(float& x, int ln, bool rot4_first) {
+    const float o = tau_partner<J>(x, rot4_first);
+    const bool down = (ln & LEN) == 0 || LEN == 64, lower = (ln & J) == 0;
+    x = (down == lower) ? fmaxf(x, o) : fminf(x, o);
+    if constexpr (J > 1) tau_wave_stage<LEN, J / 2>(x, ln, rot4_first);
+}
+
+// maximum over the wave: inside the rows of 16 by data-path moves, the four rows by reading
+// one lane of each
+__device__ __forceinline__ float tau_wave_max(float v, bool rot4_first) {
+    v = fmaxf(v, tau_partner<1>(v, rot4_first));
+    v = fmaxf(v, tau_partner<2>(v, rot4_first));
+    v = fmaxf(v, tau_partner<4>(v, rot4_first));
+    v = fmaxf(v, tau_partner<8>(v, rot4_first));
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    const float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    const float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
 
 // One step of the bitonic sort (largest first) of 256 * EE entries, entry e*256 + tid in v[e]
 // of thread tid < 256: entry i meets entry i ^ J; in a stretch that ends up descending
@@ -125,8 +171,9 @@ __global__ __launch_bounds__(kTauThreads) void k_threshold(
     const int pos = blockIdx.x;
     int head, tree;
     if (group_size > 0) {
-        head = pos;
-        tree = pos / group_size;
+        // trees in the fast index: workgroup i takes head i / T of tree i % T
+        tree = pos % num_trees;
+        head = tree * group_size + pos / num_trees;
     } else {
         tree = 0;
         while (tree + 1 < num_trees && tree_q_off[tree + 1] <= pos) ++tree;  // uniform
@@ -184,6 +231,43 @@ __global__ __launch_bounds__(kTauThreads) void k_threshold(
         for (int e = 1; e < EE; ++e) m = fmaxf(m, v[e]);
         m = tau_block_reduce(m, true, s_red);
         if (tid == 0) tau[head] = m;
+        return;
+    }
+
+    if (E == 1 && k <= 16) {
+        // ---- few of up to 1024: every wave sorts its 64 scores, largest first ------------------
+        const int ln = tid & 63, wv = tid >> 6;
+        const bool rot4 = __builtin_amdgcn_update_dpp(0, ln, 0x124, 0xF, 0xF, true) == (ln ^ 4);
+        float x = tid < S ? s_sc[0][tid] : -INFINITY;
+        tau_wave_stage<2, 1>(x, ln, rot4);
+        tau_wave_stage<4, 2>(x, ln, rot4);
+        tau_wave_stage<8, 4>(x, ln, rot4);
+        tau_wave_stage<16, 8>(x, ln, rot4);
+        tau_wave_stage<32, 16>(x, ln, rot4);
+        tau_wave_stage<64, 32>(x, ln, rot4);
+        __syncthreads();  // everybody has read its score
+        if (ln < 16) s_sc[1][wv * 16 + ln] = x;
+        __syncthreads();
+        if (wv != 0) return;
+        // the k best of the 256 that are left, one at a time: the wave's maximum, taken out of
+        // the one place (lowest lane, lowest register) that holds it
+        float c[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) c[e] = s_sc[1][e * 64 + ln];
+        float sum = 0.0f;
+        for (int r = 0; r < k; ++r) {  // uniform
+            const float mine = fmaxf(fmaxf(c[0], c[1]), fmaxf(c[2], c[3]));
+            const float best = tau_wave_max(mine, rot4);
+            sum += best;
+            const unsigned long long has = __ballot(mine == best);
+            if (ln == __ffsll((long long)has) - 1) {
+                if (c[0] == best) c[0] = -INFINITY;
+                else if (c[1] == best) c[1] = -INFINITY;
+                else if (c[2] == best) c[2] = -INFINITY;
+                else c[3] = -INFINITY;
+            }
+        }
+        if (ln == 0) tau[head] = sum / (float)k;
         return;
     }
 

@@ -18,6 +18,8 @@ CASES = [
     (3, 37, 32, 3, torch.float32, 1),         # k = 1: the maximum; ragged sample count
     (2, 1, 256, 4, torch.bfloat16, 1),        # one sample
     (4, 513, 16, 16, torch.bfloat16, 100),    # just past a power of two
+    (2, 1024, 64, 4, torch.float32, 16),      # the most that the few-of-many path takes
+    (2, 65, 32, 8, torch.bfloat16, 7),        # a second wave holding a single score
 ]
 
 
