@@ -536,6 +536,46 @@ def main():
                "same_outputs": same}
         del copies, plans, g3
 
+    # ---- the same steps over an index that also keeps an 8-bit shadow of its keys (layout q8):
+    # the scan reads the shadow, the exact test only the rows the shadow cannot rule out
+    q8_leg = None
+    if not index.q8 and not a.profile and w.dtype == torch.bfloat16 and w.d % 64 == 0 \
+            and index.num_levels >= 2 and a.kernel != 1:
+        try:
+            qindex = HIPIndexer(w.num_levels, niter, w.bf, device="cuda:0", layout="q8").build(keys_d, values_d)
+            qstats = torch.zeros_like(stats)
+            qsplan = searcher.plan_attention(qindex, h_all, scaling=torch.full((h_all,), scale), stats=qstats)
+            qouts = torch.empty_like(outs)
+            for i in range(W, total):
+                qsplan.run(q_d[i], taus[i], qouts[i])
+            torch.cuda.synchronize()
+            qb, qb16, qcounts = algorithmic_bytes(qstats.cpu().numpy(), w, qindex.num_levels, K, shadow=True)
+            qplan = searcher.plan_attention(qindex, h_all, scaling=torch.full((h_all,), scale))
+            gq = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(stream):
+                with torch.cuda.graph(gq, stream=stream):
+                    for i in range(W, total):
+                        qplan.run(q_d[i], taus[i], qouts[i])
+                gq.replay()
+                stream.synchronize()
+                q0, q1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                q0.record(stream)
+                gq.replay()
+                q1.record(stream)
+                stream.synchronize()
+            q_us = q0.elapsed_time(q1) * 1e3 / K
+            q8_leg = {"us_per_step": round(q_us, 3), "algorithmic_bytes_per_step": round(qb),
+                      "achieved_GBps": round(qb / (q_us * 1e-6) / 1e9, 1),
+                      "frac_of_hbm_peak": round(qb / (q_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                      "exact_rows_per_step": round(qcounts["exact_rows_per_step"], 1),
+                      "same_selection_counts": bool(
+                          qcounts["selected_pairs_per_step"] == counts["selected_pairs_per_step"]
+                          and qcounts["candidates_per_step"] == counts["candidates_per_step"]),
+                      "max_abs_diff_of_outputs": float((qouts[W:] - outs[W:]).abs().max())}
+            del qindex, qsplan, qplan, gq
+        except Exception as ex:  # noqa: BLE001
+            log(f"[bench] q8 leg failed: {ex!r}")
+
     # ---- dense comparators ------------------------------------------------------------
     dense_us = {}
     if a.profile:
@@ -655,6 +695,7 @@ def main():
                           "p99": round(float(np.percentile(per_step, 99)), 2)},
         "streaming_add_GBps": round(stream_gbs, 1),
         "rotating_indexes": rot,
+        "q8_shadow_layout": q8_leg,
         "sample_threshold_us": round(thr_us, 2),
         "step_with_sample_threshold_us": round(step_thr_us, 2),
         "dense_attention_us": {k: round(v, 2) for k, v in dense_us.items()},

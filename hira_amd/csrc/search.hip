@@ -96,8 +96,11 @@ __global__ __launch_bounds__(256) void search_kernel(const SearchParams p) {
     const bool vchunk_ok = ch * EPL < Dv;
     const bool want_attn = p.part_acc != nullptr;
 
-    const int hoff = p.tree_q_off[tree] + blockIdx.z * GMAX;
-    const int G = min(GMAX, p.tree_q_off[tree + 1] - hoff);
+    // (group_size > 0: head h of the launch belongs to tree h / group_size; the head map is not
+    // read, which saves every wave two dependent trips to memory)
+    const bool by_group = p.group_size > 0;
+    const int hoff = (by_group ? tree * p.group_size : p.tree_q_off[tree]) + blockIdx.z * GMAX;
+    const int G = min(GMAX, (by_group ? (tree + 1) * p.group_size : p.tree_q_off[tree + 1]) - hoff);
     if (G <= 0) return;  // uniform for the workgroup
     const unsigned gmask = (1u << G) - 1u;
 
@@ -107,7 +110,7 @@ __global__ __launch_bounds__(256) void search_kernel(const SearchParams p) {
     float tau[GMAX], sc[GMAX], qn[GMAX];
 #pragma unroll
     for (int g = 0; g < GMAX; ++g) {
-        qh[g] = (g < G) ? p.tree_q_heads[hoff + g] : 0;
+        qh[g] = (g < G) ? (by_group ? hoff + g : p.tree_q_heads[hoff + g]) : 0;
         uint4 raw = make_uint4(0, 0, 0, 0);
         if (g < G && chunk_ok) raw = load_chunk<T>(p.q, (size_t)qh[g] * D, ch);
         unpack<T>(raw, qf[g]);
@@ -156,7 +159,20 @@ __global__ __launch_bounds__(256) void search_kernel(const SearchParams p) {
         unsigned alive = node_ok ? gmask : 0u;
         int cnt = 0;
         if (real_nodes) {
-            // ancestors at levels L-1 .. 2 (independent loads, issued together)
+            // the node's own row, radius and child count, and its ancestors at levels L-1 .. 2:
+            // independent loads, issued together (the node's are wasted when an ancestor
+            // prunes it, which costs bandwidth the gates have to spare, not a trip to memory)
+            uint4 raw1 = make_uint4(0, 0, 0, 0);
+            float rad1 = 0.0f;
+            int cnt1 = 0;
+            if (node_ok) {
+                const size_t r = (size_t)tree * p.cap[1] + node;
+                if (chunk_ok)
+                    raw1 = load_row_chunk<T>(p.centers[1], p.layout, D, (size_t)tree * p.cap[1],
+                                             node, ch);
+                rad1 = p.radii[1][r];
+                cnt1 = p.counts[1][r];
+            }
             uint4 araw[HIRA_MAX_LEVELS - 2];
             float arad[HIRA_MAX_LEVELS - 2];
             int aid[HIRA_MAX_LEVELS - 2];
@@ -203,16 +219,11 @@ __global__ __launch_bounds__(256) void search_kernel(const SearchParams p) {
             }
             // the level-1 node itself, only if some head is still alive above it
             if (alive) {
-                const size_t r = (size_t)tree * p.cap[1] + node;
-                uint4 raw = make_uint4(0, 0, 0, 0);
-                if (chunk_ok)
-                    raw = load_row_chunk<T>(p.centers[1], p.layout, D, (size_t)tree * p.cap[1],
-                                            node, ch);
-                const float rad = p.radii[1][r];
-                cnt = p.counts[1][r];
+                const float rad = rad1;
+                cnt = cnt1;
                 if (p.stats && ch == 0 && rad > -INFINITY) st_nodes[1]++;
                 float kf[EPL];
-                unpack<T>(raw, kf);
+                unpack<T>(raw1, kf);
                 unsigned pass = 0;
 #pragma unroll
                 for (int g = 0; g < GMAX; ++g) {
@@ -369,7 +380,7 @@ __global__ __launch_bounds__(256) void search_kernel(const SearchParams p) {
             a += ws[e] * f;
             lsum += ws[DVP + 1] * f;
         }
-        const int head = p.tree_q_heads[hoff + g];
+        const int head = by_group ? hoff + g : p.tree_q_heads[hoff + g];
         const size_t slot = (size_t)head * p.num_parts + blockIdx.x;
         // device-scope stores: written through, so that the workgroup that folds the partials
         // (maybe behind another L2) reads them without cache-wide flushes
@@ -395,7 +406,7 @@ __global__ __launch_bounds__(256) void search_kernel(const SearchParams p) {
     __syncthreads();
     if (!s_last) return;
     for (int g = 0; g < G; ++g) {  // uniform
-        const int head = p.tree_q_heads[hoff + g];
+        const int head = by_group ? hoff + g : p.tree_q_heads[hoff + g];
         fold_partials(p.part_m + (size_t)head * p.num_parts, p.part_l + (size_t)head * p.num_parts,
                       p.part_acc + (size_t)head * p.num_parts * Dv, p.num_parts, Dv, p.fold_dvl,
                       p.attn_out + (size_t)head * Dv, smem, s_fold_red);

@@ -129,7 +129,8 @@ def test_cache_layer_uses_its_sample_rule(gpu_device):
             continue
         compared += 1
         ref = ho.attention(keys[:, :n], vals[:, :n], q, sc, mask, q2kv)
-        assert rel_err(att.float().cpu().numpy().reshape(h_q, d), ref) <= 1e-2, step
+        # (2e-3 for the attention plus the rounding of the returned tensor to bf16)
+        assert rel_err(att.float().cpu().numpy().reshape(h_q, d), ref) <= 2e-3 + 2.0 ** -8, step
         assert 0 < mask[:, : layer.indexed_len].mean() < 0.5
     assert compared >= 3
 

@@ -211,7 +211,9 @@ def test_cache_layer_end_to_end(gpu_device):
         vv = V[:, :, :n].float().repeat_interleave(h_q // h_kv, 1)
         ref = torch.nn.functional.scaled_dot_product_attention(q.float(), kk, vv, scale=d ** -0.5)
         err = (att.float().transpose(1, 2) - ref).abs().max() / ref.abs().max()
-        assert float(err) < 1e-2, float(err)
+        # 2e-3 for the attention itself plus the rounding of the returned tensor to bf16 (half a
+        # unit in the last place of the largest component: 2^-9, at most twice that below it)
+        assert float(err) <= 2e-3 + 2.0 ** -8, float(err)
 
 
 def test_decode_plan_survives_updates_and_queue_changes(gpu_device):
