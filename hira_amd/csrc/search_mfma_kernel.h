@@ -281,10 +281,13 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     // level-1 node behind entry n (tile n / 16 of mine, node n % 16 of the tile)
     auto node_of = [&](int n) { return tile_of(n >> 4) * 16 + (n & 15); };
     const bool is_queue = (int)blockIdx.y >= p.tree_blocks;  // the workgroup after the tree's
-#ifdef HIRA_TIMELINE  // experiment builds only: p.stats receives 8 time stamps per workgroup
+#ifdef HIRA_TIMELINE  // experiment builds only: p.stats receives 32 entries per workgroup: 16
+                      // time stamps of its first thread, then per wave the time its rounds
+                      // ended and the rows it listed
     unsigned long long* stats = nullptr;
     unsigned long long* tl =
-        p.stats + (((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 16;
+        p.stats + (((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 32;
+    unsigned long long tl_rows = 0;
 #define HIRA_TL(k) do { if (threadIdx.x == 0) tl[k] = wall_clock64(); } while (0)
 #else
     unsigned long long* stats = p.stats ? p.stats + (size_t)tree * HIRA_STATS_COLS : nullptr;
@@ -930,6 +933,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
 #ifdef HIRA_TIMELINE
             if (pr == 0) HIRA_TL(9);
             if (threadIdx.x == 0 && pr == 0) { tl[6] = (unsigned long long)tot; tl[12] = (unsigned long long)rounds; }
+            tl_rows += (unsigned long long)tot;
 #endif
             if (tot == 0) return;  // uniform in the wave: nothing selected in my rows
 
@@ -1036,6 +1040,12 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         }
     }  // tree or queue
     if (!want_attn) return;  // uniform
+#ifdef HIRA_TIMELINE
+    if (lane == 0) {
+        tl[16 + wave] = wall_clock64();
+        tl[24 + wave] = tl_rows;
+    }
+#endif
     HIRA_TL(2);
 
     // ---- merge the waves: first one maximum per head for the workgroup, to which every wave
