@@ -865,7 +865,8 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
 #pragma unroll
                 for (int ps = 0; ps < NPASS; ++ps)
                     slot_v[ps] = at_v[ps] >= 0 ? (int)(lst_tslot[at_v[ps] >> 4] + (unsigned)(at_v[ps] & 15)) : 0;
-                // (a batch is always loaded whole, rows past the end as slot 0: straight-line code)
+                // (a batch is always loaded whole, rows past the end as slot 0: straight-line code;
+                // loads under conditions of their own cost more than they save)
 #pragma unroll
                 for (int i = 0; i < kVBatch; ++i) {
                     {
@@ -922,39 +923,29 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
             };
             // ---- what is left to do with the rows of a round (`pr`; the lists and `tot` are its):
             // the best selected score of every head, the sums rescaled to it, the value rows ----------
-            auto finish = [&](int pr, const int (&at_v0)[NPASS], const uint32_t (&vraw0)[kVBatch][VW]) {
-                (void)pr;
-            if (!want_attn) return;  // uniform in the launch
-
-            // ---- the best selected score of every head in my rows of this round --------------------
-            zmax = fmaxf(zmax, __shfl_xor(zmax, 16, 64));
-            zmax = fmaxf(zmax, __shfl_xor(zmax, 32, 64));
-            const float rmax = zmax;
-#ifdef HIRA_TIMELINE
-            if (pr == 0) HIRA_TL(9);
-            if (threadIdx.x == 0 && pr == 0) { tl[6] = (unsigned long long)tot; tl[12] = (unsigned long long)rounds; }
-            tl_rows += (unsigned long long)tot;
-#endif
-            if (tot == 0) return;  // uniform in the wave: nothing selected in my rows
-
-            // the new maximum of every head, and what it does to the sums so far; head g lives in
-            // lane g; the weights below are computed with lane = (row, head), head = lane % GS
-            const float mnew = fmaxf(m_run, rmax);
-            const float f = (m_run == mnew) ? 1.0f : exp2f(m_run - mnew);
-            m_run = mnew;
-            // a head without a selected key has m = -inf and only z = -inf: any finite stand-in
-            const float m_lane = __shfl(mnew == -INFINITY ? 0.0f : mnew, lane_o & (GS - 1), 64);
-            if (__ballot(f != 1.0f) != 0ull) {  // uniform
-                l_mine *= __shfl(f, lane_o & (GS - 1), 64);
+            // ---- the best selected score of every head among rows just scored (zmax), the new
+            // running maximum, and what it does to the sums so far; head g lives in lane g; the
+            // weights are computed with lane = (row, head), head = lane % GS -----------------------
+            float m_lane = 0.0f;  // the running maximum of head lane % GS (a finite stand-in for -inf)
+            auto raise_max = [&]() {
+                zmax = fmaxf(zmax, __shfl_xor(zmax, 16, 64));
+                zmax = fmaxf(zmax, __shfl_xor(zmax, 32, 64));
+                const float mnew = fmaxf(m_run, zmax);
+                const float f = (m_run == mnew) ? 1.0f : exp2f(m_run - mnew);
+                m_run = mnew;
+                // a head without a selected key has m = -inf and only z = -inf: any finite stand-in
+                m_lane = __shfl(mnew == -INFINITY ? 0.0f : mnew, lane_o & (GS - 1), 64);
+                if (__ballot(f != 1.0f) != 0ull) {  // uniform
+                    l_mine *= __shfl(f, lane_o & (GS - 1), 64);
 #pragma unroll
-                for (int g = 0; g < GS; ++g) {
-                    const float fg = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), g));
+                    for (int g = 0; g < GS; ++g) {
+                        const float fg = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), g));
 #pragma unroll
-                    for (int e = 0; e < VPL; ++e) acc[g][e] *= fg;
+                        for (int e = 0; e < VPL; ++e) acc[g][e] *= fg;
+                    }
                 }
-            }
-
-            // ---- gather my listed rows ------------------------------------------------------------
+            };
+            // ---- a batch of value rows into the sums -----------------------------------------------
             auto consume = [&](int e0, const int (&at_v)[NPASS], const uint32_t (&vraw)[kVBatch][VW]) {
                 // (nothing of what follows may be scheduled ahead of loads issued before this point)
                 __builtin_amdgcn_sched_barrier(0);
@@ -991,51 +982,83 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                     }
                 }
             };
-            if constexpr (Q8) consume(0, at_v0, vraw0);
-            for (int e0 = Q8 ? kVBatch : 0; e0 < tot; e0 += kVBatch) {  // uniform in the wave
-                int at_v[NPASS];
-                uint32_t vraw[kVBatch][VW];
-                issue(e0, at_v, vraw);
-                consume(e0, at_v, vraw);
-            }
-            if (pr == 0) HIRA_TL(11);
-            if (pr == 1) HIRA_TL(13);
-            if (pr == 2) HIRA_TL(14);
-            };
+#ifdef HIRA_TIMELINE
+            if (threadIdx.x == 0 && r == 0) { tl[6] = (unsigned long long)tot; tl[12] = (unsigned long long)rounds; }
+            tl_rows += (unsigned long long)tot;
+#endif
             if constexpr (Q8) {
-                // Order of the requests: the value rows of the first batch (most rows that the shadow
-                // lets through are selected), the key rows of the first KB0 * 16 listed rows, and only
-                // then the tiles of the next round -- loads come back in the order they were asked
-                // for, so the exact test and the gather wait for the rows alone and run while the
-                // next round's tiles are on their way.
-                int at_v0[NPASS], at_k[KB0];
-                uint32_t vraw0[kVBatch][VW];
-                unsigned slot_k[KB0];
-                uint4 kr0[KB0][KS];
-                __builtin_amdgcn_sched_barrier(0);
-                if (want_attn) issue(0, at_v0, vraw0);
-                __builtin_amdgcn_sched_barrier(0);
+                // The listed rows go kVBatch at a time: the value rows of the batch (most rows that
+                // the shadow lets through are selected) and their key rows are asked for together,
+                // so a batch costs one trip to memory: exact test, the running maximum raised to the
+                // batch's best scores, the batch's values into the sums.  The first batch is asked
+                // for ahead of the next round's tiles -- loads come back in the order they were asked
+                // for, so its rows are waited for alone, and its work runs while the tiles are on
+                // their way.
+                constexpr int KBV = kVBatch / 16;  // batches of 16 key rows per batch of value rows
+                {
+                    int at_v0[NPASS], at_k[KB0];
+                    uint32_t vraw0[kVBatch][VW];
+                    unsigned slot_k[KB0];
+                    uint4 kr0[KB0][KS];
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (want_attn) issue(0, at_v0, vraw0);
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int b = 0; b < KB0; ++b) rows16(16 * b, at_k[b], slot_k[b], kr0[b]);
-                __builtin_amdgcn_sched_barrier(0);
-                fetch(r + 1, -1);  // (past the last round: no node, nothing read)
-                __builtin_amdgcn_sched_barrier(0);
+                    for (int b = 0; b < KB0; ++b) rows16(16 * b, at_k[b], slot_k[b], kr0[b]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    fetch(r + 1, -1);  // (past the last round: no node, nothing read)
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int b = 0; b < KB0; ++b)
-                    if (16 * b < tot) exact16(at_k[b], slot_k[b], kr0[b]);  // uniform
-                for (int e0 = 16 * KB0; e0 < tot; e0 += 16) {  // uniform in the wave; seldom
-                    int at;
-                    unsigned slot;
-                    uint4 kr[KS];
-                    rows16(e0, at, slot, kr);
-                    exact16(at, slot, kr);
+                    for (int b = 0; b < KB0; ++b)
+                        if (16 * b < tot) exact16(at_k[b], slot_k[b], kr0[b]);  // uniform
+                    for (int e0 = 16 * KB0; e0 < min(tot, kVBatch); e0 += 16) {  // (wide rows only)
+                        int at;
+                        unsigned slot;
+                        uint4 kr[KS];
+                        rows16(e0, at, slot, kr);
+                        exact16(at, slot, kr);
+                    }
+                    if (r == 0) HIRA_TL(9);
+                    if (want_attn && tot > 0) {  // uniform
+                        raise_max();
+                        consume(0, at_v0, vraw0);
+                    }
                 }
-                finish(r, at_v0, vraw0);
+                for (int e0 = kVBatch; e0 < tot; e0 += kVBatch) {  // uniform in the wave; a hot wave
+                    int at_v[NPASS], at_k[KB0];
+                    uint32_t vraw[kVBatch][VW];
+                    unsigned slot_k[KB0];
+                    uint4 kr[KB0][KS];
+                    zmax = -INFINITY;
+                    if (want_attn) issue(e0, at_v, vraw);
+#pragma unroll
+                    for (int b0 = 0; b0 < KBV; b0 += KB0) {
+#pragma unroll
+                        for (int b = 0; b < KB0; ++b) rows16(e0 + 16 * (b0 + b), at_k[b], slot_k[b], kr[b]);
+#pragma unroll
+                        for (int b = 0; b < KB0; ++b)
+                            if (e0 + 16 * (b0 + b) < tot) exact16(at_k[b], slot_k[b], kr[b]);  // uniform
+                    }
+                    if (want_attn) {
+                        raise_max();
+                        consume(e0, at_v, vraw);
+                    }
+                }
             } else {
-                int none_at[NPASS];
-                uint32_t none_v[kVBatch][VW];
-                finish(r, none_at, none_v);
+                if (r == 0) HIRA_TL(9);
+                if (want_attn && tot > 0) {  // uniform in the launch / in the wave
+                    raise_max();
+                    for (int e0 = 0; e0 < tot; e0 += kVBatch) {  // uniform in the wave
+                        int at_v[NPASS];
+                        uint32_t vraw[kVBatch][VW];
+                        issue(e0, at_v, vraw);
+                        consume(e0, at_v, vraw);
+                    }
+                }
             }
+            if (r == 0) HIRA_TL(11);
+            if (r == 1) HIRA_TL(13);
+            if (r == 2) HIRA_TL(14);
             if (r == 3) HIRA_TL(15);
         }
     }  // tree or queue
