@@ -286,12 +286,14 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                       // ended and the rows it listed
     unsigned long long* stats = nullptr;
     unsigned long long* tl =
-        p.stats + (((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 32;
+        p.stats + (((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 64;
     unsigned long long tl_rows = 0;
+#define HIRA_TLW(k) do { if ((threadIdx.x & 63) == 0) tl[(k) + (threadIdx.x >> 6)] = wall_clock64(); } while (0)
 #define HIRA_TL(k) do { if (threadIdx.x == 0) tl[k] = wall_clock64(); } while (0)
 #else
     unsigned long long* stats = p.stats ? p.stats + (size_t)tree * HIRA_STATS_COLS : nullptr;
 #define HIRA_TL(k) do { } while (0)
+#define HIRA_TLW(k) do { } while (0)
 #endif
     HIRA_TL(0);
 
@@ -850,6 +852,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 }
                 }  // shadow or bf16 tiles
             }
+            if (r == 0) HIRA_TLW(32);
             const int tot = nsel;  // rows on my list
             if (r == 0) HIRA_TL(10);
 
@@ -959,18 +962,24 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                         *zp = w;
                     }
                 }
+                // eight rows at a time: one test whether the list goes that far, no branch between
+                // the rows of an eight (their weights and products can then be in flight together);
+                // a row past the end reads the weights of the batch's first row and counts for nothing
+                const int at_first = __builtin_amdgcn_readlane(at_v[0], 0);
 #pragma unroll
                 for (int i = 0; i < kVBatch; ++i) {
-                    if (e0 + i >= tot) break;  // uniform
-                    const int at = __builtin_amdgcn_readlane(at_v[i / RP], (i % RP) * GS);
+                    if ((i & 7) == 0 && e0 + i >= tot) break;  // uniform
+                    const bool there = e0 + i < tot;           // uniform
+                    const int at_i = __builtin_amdgcn_readlane(at_v[i / RP], (i % RP) * GS);
+                    const int at = there ? at_i : at_first;
                     float vf[VPL];
                     if (VPL == 1) {
-                        vf[0] = bf16_lo(vraw[i][0]);
+                        vf[0] = there ? bf16_lo(vraw[i][0]) : 0.0f;
                     } else {
 #pragma unroll
                         for (int e = 0; e < VPL / 2; ++e) {
-                            vf[2 * e] = bf16_lo(vraw[i][e]);
-                            vf[2 * e + 1] = bf16_hi(vraw[i][e]);
+                            vf[2 * e] = there ? bf16_lo(vraw[i][e]) : 0.0f;
+                            vf[2 * e + 1] = there ? bf16_hi(vraw[i][e]) : 0.0f;
                         }
                     }
                     const float* wr = lst_z + at * GS;  // weights of this row, one per head
@@ -1000,6 +1009,9 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                     uint32_t vraw0[kVBatch][VW];
                     unsigned slot_k[KB0];
                     uint4 kr0[KB0][KS];
+                    // (these loads go out whatever the list holds, rows past its end as slot 0: under
+                    // a condition -- even one for all of them -- the waits below can no longer count
+                    // the loads behind them and wait for the next round's tiles as well)
                     __builtin_amdgcn_sched_barrier(0);
                     if (want_attn) issue(0, at_v0, vraw0);
                     __builtin_amdgcn_sched_barrier(0);
@@ -1019,10 +1031,12 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                         exact16(at, slot, kr);
                     }
                     if (r == 0) HIRA_TL(9);
+                    if (r == 0) HIRA_TLW(40);
                     if (want_attn && tot > 0) {  // uniform
                         raise_max();
                         consume(0, at_v0, vraw0);
                     }
+                    if (r == 0) HIRA_TLW(48);
                 }
                 for (int e0 = kVBatch; e0 < tot; e0 += kVBatch) {  // uniform in the wave; a hot wave
                     int at_v[NPASS], at_k[KB0];
@@ -1052,7 +1066,9 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                         int at_v[NPASS];
                         uint32_t vraw[kVBatch][VW];
                         issue(e0, at_v, vraw);
+                        if (r == 0 && e0 == 0) HIRA_TLW(40);
                         consume(e0, at_v, vraw);
+                        if (r == 0 && e0 == 0) HIRA_TLW(48);
                     }
                 }
             }
