@@ -70,8 +70,13 @@ struct SearchPlan {
     int num_nodes, num_queue_blocks;
     int tree_blocks, queue_blocks, head_chunks;
     int share;        // MFMA kernel: see SearchParams
+    int gate_steps;   // vector-ALU kernel: steps of gates a wave batches (1 or 4)
     size_t smem;
 };
+
+// search_vec_f32.hip, search_vec_bf16.hip: the vector-ALU kernel for rows of one element type
+int launch_vec_f32(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
+int launch_vec_bf16(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
 
 // search_mfma.hip
 bool mfma_search_supported(const HiraTree* t, const HiraQueue* queue);

@@ -211,6 +211,81 @@ def test_device_counters_match_oracle_traffic(gpu_device):
     assert (tr[:, 0] < 4096).all()  # the clustered keys are really pruned
 
 
+BATCHED_GATE_CASES = [
+    # h_kv, h_q, n, d, bf, levels, dtype, keep, nodes per wave
+    (1, 1, 3001, 128, 4, 3, torch.float32, 30, 8),
+    (1, 1, 3001, 128, 4, 3, torch.float32, 30, 5),     # a batch that ends inside a step of gates
+    (2, 8, 1500, 128, 4, 3, torch.float32, 25, 16),    # 4 heads per tree, two batches per wave
+    (1, 12, 900, 128, 2, 3, torch.float32, 20, 8),     # fan-out 2, 12 heads per tree: two passes
+    (2, 4, 1111, 128, 3, 4, torch.float32, 22, 8),     # odd fan-out, four levels
+    (2, 4, 1500, 256, 4, 3, torch.bfloat16, 25, 8),
+    (1, 2, 2000, 128, 2, 2, torch.bfloat16, 40, 16),
+]
+
+
+@pytest.mark.parametrize("case", BATCHED_GATE_CASES,
+                         ids=[f"hkv{c[0]}_hq{c[1]}_n{c[2]}_d{c[3]}_bf{c[4]}_L{c[5]}_"
+                              f"{'bf16' if c[6] == torch.bfloat16 else 'f32'}_npw{c[8]}"
+                              for c in BATCHED_GATE_CASES])
+def test_small_fanout_with_batched_gates(case, gpu_device):
+    """Fan-outs of 2 .. 4: a wave evaluates the gates of several steps of nodes together and scans
+    their keys as one block (what the library picks by itself for large trees; forced here through
+    the launch override).  Same selected set, scores, lists, counters and attention output as the
+    oracle and as the launch that takes one step of nodes at a time."""
+    from hira_amd.searcher.hip import HIPSearcher
+    from hira_amd import _lib
+
+    h_kv, h_q, n, d, bf, nl, dtype, keep, npw = case
+    print(f"case {case}", flush=True)
+    c = _setup(h_kv, h_q, n, d, bf, nl, dtype, seed=700 + n, keep=keep)
+    scale = d ** -0.5
+    sc = torch.full((h_q,), scale)
+    q, th = torch.from_numpy(c["q"]), torch.from_numpy(c["th"])
+    plain, batched = HIPSearcher(nodes_per_wave=1), HIPSearcher(nodes_per_wave=npw)
+    st0 = torch.zeros((h_kv, _lib.HIRA_STATS_COLS), dtype=torch.int64, device="cuda")
+    st1 = torch.zeros_like(st0)
+    ref_out = plain.search(q, th, c["idx"], scaling=sc, stats=st0)
+    out = batched.search(q, th, c["idx"], scaling=sc, stats=st1)
+    assert torch.equal(out, ref_out)
+    assert torch.equal(st0, st1)
+    out = out.cpu().numpy()
+    s = np.where(c["valid"], c["s"], -np.inf).astype(np.float32)
+    assert_same_selection(out != 0, s, c["th"])
+    m = out != 0
+    np.testing.assert_allclose(out[m], (c["s"] * scale)[m], rtol=2e-5, atol=1e-6)
+    idx, score, count = batched.search_compact(q, th, c["idx"], scaling=sc)
+    idx, count = idx.cpu().numpy(), count.cpu().numpy()
+    for h in range(h_q):
+        assert np.array_equal(np.sort(idx[h, :count[h]]), np.nonzero(m[h])[0])
+    att = batched.search_attention(q, th, c["idx"], scaling=sc).cpu().numpy()
+    mask = (c["s"] >= c["th"][:, None]) & c["valid"]
+    ref = ho.attention(c["ff"].keys, c["vslot"], c["q"], sc.numpy(), mask, c["q2kv"])
+    ok = band_free_heads(c["s"], c["th"], c["valid"])
+    assert ok.sum() >= max(1, h_q - 1)
+    tol = 2e-3 if dtype == torch.bfloat16 else 1e-5
+    assert rel_err(att[ok], ref[ok]) <= tol, rel_err(att[ok], ref[ok])
+
+
+@pytest.mark.parametrize("n", [40000, 90000])
+def test_large_tree_of_small_fanout_picks_batched_gates(n, gpu_device):
+    """At 40k / 90k keys with fan-out 4 the library batches two / four steps of gates by itself:
+    same output as the one-step launch, and the selected set is the brute-force one."""
+    from hira_amd.indexer.hip import HIPIndexer
+    from hira_amd.searcher.hip import HIPSearcher
+
+    g = torch.Generator().manual_seed(n)
+    keys = torch.nn.functional.normalize(torch.randn(1, 1, n, 128, generator=g), dim=-1).cuda()
+    q = torch.nn.functional.normalize(torch.randn(1, 128, generator=g), dim=-1).cuda()
+    idx = HIPIndexer(3, 1, 4).build(keys)
+    s = (keys[0, 0] @ q[0]).cpu().numpy()
+    th = midpoint_threshold(s[None], 50)
+    auto = HIPSearcher().search(q, torch.from_numpy(th), idx, index_space="position")
+    plain = HIPSearcher(nodes_per_wave=2).search(q, torch.from_numpy(th), idx,
+                                                 index_space="position")
+    assert torch.equal(auto, plain)
+    assert_same_selection(auto.cpu().numpy() != 0, s[None], th)
+
+
 ATTN_CASES = [
     (1, 1, 4096, 128, 16, 2, torch.float32, 205, 1e-5),
     (2, 8, 2048, 128, 32, 3, torch.bfloat16, 41, 2e-3),
