@@ -40,6 +40,8 @@ struct SearchParams {
     int32_t tree_blocks;     // workgroups that walk the tree; the rest scan the queue
     int32_t share;           // MFMA kernel: workgroups that gate the same tiles and split what
                              // survives (tree_blocks is a multiple of it)
+    int32_t key_policy;      // MFMA kernel: which cache policy the scan's loads use (0: default,
+                             // 1: key tiles non-temporal, 2: value rows too), by the launch's size
     int32_t num_nodes;       // level-1 nodes (or pseudo blocks over the keys when L == 1)
     int32_t num_queue_blocks;
     // outputs

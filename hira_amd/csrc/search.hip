@@ -269,6 +269,11 @@ static int search_impl(const HiraTree* tree, const HiraQuery* query, const HiraQ
     p.nodes_per_wave = plan.nodes_per_wave;
     p.tree_blocks = plan.tree_blocks;
     p.share = plan.kernel == 2 ? plan.share : 1;
+    {   // up to what the eight L2s hold together (32 MiB) the default policy; up to 512 MiB the
+        // key tiles and the value rows non-temporal; beyond, the key tiles only
+        const size_t key_bytes = (size_t)tree->num_trees * (size_t)tree->size[0] * (size_t)tree->dim * 2;
+        p.key_policy = key_bytes <= ((size_t)32 << 20) ? 0 : (key_bytes <= ((size_t)512 << 20) ? 2 : 1);
+    }
     p.num_nodes = plan.num_nodes;
     p.num_queue_blocks = use_queue ? plan.num_queue_blocks : 0;
     p.dense = out->dense;

@@ -18,10 +18,17 @@ bool mfma_search_supported(const HiraTree* t, const HiraQueue* queue) {
 // grid: x = tree, y = tile of 16 level-1 nodes, z = pass of 16 heads
 int launch_search_mfma(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s) {
     const bool q8 = p.keys8 != nullptr;  // the scan reads the keys' 8-bit shadow
+    const int pol = q8 ? 0 : p.key_policy;  // cache policy of the bf16 tiles and the value rows
+    typedef void (*Launch)(const SearchPlan&, const SearchParams&, dim3, hipStream_t);
+    static const Launch table[3][4] = {
+        {launch_mfma_d64, launch_mfma_nt1_d64, launch_mfma_nt2_d64, launch_mfma_q8_d64},
+        {launch_mfma_d128, launch_mfma_nt1_d128, launch_mfma_nt2_d128, launch_mfma_q8_d128},
+        {launch_mfma_d256, launch_mfma_nt1_d256, launch_mfma_nt2_d256, launch_mfma_q8_d256}};
+    const int col = q8 ? 3 : pol;
     switch (p.dim) {
-        case 64: (q8 ? launch_mfma_q8_d64 : launch_mfma_d64)(plan, p, grid, s); return HIRA_OK;
-        case 128: (q8 ? launch_mfma_q8_d128 : launch_mfma_d128)(plan, p, grid, s); return HIRA_OK;
-        case 256: (q8 ? launch_mfma_q8_d256 : launch_mfma_d256)(plan, p, grid, s); return HIRA_OK;
+        case 64: table[0][col](plan, p, grid, s); return HIRA_OK;
+        case 128: table[1][col](plan, p, grid, s); return HIRA_OK;
+        case 256: table[2][col](plan, p, grid, s); return HIRA_OK;
         default: return fail(HIRA_EINVAL, "MFMA kernel: dim %d", p.dim);
     }
 }

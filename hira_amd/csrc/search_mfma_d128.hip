@@ -3,6 +3,6 @@
 
 namespace hira {
 void launch_mfma_d128(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s) {
-    launch_mfma_mt<4, false>(plan, p, grid, s);
+    launch_mfma_mt<4, false, 0>(plan, p, grid, s);
 }
 }  // namespace hira

@@ -99,13 +99,27 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, si
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)(uint32_t)bytes, 0x00020000);
 }
 
-template <int KS>
+// Cache policy of the scan's two streams.  A step reads a key tile once, so where the keys of a
+// launch are more than the L2s hold they are better loaded non-temporal: they then do not push the
+// centres, the queries and the value rows out on their way through.  POL 0: default policy for
+// both; 1: key tiles non-temporal; 2: key tiles and value rows non-temporal.  Measured per step
+// (keys of the launch: 67 MB / 268 MB / 1.07 GB): POL 0 20.11 / 65.05 / 197.3 us, POL 1 21.34 /
+// 65.6 / 181.3 us, POL 2 19.86 / 66.1 / 185.1 us; with eight 67 MB indexes taking turns 22.9 /
+// 22.2 / 22.2 us; and 15 % MORE than POL 0 where a caller searches the same 23 MB of keys again
+// and again, which the L2s would have kept.  The host picks by the size of the launch's keys; a
+// branch around the loads instead of instantiations costs the small launches a microsecond.  The
+// coherence bits of the policy (sc0, sc1) change nothing.  The tiles of the 8-bit shadow keep the
+// default policy: non-temporal they lose more than they gain.
+constexpr int kReadOnce = 2;   // the `nt` bit of a buffer load's cache policy
+
+template <int KS, bool ONCE>
 __device__ __forceinline__ void load_tile_buf(__amdgpu_buffer_rsrc_t rsrc, unsigned lane_off,
                                               unsigned tile_off, uint4 (&a)[KS]) {
 #pragma unroll
     for (int s = 0; s < KS; ++s)
-        a[s] = __builtin_bit_cast(
-            uint4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, lane_off + (unsigned)(s * 1024), tile_off, 0));
+        a[s] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
+                                             rsrc, lane_off + (unsigned)(s * 1024), tile_off,
+                                             ONCE ? kReadOnce : 0));
 }
 
 // the same with the B operand parked in LDS (chunk s of lane l at [s*64 + l]): the scan keeps
@@ -228,7 +242,7 @@ __device__ __forceinline__ void gate_issue(const SearchParams& p, int tree, int 
 // head; their bf16 rows (row-major) are fetched, 16 at a time as one MFMA operand, and take the
 // exact test -- with the very products of the other layout, so the selected set and the scores
 // are the same bit for bit.
-template <int KS, int MT, int GS, bool OUT, bool Q8>
+template <int KS, int MT, int GS, bool OUT, bool Q8, int POL>
 __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const SearchParams p) {
     using S = MfmaShape<KS, MT, GS, Q8>;
     constexpr int D = S::D;
@@ -581,12 +595,12 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         // share, ... of them, dealt round-robin to the waves ----------------------------------------
         int rounds, alive = 0;
         {
-            const int NT = ntile * 16;
+            const int n_info = ntile * 16;
             const unsigned long long lt = (1ull << lane) - 1ull;
 #pragma unroll
             for (int i = 0; i < kMfmaMaxTilesPerWg * 16 / 64; ++i) {
-                if (64 * i >= NT) break;  // uniform
-                const uint32_t info = 64 * i + lane < NT ? s_ninfo[64 * i + lane] : 0u;
+                if (64 * i >= n_info) break;  // uniform
+                const uint32_t info = 64 * i + lane < n_info ? s_ninfo[64 * i + lane] : 0u;
                 const bool live = (info & 0xFFFFu) != 0u;
                 const unsigned long long all = __ballot(live);
                 if (live)
@@ -652,11 +666,11 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                         // every load is issued, whatever the node (straight-line code, so that the
                         // waits further down can count the loads behind them); a tile that is not
                         // there is asked for beyond the end of the buffer: zeros, no memory access
-                        load_tile_buf<KA>(k8rsrc, (unsigned)lane * 16u + (tt * 16 < nx_cnt[u] ? 0u : 0x80000000u),
+                        load_tile_buf<KA, false>(k8rsrc, (unsigned)lane * 16u + (tt * 16 < nx_cnt[u] ? 0u : 0x80000000u),
                                           (tile_first + tt) * (unsigned)(KA * 1024), a[u][tt]);
                     } else {
                         if (tt * 16 < nx_cnt[u])
-                            load_tile_buf<KA>(krsrc, (unsigned)lane * 16u,
+                            load_tile_buf<KA, POL != 0>(krsrc, (unsigned)lane * 16u,
                                               (tile_first + tt) * (unsigned)(KA * 1024), a[u][tt]);
                     }
                 }
@@ -877,11 +891,11 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                         const unsigned voff = (unsigned)lane_o * (unsigned)(VPL * 2);
                         const unsigned soff = slot * (unsigned)(D * 2);
                         if (VPL == 1) {
-                            vraw[i][0] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(vrsrc, voff, soff, 0);
+                            vraw[i][0] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(vrsrc, voff, soff, POL == 2 ? kReadOnce : 0);
                         } else if (VPL == 2) {
-                            vraw[i][0] = __builtin_amdgcn_raw_buffer_load_b32(vrsrc, voff, soff, 0);
+                            vraw[i][0] = __builtin_amdgcn_raw_buffer_load_b32(vrsrc, voff, soff, POL == 2 ? kReadOnce : 0);
                         } else {
-                            const u32x2_t v2 = __builtin_amdgcn_raw_buffer_load_b64(vrsrc, voff, soff, 0);
+                            const u32x2_t v2 = __builtin_amdgcn_raw_buffer_load_b64(vrsrc, voff, soff, POL == 2 ? kReadOnce : 0);
                             vraw[i][0] = v2.x;
                             vraw[i][VW - 1] = v2.y;
                         }
@@ -1239,38 +1253,44 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     HIRA_TL(5);
 }
 
-template <int KS, int MT, bool Q8>
+template <int KS, int MT, bool Q8, int POL>
 void launch_mfma_gs(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s) {
     const dim3 block(plan.threads);
     const bool out = p.dense != nullptr || p.sel_count != nullptr;
     if (plan.gmax <= 4) {
-        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 4, true, Q8>), grid, block, 0, s, p);
-        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 4, false, Q8>), grid, block, 0, s, p);
+        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 4, true, Q8, POL>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 4, false, Q8, POL>), grid, block, 0, s, p);
     } else if (plan.gmax <= 8) {
-        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 8, true, Q8>), grid, block, 0, s, p);
-        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 8, false, Q8>), grid, block, 0, s, p);
+        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 8, true, Q8, POL>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 8, false, Q8, POL>), grid, block, 0, s, p);
     } else {
-        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 16, true, Q8>), grid, block, 0, s, p);
-        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 16, false, Q8>), grid, block, 0, s, p);
+        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 16, true, Q8, POL>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 16, false, Q8, POL>), grid, block, 0, s, p);
     }
 }
 
-template <int KS, bool Q8>
+template <int KS, bool Q8, int POL>
 void launch_mfma_mt(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s) {
     const int mt = p.bf / 16;
     if (mt <= 1)
-        launch_mfma_gs<KS, 1, Q8>(plan, p, grid, s);
+        launch_mfma_gs<KS, 1, Q8, POL>(plan, p, grid, s);
     else if (mt == 2)
-        launch_mfma_gs<KS, 2, Q8>(plan, p, grid, s);
+        launch_mfma_gs<KS, 2, Q8, POL>(plan, p, grid, s);
     else
-        launch_mfma_gs<KS, 4, Q8>(plan, p, grid, s);
+        launch_mfma_gs<KS, 4, Q8, POL>(plan, p, grid, s);
 }
 
-// one translation unit per key width (and per kind of scan: bf16 tiles, 8-bit shadow) keeps the
-// build parallel
+// one translation unit per key width and per kind of scan (bf16 tiles under each cache policy,
+// 8-bit shadow) keeps the build parallel
 void launch_mfma_d64(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
 void launch_mfma_d128(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
 void launch_mfma_d256(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
+void launch_mfma_nt1_d64(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
+void launch_mfma_nt2_d64(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
+void launch_mfma_nt1_d128(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
+void launch_mfma_nt2_d128(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
+void launch_mfma_nt1_d256(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
+void launch_mfma_nt2_d256(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
 void launch_mfma_q8_d64(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
 void launch_mfma_q8_d128(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
 void launch_mfma_q8_d256(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);

@@ -3,6 +3,6 @@
 
 namespace hira {
 void launch_mfma_q8_d64(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s) {
-    launch_mfma_mt<2, true>(plan, p, grid, s);
+    launch_mfma_mt<2, true, 0>(plan, p, grid, s);
 }
 }  // namespace hira
