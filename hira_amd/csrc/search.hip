@@ -119,8 +119,18 @@ static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* que
             tpw = (int)((all + cus - 1) / cus);
             if (tpw * 64 < tiles) tpw = (tiles + 63) / 64;
             if (tpw < 1) tpw = 1;
-            // more work than one workgroup per CU can take: several rounds of smaller ones
-            if (tpw > kMfmaMaxTilesPerWg) tpw = kMfmaMaxTilesPerWg / 2;
+            // more work than one workgroup per CU can take: several rounds of workgroups of 8 to 16
+            // tiles, of the size whose rounds add up to the least (a workgroup costs some two
+            // tiles' time before and after its scan; measured at 128 trees x 64 tiles: 16 tiles a
+            // workgroup 178 us, 8 tiles 182 us, 4 tiles 206 us)
+            if (tpw > kMfmaMaxTilesPerWg) {
+                int64_t best = 0;
+                for (int c = kMfmaMaxTilesPerWg; c >= kMfmaMaxTilesPerWg / 2; --c) {
+                    const int64_t wgs = (int64_t)((tiles + c - 1) / c) * t->num_trees * plan->head_chunks;
+                    const int64_t cost = ((wgs + cus - 1) / cus) * (c + 2);
+                    if (best == 0 || cost < best) best = cost, tpw = c;
+                }
+            }
         }
         // groups of `share` workgroups may gate the same share*tpw tiles (at most 16: two a wave)
         // and split the survivors evenly.  Off unless asked for: measured at the benchmark's
