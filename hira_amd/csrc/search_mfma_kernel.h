@@ -242,7 +242,7 @@ __device__ __forceinline__ void gate_issue(const SearchParams& p, int tree, int 
 // head; their bf16 rows (row-major) are fetched, 16 at a time as one MFMA operand, and take the
 // exact test -- with the very products of the other layout, so the selected set and the scores
 // are the same bit for bit.
-template <int KS, int MT, int GS, bool OUT, bool Q8, int POL>
+template <int KS, int MT, int GS, bool OUT, bool Q8, int POL, int HV>
 __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const SearchParams p) {
     using S = MfmaShape<KS, MT, GS, Q8>;
     constexpr int D = S::D;
@@ -256,7 +256,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     __shared__ uint32_t s_ninfo[kMfmaMaxTilesPerWg * 16];
     // the surviving ones in order, a copy per wave (each wave makes its own: no barrier):
     // node | child count << 8 | heads << 16
-    __shared__ uint32_t s_order[kMfmaWaves][kMfmaMaxTilesPerWg * 16];
+    __shared__ uint32_t s_order[kMfmaWaves][kMfmaMaxTilesPerWg * 16 * HV];
     __shared__ float s_mxw[kMfmaWaves * 16];           // a wave's running maximum per head
     __shared__ float s_lw[kMfmaWaves * 16];
     __shared__ float s_mh[kHeadsPerPass];
@@ -603,11 +603,20 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 const uint32_t info = 64 * i + lane < n_info ? s_ninfo[64 * i + lane] : 0u;
                 const bool live = (info & 0xFFFFu) != 0u;
                 const unsigned long long all = __ballot(live);
-                if (live)
-                    s_order[wave][alive + __popcll(all & lt)] =
-                        (uint32_t)(64 * i + lane) | ((info >> 16) << 8) | (info << 16);
+                if (live) {
+                    // (HV = 2: a node goes in as two entries of MT tiles each, the second marked
+                    // by bit 15; a half without keys costs its wave nothing but the entry)
+                    const int at = (alive + __popcll(all & lt)) * HV;
+                    const int cnt_n = (int)(info >> 16);
+#pragma unroll
+                    for (int h = 0; h < HV; ++h)
+                        s_order[wave][at + h] =
+                            (uint32_t)(64 * i + lane) | ((uint32_t)min(max(cnt_n - h * MT * 16, 0), MT * 16) << 8) |
+                            ((uint32_t)h << 15) | (info << 16);
+                }
                 alive += __popcll(all);
             }
+            alive *= HV;
             const int mine = alive > rep ? (alive - rep + share - 1) / share : 0;
             rounds = ((mine + nw - 1) / nw + NB - 1) / NB;
         }
@@ -636,7 +645,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
             reinterpret_cast<const uint16_t*>(p.values) + row0 * (size_t)D, (size_t)p.cap[0] * D * 2);
         // The nodes a wave takes in a round (up to NB of its share), what LDS says about them,
         // and the loads of their key tiles.
-        int nx_node[NB], nx_cnt[NB];
+        int nx_node[NB], nx_cnt[NB], nx_half[NB];
         uint32_t nx_mask[NB];
         float nx_eps[Q8 ? NB : 1];
         uint4 a[NB][MT][KA];
@@ -656,10 +665,11 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 const uint32_t e = (uint32_t)__builtin_amdgcn_readfirstlane((int)ent[u]);
                 const int n = (e >> 16) != 0u ? (int)(e & 0xFFu) : -1;
                 nx_node[u] = n;
-                nx_cnt[u] = (int)((e >> 8) & 0xFFu);
+                nx_cnt[u] = (int)((e >> 8) & 0x7Fu);
+                nx_half[u] = (int)((e >> 15) & 1u);
                 nx_mask[u] = e >> 16;
                 if constexpr (Q8) nx_eps[u] = s_keps[max(n, 0)];
-                const unsigned tile_first = (unsigned)(node_of(max(n, 0)) * bf) / 16u;
+                const unsigned tile_first = (unsigned)(node_of(max(n, 0)) * bf) / 16u + (unsigned)(nx_half[u] * MT);
 #pragma unroll
                 for (int tt = 0; tt < MT; ++tt) {
                     if constexpr (Q8) {
@@ -775,7 +785,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 node[u] = nx_node[u];
                 cnt[u] = nx_cnt[u];
                 nmask[u] = nx_mask[u];
-                const unsigned slot0 = (unsigned)(node_of(max(node[u], 0)) * bf);
+                const unsigned slot0 = (unsigned)(node_of(max(node[u], 0)) * bf) + (unsigned)(nx_half[u] * MT * 16);
                 if constexpr (Q8) {
                     // ---- the shadow's tiles: which rows can it not rule out, for which heads? ----
                     const float eps_u = nx_eps[u];
@@ -1303,19 +1313,19 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     HIRA_TL(5);
 }
 
-template <int KS, int MT, bool Q8, int POL>
+template <int KS, int MT, bool Q8, int POL, int HV = 1>
 void launch_mfma_gs(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s) {
     const dim3 block(plan.threads);
     const bool out = p.dense != nullptr || p.sel_count != nullptr;
     if (plan.gmax <= 4) {
-        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 4, true, Q8, POL>), grid, block, 0, s, p);
-        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 4, false, Q8, POL>), grid, block, 0, s, p);
+        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 4, true, Q8, POL, HV>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 4, false, Q8, POL, HV>), grid, block, 0, s, p);
     } else if (plan.gmax <= 8) {
-        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 8, true, Q8, POL>), grid, block, 0, s, p);
-        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 8, false, Q8, POL>), grid, block, 0, s, p);
+        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 8, true, Q8, POL, HV>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 8, false, Q8, POL, HV>), grid, block, 0, s, p);
     } else {
-        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 16, true, Q8, POL>), grid, block, 0, s, p);
-        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 16, false, Q8, POL>), grid, block, 0, s, p);
+        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 16, true, Q8, POL, HV>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 16, false, Q8, POL, HV>), grid, block, 0, s, p);
     }
 }
 
@@ -1326,6 +1336,10 @@ void launch_mfma_mt(const SearchPlan& plan, const SearchParams& p, dim3 grid, hi
         launch_mfma_gs<KS, 1, Q8, POL>(plan, p, grid, s);
     else if (mt == 2)
         launch_mfma_gs<KS, 2, Q8, POL>(plan, p, grid, s);
+    else if (KS == 8 && plan.gmax > 4)
+        // 256 columns x 64 keys a node x 8 or 16 heads: a node's four tiles do not fit the
+        // registers next to the accumulators; it is scanned as two halves of two tiles
+        launch_mfma_gs<KS, (KS == 8 ? 2 : 4), Q8, POL, (KS == 8 ? 2 : 1)>(plan, p, grid, s);
     else
         launch_mfma_gs<KS, 4, Q8, POL>(plan, p, grid, s);
 }

@@ -48,6 +48,8 @@ Q8_CASES = [
     (1, 4, 3000, 256, 48, 2, 60),       # d = 256, fan-out 48 (3 tiles per block)
     (1, 4, 5000, 128, 64, 3, 50),       # fan-out 64
     (2, 8, 40000, 128, 32, 4, 400),     # four levels
+    (1, 8, 3000, 256, 64, 2, 40),       # d = 256, fan-out 64, 8 heads: nodes scanned as two halves
+    (1, 16, 2600, 256, 64, 3, 30),      # the same with 16 heads
 ]
 
 
