@@ -18,7 +18,7 @@ namespace hira {
 constexpr int kTauThreads = 1024;
 constexpr int kTauWaves = kTauThreads / 64;
 constexpr int kTauMaxSamples = 4096;
-constexpr int kTauRows = 8;  // sample rows a lane group has in flight
+constexpr int kTauRows = 16;  // sample rows a lane group has in flight
 
 __device__ __forceinline__ float tau_block_reduce(float v, bool is_max, float* s_red) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -180,24 +180,38 @@ __global__ __launch_bounds__(kTauThreads) void k_threshold(
         head = tree_q_heads[pos];
     }
 
-    // ---- scores: 16 lanes per sample row, 64 rows per pass, kTauRows passes at a time --------
+    // ---- scores: 16 lanes per sample row, 64 rows per pass, kTauRows passes at a time ---------
+    // (buffer loads: the tree's sample behind one scalar descriptor, the pass in a scalar offset,
+    // one address register for all the rows a lane has in flight -- which is what lets sixteen of
+    // them fit.  The range check of a buffer load looks at the vector offset only, so the scalar
+    // one must stay inside the sample by itself: the last pass is moved back to end with the
+    // sample and scores some rows a second time; with fewer than 64 rows the vector offset alone
+    // says which lanes have none.)
     const int sub = tid & 15, grp = tid >> 4;
     const int chunks = D / EPL;
     const T* xs = samples + (size_t)tree * S * D;
     const T* qh = q + (size_t)head * D;
     constexpr int PASS = kTauThreads / 16;
+    const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<T*>(xs), 0, (int)((size_t)S * D * sizeof(T)), 0x00020000);
+    const int last_pass = max(S - PASS, 0);
     for (int r0 = 0; r0 < S; r0 += PASS * kTauRows) {  // uniform
         float dot[kTauRows];
-        int row[kTauRows];
 #pragma unroll
-        for (int u = 0; u < kTauRows; ++u) {
-            dot[u] = 0.0f;
-            row[u] = min(r0 + u * PASS + grp, S - 1);
-        }
+        for (int u = 0; u < kTauRows; ++u) dot[u] = 0.0f;
         for (int c = sub; c < chunks; c += 16) {
+            typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+            const unsigned voff = (unsigned)((grp * D + c * EPL) * (int)sizeof(T));
             uint4 raw[kTauRows];
 #pragma unroll
-            for (int u = 0; u < kTauRows; ++u) raw[u] = load_chunk<T>(xs, (size_t)row[u] * D, c);
+            for (int u = 0; u < kTauRows; ++u) {
+                raw[u] = make_uint4(0, 0, 0, 0);
+                if (r0 + u * PASS < S) {  // uniform
+                    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(
+                        xrsrc, voff, (unsigned)(min(r0 + u * PASS, last_pass) * D * (int)sizeof(T)), 0);
+                    raw[u] = make_uint4(v.x, v.y, v.z, v.w);
+                }
+            }
             float b[EPL];
             unpack<T>(load_chunk<T>(qh, 0, c), b);
 #pragma unroll
@@ -211,7 +225,8 @@ __global__ __launch_bounds__(kTauThreads) void k_threshold(
 #pragma unroll
         for (int u = 0; u < kTauRows; ++u) {
             const float d = group_sum<16>(dot[u]);
-            if (sub == 0 && r0 + u * PASS + grp < S) s_sc[0][r0 + u * PASS + grp] = d;
+            const int row = min(r0 + u * PASS, last_pass) + grp;
+            if (sub == 0 && r0 + u * PASS < S && row < S) s_sc[0][row] = d;
         }
     }
     __syncthreads();

@@ -20,6 +20,7 @@ CASES = [
     (4, 513, 16, 16, torch.bfloat16, 100),    # just past a power of two
     (2, 1024, 64, 4, torch.float32, 16),      # the most that the few-of-many path takes
     (2, 65, 32, 8, torch.bfloat16, 7),        # a second wave holding a single score
+    (1, 1500, 128, 4, torch.bfloat16, 12),    # two registers per sorting thread, ragged last pass
 ]
 
 
