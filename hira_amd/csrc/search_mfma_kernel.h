@@ -1289,7 +1289,18 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 const int nc = s_nc[g];
                 const int* cl = clist + g * P;
                 const float* cw = cwt + g * P;
-                for (int k = 0; k < nc; k += 8) {  // uniform over the columns of a head
+                int k = 0;
+                for (; k + 8 < nc; k += 16) {  // uniform over the columns of a head (32 in flight: slower)
+                    float v[16];
+#pragma unroll
+                    for (int u = 0; u < 16; ++u) v[u] = ld(pa + (size_t)cl[min(k + u, nc - 1)] * D);
+#pragma unroll
+                    for (int u = 0; u < 16; u += 2) {
+                        s0 += (k + u < nc ? cw[k + u] : 0.0f) * v[u];
+                        s1 += (k + u + 1 < nc ? cw[k + u + 1] : 0.0f) * v[u + 1];
+                    }
+                }
+                for (; k < nc; k += 8) {  // (at most eight are left)
                     float v[8];
 #pragma unroll
                     for (int u = 0; u < 8; ++u) v[u] = ld(pa + (size_t)cl[min(k + u, nc - 1)] * D);
