@@ -107,9 +107,13 @@ static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* que
                        "block_threads %d must be a multiple of 64 up to %d", threads, kMfmaThreads);
         plan->threads = threads;
         // a workgroup walks `tpw` tiles of 16 level-1 nodes (a stride apart): as few as keep
-        // one workgroup per CU in the launch (the kernel runs one at a time on a CU) and at
-        // most 64 partials per head to fold
+        // one workgroup per CU in the launch (the kernel runs one at a time on a CU) and no
+        // more partials per head than the fold can list in LDS, 128 at most: a tree alone on
+        // the chip is scanned by up to 128 workgroups (131072 keys: 20.5 us; with 64 workgroups
+        // of four tiles 23.9 us, with 256 of one tile 24.1 us)
         const int tiles = (t->size[1] + 15) / 16;
+        int max_parts = 16 * t->dim / plan->gmax;
+        max_parts = max_parts < 64 ? 64 : (max_parts > 128 ? 128 : max_parts);
         int tpw = launch ? launch->nodes_per_wave : 0;
         HIRA_CHECK_ARG(tpw >= 0 && tpw <= kMfmaMaxTilesPerWg,
                        "MFMA kernel: %d tiles per workgroup (at most %d)", tpw, kMfmaMaxTilesPerWg);
@@ -117,7 +121,7 @@ static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* que
             const int64_t all = (int64_t)tiles * t->num_trees * plan->head_chunks;
             const int cus = compute_units();
             tpw = (int)((all + cus - 1) / cus);
-            if (tpw * 64 < tiles) tpw = (tiles + 63) / 64;
+            if (tpw * max_parts < tiles) tpw = (tiles + max_parts - 1) / max_parts;
             if (tpw < 1) tpw = 1;
             // more work than one workgroup per CU can take: several rounds of workgroups of 8 to 16
             // tiles, of the size whose rounds add up to the least (a workgroup costs some two
@@ -154,7 +158,7 @@ static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* que
             // few nodes since the last rebuild looks like: 24.6 -> 21 us per step)
             const int64_t per_tree = compute_units() / ((int64_t)t->num_trees * plan->head_chunks);
             int64_t blocks = per_tree < tiles ? per_tree : tiles;
-            if (blocks > 64) blocks = 64;
+            if (blocks > max_parts) blocks = max_parts;
             if (blocks > plan->tree_blocks) plan->tree_blocks = (int)blocks;
         }
         plan->queue_blocks = plan->num_queue_blocks > 0 ? 1 : 0;  // one workgroup takes the whole queue
