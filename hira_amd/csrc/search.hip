@@ -37,8 +37,9 @@ static int compute_units() {
     return cus;
 }
 
+// attn: the launch writes attention partials (the plan then also weighs what folding them costs)
 static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* queue,
-                     const HiraLaunch* launch, SearchPlan* plan) {
+                     const HiraLaunch* launch, bool attn, SearchPlan* plan) {
     HIRA_CHECK_ARG(t && q, "tree and query must not be NULL");
     HIRA_CHECK_ARG(t->dtype == HIRA_F32 || t->dtype == HIRA_BF16, "dtype %d", t->dtype);
     const int esize = t->dtype == HIRA_F32 ? 4 : 2;
@@ -185,9 +186,20 @@ static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* que
     }
     int npw = launch && launch->nodes_per_wave ? launch->nodes_per_wave : rpw * plan->gate_steps;
     HIRA_CHECK_ARG(npw >= 1, "nodes_per_wave %d", npw);
-    plan->nodes_per_wave = npw;
     plan->num_nodes = t->num_levels >= 2 ? t->size[1]
                                          : (t->size[0] + kPseudoBlock - 1) / kPseudoBlock;
+    // large trees under attention: a wave takes more steps of nodes, towards 64 partials a head to
+    // fold, as long as the launch keeps two workgroups per compute unit (8 trees x 65536 fp32
+    // keys, fan-out 32, 4 heads a tree: 256 partials 127 us, 128: 103, 64: 94, 32: 158; one such
+    // tree alone: 256 partials 47 us, 128: 55, 64: 82)
+    if (attn && !(launch && launch->nodes_per_wave) && plan->gate_steps == 1) {
+        const int wpb = threads / 64;
+        auto parts = [&](int n) { return (plan->num_nodes + wpb * n - 1) / (wpb * n); };
+        while (parts(npw) > 64 &&
+               (int64_t)t->num_trees * plan->head_chunks * parts(2 * npw) >= 2 * compute_units())
+            npw *= 2;
+    }
+    plan->nodes_per_wave = npw;
     const int per_block = (threads / 64) * npw;
     plan->tree_blocks = (plan->num_nodes + per_block - 1) / per_block;
     plan->queue_blocks = (plan->num_queue_blocks + per_block - 1) / per_block;
@@ -221,7 +233,7 @@ extern "C" size_t hira_search_workspace_bytes(const HiraTree* tree, const HiraQu
                                               const HiraQueue* queue,
                                               const HiraLaunch* launch) {
     SearchPlan plan;
-    if (make_plan(tree, query, queue, launch, &plan) != HIRA_OK) return 0;
+    if (make_plan(tree, query, queue, launch, true, &plan) != HIRA_OK) return 0;
     const size_t P = (size_t)plan.tree_blocks + plan.queue_blocks;
     return workspace_need(query->num_q_heads, P, tree->vdim, tree->num_trees, plan.head_chunks);
 }
@@ -234,10 +246,10 @@ static int search_impl(const HiraTree* tree, const HiraQuery* query, const HiraQ
                        const HiraSearchOut* out, const HiraLaunch* launch, void* workspace,
                        size_t workspace_bytes, size_t fixed_counters, void* stream) {
     SearchPlan plan;
-    int rc = make_plan(tree, query, queue, launch, &plan);
-    if (rc != HIRA_OK) return rc;
     HIRA_CHECK_ARG(out != nullptr, "out is NULL");
     const bool attn = out->attn_out != nullptr;
+    int rc = make_plan(tree, query, queue, launch, attn, &plan);
+    if (rc != HIRA_OK) return rc;
     if (attn) {
         HIRA_CHECK_ARG(tree->values != nullptr && tree->vdim > 0,
                        "attention needs values in the tree");
