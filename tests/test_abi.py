@@ -81,3 +81,48 @@ def test_new_entry_points_validate_without_a_gpu():
     assert lib.hira_sparse_attention(ctypes.byref(t), ctypes.byref(q), one, one, one, 8, one, None) == -1
     t.vdim = 32
     assert lib.hira_sparse_attention(ctypes.byref(t), ctypes.byref(q), one, one, one, 0, one, None) == -1
+
+
+def _partials_per_head(num_trees, keys_per_tree, heads_per_tree, dim=128, bf=32, levels=3):
+    """Workgroups (= attention partials per head) the launch plan makes for a tiled bf16 index of
+    this shape, read off hira_search_workspace_bytes (host arithmetic only; the pointers in the
+    descriptors are never followed)."""
+    lib = _lib.lib()
+    t = _lib.HiraTree()
+    t.num_trees, t.num_levels, t.bf, t.dim, t.vdim = num_trees, levels, bf, dim, dim
+    t.dtype, t.layout = _lib.HIRA_BF16, _lib.HIRA_TILE16
+    n = keys_per_tree
+    sizes = [n]
+    for _ in range(1, levels):
+        sizes.append(-(-sizes[-1] // bf))
+    for l in range(levels - 2, -1, -1):  # the padded layout: every node owns bf slots below it
+        sizes[l] = sizes[l + 1] * bf
+    for l in range(levels):
+        t.size[l] = sizes[l]
+        t.cap[l] = -(-sizes[l] // 16) * 16
+    dummy = ctypes.c_void_p(4096)
+    t.keys = t.values = t.perm = dummy
+    for l in range(1, levels):
+        t.centers[l] = t.radii[l] = t.counts[l] = dummy
+    q = _lib.HiraQuery(num_trees * heads_per_tree, dummy, dummy, dummy, dummy, dummy,
+                       heads_per_tree, heads_per_tree)
+    need = lib.hira_search_workspace_bytes(ctypes.byref(t), ctypes.byref(q), None, None)
+    assert need > 0, lib.hira_last_error()
+    counters = -(-num_trees * 4 // 256) * 256
+    per_part = num_trees * heads_per_tree * (dim + 2) * 4
+    assert (need - counters) % per_part == 0
+    return (need - counters) // per_part
+
+
+def test_launch_plan_fills_the_compute_units():
+    """What the plan of the matrix-core kernel promises (256 compute units assumed where no GPU
+    is present): one workgroup per compute unit where the launch fits one round -- also when a
+    tree's tiles do not divide evenly, as in an index that grew since its last rebuild --, at
+    most 128 partials per head for a tree alone on the chip, workgroups of up to 16 tiles where
+    the launch takes several rounds."""
+    assert _partials_per_head(8, 32768, 4) == 32            # 64 tiles a tree, 8 trees
+    assert _partials_per_head(8, 32768 + 32 * 32, 4) == 32  # 66 tiles: 2 or 3 a workgroup, not 22 x 3
+    assert _partials_per_head(8, 131072, 8, levels=4) == 32
+    assert _partials_per_head(1, 131072, 4) == 128          # 256 tiles, one tree
+    assert _partials_per_head(1, 8192, 4) == 16             # fewer tiles than compute units
+    assert _partials_per_head(128, 32768, 4) == 4           # several rounds: 16 tiles a workgroup
