@@ -109,3 +109,37 @@ def test_build_and_growth_keep_the_tree_valid_at_full_size(gpu_device):
     idx.rebuild_subtree(3)
     assert idx.num_keys == w.n + 2088
     _check_tree_on_device(idx, torch.cat([kd[0], md[0]], dim=1))
+
+
+@pytest.mark.parametrize("n,heads", [(131072, 4), (200000, 8), (33000, 4)])
+def test_lone_tree_is_scanned_by_many_workgroups(n, heads, gpu_device):
+    """One tree alone on the chip: the launch plan gives it up to 128 workgroups (a head then has
+    up to 128 partials to fold) or, at 33000 keys, workgroups of unequal tile counts.  The sparse
+    output must equal softmax over exactly the k best keys (fp64 on the device, 2e-3 through the
+    bf16 storage), and every key selected must equal dense attention."""
+    from hira_amd.cache.threshold_finder import exact_topk
+    from hira_amd.indexer import HIPIndexer
+    from hira_amd.searcher import HIPSearcher
+
+    g = torch.Generator().manual_seed(n)
+    d = 128
+    K = torch.randn(1, 1, n, d, generator=g).bfloat16().cuda()
+    V = torch.randn(1, 1, n, d, generator=g).bfloat16().cuda()
+    q = torch.randn(heads, d, generator=g).bfloat16().cuda()
+    idx = HIPIndexer(3, 1, 32).build(K, V)
+    k = n // 200
+    tau = exact_topk(K[0], q, k)
+    sc = torch.full((heads,), d ** -0.5)
+    se = HIPSearcher()
+    out = se.search_attention(q, tau, idx, scaling=sc)
+    assert torch.equal(out, se.search_attention(q, tau, idx, scaling=sc))
+    s = (q.double() @ K[0, 0].double().T)                      # (heads, n)
+    top = s.topk(k, dim=-1)
+    w = torch.softmax(top.values * d ** -0.5, dim=-1)
+    ref = torch.einsum("hk,hkd->hd", w, V[0, 0].double()[top.indices])
+    err = ((out.double() - ref).abs().max(dim=1).values / ref.abs().max(dim=1).values).max()
+    assert float(err) <= 2e-3, float(err)
+    dense = se.search_attention(q, torch.full((heads,), -3.0e38), idx, scaling=sc)
+    refd = torch.softmax(s * d ** -0.5, dim=-1) @ V[0, 0].double()
+    err = ((dense.double() - refd).abs().max(dim=1).values / refd.abs().max(dim=1).values).max()
+    assert float(err) <= 2e-3, float(err)
