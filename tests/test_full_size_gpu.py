@@ -143,3 +143,31 @@ def test_lone_tree_is_scanned_by_many_workgroups(n, heads, gpu_device):
     refd = torch.softmax(s * d ** -0.5, dim=-1) @ V[0, 0].double()
     err = ((dense.double() - refd).abs().max(dim=1).values / refd.abs().max(dim=1).values).max()
     assert float(err) <= 2e-3, float(err)
+
+
+def test_large_fp32_trees_on_the_vector_kernel(gpu_device):
+    """fp32 keys (the vector-ALU kernel) at a size where a wavefront takes several steps of nodes
+    so that a head has fewer partials to fold: the sparse output equals softmax over exactly the k
+    best keys of every head (fp64 on the device, 1e-5)."""
+    from hira_amd.cache.threshold_finder import exact_topk
+    from hira_amd.indexer import HIPIndexer
+    from hira_amd.searcher import HIPSearcher
+
+    g = torch.Generator().manual_seed(5)
+    t, grp, n, d = 4, 2, 65536, 128
+    K = torch.randn(1, t, n, d, generator=g).cuda()
+    V = torch.randn(1, t, n, d, generator=g).cuda()
+    q = torch.randn(t * grp, d, generator=g).cuda()
+    idx = HIPIndexer(3, 1, 32).build(K, V)
+    k = 300
+    tau = exact_topk(K[0], q, k)
+    sc = torch.full((t * grp,), d ** -0.5)
+    out = HIPSearcher().search_attention(q, tau, idx, scaling=sc)
+    s = torch.einsum("tgd,tnd->tgn", q.view(t, grp, d).double(), K[0].double())
+    top = s.topk(k, dim=-1)
+    w = torch.softmax(top.values * d ** -0.5, dim=-1)
+    vsel = torch.gather(V[0].double()[:, None].expand(t, grp, n, d), 2,
+                        top.indices[..., None].expand(t, grp, k, d))
+    ref = torch.einsum("tgk,tgkd->tgd", w, vsel).reshape(t * grp, d)
+    err = ((out.double() - ref).abs().max(dim=1).values / ref.abs().max(dim=1).values).max()
+    assert float(err) <= 1e-5, float(err)
