@@ -323,18 +323,26 @@ __global__ void k_mark_absent(const int32_t* n_live, int n_c, int K, int bf, int
     if (i < K) fill[(size_t)t * K + i] = i >= max((n_t + bf - 1) / bf, 1) ? bf : 0;
 }
 
-__global__ void k_collect_unplaced(const int32_t* placed, int n_c, int32_t* list,
-                                   int32_t* list_count) {
+// (one atomic per workgroup of 256 items, not per wave: the tree's counter is one address)
+__global__ __launch_bounds__(256) void k_collect_unplaced(const int32_t* placed, int n_c,
+                                                          int32_t* list, int32_t* list_count) {
+    __shared__ int32_t s_cnt[4];
+    __shared__ int32_t s_base;
     const int t = blockIdx.y;
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     const bool mine = i < n_c && placed[(size_t)t * n_c + i] == 0;
     const unsigned long long bal = __ballot(mine);
-    if (bal == 0ull) return;
-    const int lane = lane_id();
-    int base = 0;
-    if (lane == __ffsll((long long)bal) - 1) base = atomicAdd(&list_count[t], __popcll(bal));
-    base = __shfl(base, __ffsll((long long)bal) - 1, 64);
-    if (mine) list[(size_t)t * n_c + base + __popcll(bal & ((1ull << lane) - 1ull))] = i;
+    const int lane = lane_id(), wave = threadIdx.x >> 6;
+    if (lane == 0) s_cnt[wave] = __popcll(bal);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int total = s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3];
+        s_base = total > 0 ? atomicAdd(&list_count[t], total) : 0;
+    }
+    __syncthreads();
+    int before = s_base;
+    for (int w = 0; w < wave; ++w) before += s_cnt[w];
+    if (mine) list[(size_t)t * n_c + before + __popcll(bal & ((1ull << lane) - 1ull))] = i;
 }
 
 // Whatever is still unplaced goes to the free slots in order: the u-th unplaced item (by
