@@ -208,21 +208,25 @@ __global__ void k_bucket_fill(const int32_t* assign, int n_c, const int32_t* lis
     members[(size_t)t * n_c + at] = i;
 }
 
-// one wave per bucket: rank every member by (dist, item id) and write it to its rank
+// one workgroup per bucket: rank every member by (dist, item id) and write it to its rank (four
+// waves: nearest-centroid buckets of seeds drawn from the keys are very uneven in 128 dimensions,
+// and a bucket of m members costs m * m / threads comparisons)
 constexpr int kSortTile = 1024;
-__global__ __launch_bounds__(64) void k_bucket_sort(const int32_t* members, const int32_t* offsets,
-                                                    const float* dist, int n_c, int K,
-                                                    int32_t* sorted) {
+constexpr int kSortThreads = 256;
+__global__ __launch_bounds__(kSortThreads) void k_bucket_sort(const int32_t* members,
+                                                              const int32_t* offsets,
+                                                              const float* dist, int n_c, int K,
+                                                              int32_t* sorted) {
     __shared__ uint64_t keys[kSortTile];
     const int k = blockIdx.x, t = blockIdx.y;
-    const int lane = threadIdx.x;
+    const int tid = threadIdx.x;
     const int b0 = offsets[(size_t)t * (K + 1) + k], b1 = offsets[(size_t)t * (K + 1) + k + 1];
     const int m = b1 - b0;
     if (m <= 0) return;
     const int32_t* mem = members + (size_t)t * n_c + b0;
     const float* dt = dist + (size_t)t * n_c;
-    for (int e0 = 0; e0 < m; e0 += 64) {
-        const int e = e0 + lane;
+    for (int e0 = 0; e0 < m; e0 += kSortThreads) {
+        const int e = e0 + tid;
         uint64_t mykey = 0;
         int myitem = -1;
         if (e < m) {
@@ -233,7 +237,7 @@ __global__ __launch_bounds__(64) void k_bucket_sort(const int32_t* members, cons
         for (int tile = 0; tile < m; tile += kSortTile) {
             const int tn = min(kSortTile, m - tile);
             __syncthreads();
-            for (int j = lane; j < tn; j += 64) {
+            for (int j = tid; j < tn; j += kSortThreads) {
                 const int it = mem[tile + j];
                 keys[j] = ((uint64_t)__float_as_uint(dt[it]) << 32) | (uint32_t)it;
             }
@@ -251,12 +255,16 @@ __global__ __launch_bounds__(64) void k_bucket_sort(const int32_t* members, cons
 //    An empty centroid keeps its value.  out_t != NULL: also store rounded to T.
 // ------------------------------------------------------------------------------------
 template <typename T>
-__global__ __launch_bounds__(64) void k_mean(const void* x, size_t x_tree_stride, int n_c, int K,
-                                             int D, const int32_t* offsets,
-                                             const int32_t* members, const int32_t* slots, int bf,
-                                             float* cent, void* out_t) {
+__global__ __launch_bounds__(256) void k_mean(const void* x, size_t x_tree_stride, int n_c, int K,
+                                              int D, const int32_t* offsets,
+                                              const int32_t* members, const int32_t* slots, int bf,
+                                              float* cent, void* out_t) {
+    // launched with one wave (the sums then run in list order) or four (wave w sums members
+    // w, w + 4, ..., the four sums are added in wave order: large buckets, still reproducible)
+    __shared__ float s_part[3][64];
+    __shared__ int s_cnt[3];
     const int k = blockIdx.x, t = blockIdx.y;
-    const int lane = threadIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     const int32_t* lst;
     int m;
     if (slots) {
@@ -271,13 +279,26 @@ __global__ __launch_bounds__(64) void k_mean(const void* x, size_t x_tree_stride
         const int j = j0 + lane;
         float s = 0.0f;
         int cnt = 0;
-        for (int e = 0; e < m; ++e) {
+        for (int e = wave; e < m; e += nw) {
             const int it = lst[e];
             if (it < 0) continue;
             ++cnt;
             if (j < D) s += load_elem<T>(x, ((size_t)t * x_tree_stride + it) * D + j);
         }
-        if (j < D) {
+        if (nw > 1) {  // uniform
+            __syncthreads();
+            if (wave > 0) {
+                s_part[wave - 1][lane] = s;
+                if (lane == 0) s_cnt[wave - 1] = cnt;
+            }
+            __syncthreads();
+            if (wave == 0)
+                for (int w = 1; w < nw; ++w) {
+                    s += s_part[w - 1][lane];
+                    cnt += s_cnt[w - 1];
+                }
+        }
+        if (wave == 0 && j < D) {
             const size_t o = ((size_t)t * K + k) * D + j;
             float v = cent[o];
             if (cnt > 0) {
@@ -671,9 +692,9 @@ static int build_impl(const HiraTree* t, const void* keys_in, const void* values
             hipLaunchKernelGGL(k_scan, dim3(NT), dim3(256), 0, s, w.counts, Kl, w.offsets, w.cursor);
             hipLaunchKernelGGL(k_bucket_fill, g_items, dim3(256), 0, s, w.assign, n_c, live,
                                live_cnt, live_stride, Kl, w.cursor, w.members);
-            hipLaunchKernelGGL(k_bucket_sort, g_cent, dim3(64), 0, s, w.members, w.offsets, w.dist,
+            hipLaunchKernelGGL(k_bucket_sort, g_cent, dim3(kSortThreads), 0, s, w.members, w.offsets, w.dist,
                                n_c, Kl, w.sorted);
-            hipLaunchKernelGGL((k_mean<T>), g_cent, dim3(64), 0, s, x, xs, n_c, Kl, D, w.offsets,
+            hipLaunchKernelGGL((k_mean<T>), g_cent, dim3(256), 0, s, x, xs, n_c, Kl, D, w.offsets,
                                w.sorted, nullptr, bf, w.cent_f32, nullptr);
         }
         // capacity packing
@@ -708,7 +729,7 @@ static int build_impl(const HiraTree* t, const void* keys_in, const void* values
             hipLaunchKernelGGL(k_scan, dim3(NT), dim3(256), 0, s, w.counts, Kl, w.offsets, w.cursor);
             hipLaunchKernelGGL(k_bucket_fill, g_items, dim3(256), 0, s, w.assign, n_c, list, lcnt,
                                (size_t)n_c, Kl, w.cursor, w.members);
-            hipLaunchKernelGGL(k_bucket_sort, g_cent, dim3(64), 0, s, w.members, w.offsets, w.dist,
+            hipLaunchKernelGGL(k_bucket_sort, g_cent, dim3(kSortThreads), 0, s, w.members, w.offsets, w.dist,
                                n_c, Kl, w.sorted);
             hipLaunchKernelGGL(k_accept, g_cent, dim3(64), 0, s, w.sorted, w.offsets, n_c, Kl, bf,
                                w.fill, w.slots[l], w.placed);
