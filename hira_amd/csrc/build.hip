@@ -368,17 +368,18 @@ __global__ __launch_bounds__(256) void k_collect_unplaced(const int32_t* placed,
 
 // Whatever is still unplaced goes to the free slots in order: the u-th unplaced item (by
 // item id) takes the u-th free slot (by block, then slot).  One workgroup per tree.
-__global__ __launch_bounds__(256) void k_leftover(int n_c, int K, int bf, int32_t* fill,
+constexpr int kLeftThreads = 1024;  // (the walk over a tree's items is serial in steps of this many)
+__global__ __launch_bounds__(kLeftThreads) void k_leftover(int n_c, int K, int bf, int32_t* fill,
                                                   int32_t* slots, int32_t* placed,
                                                   int32_t* scratch /* (T, K+1) */) {
-    __shared__ int32_t wsum[4];
+    __shared__ int32_t wsum[kLeftThreads / 64];
     __shared__ int32_t carry;
     const int t = blockIdx.x;
     const int lane = lane_id(), wave = threadIdx.x >> 6;
     int32_t* freepre = scratch + (size_t)t * (K + 1);  // exclusive prefix of free slots
     if (threadIdx.x == 0) carry = 0;
     __syncthreads();
-    for (int base = 0; base < K; base += 256) {
+    for (int base = 0; base < K; base += kLeftThreads) {
         const int k = base + threadIdx.x;
         const int v = k < K ? bf - fill[(size_t)t * K + k] : 0;
         int inc = v;
@@ -393,7 +394,7 @@ __global__ __launch_bounds__(256) void k_leftover(int n_c, int K, int bf, int32_
         for (int w = 0; w < wave; ++w) before += wsum[w];
         if (k < K) freepre[k] = before + inc - v;
         __syncthreads();
-        if (threadIdx.x == 255) carry = before + inc;
+        if (threadIdx.x == kLeftThreads - 1) carry = before + inc;
         __syncthreads();
     }
     if (threadIdx.x == 0) {
@@ -401,7 +402,7 @@ __global__ __launch_bounds__(256) void k_leftover(int n_c, int K, int bf, int32_
         carry = 0;
     }
     __syncthreads();
-    for (int base = 0; base < n_c; base += 256) {
+    for (int base = 0; base < n_c; base += kLeftThreads) {
         const int i = base + threadIdx.x;
         const int v = (i < n_c && placed[(size_t)t * n_c + i] == 0) ? 1 : 0;
         int inc = v;
@@ -427,12 +428,12 @@ __global__ __launch_bounds__(256) void k_leftover(int n_c, int K, int bf, int32_
             placed[(size_t)t * n_c + i] = 1;
         }
         __syncthreads();
-        if (threadIdx.x == 255) carry = before + inc;
+        if (threadIdx.x == kLeftThreads - 1) carry = before + inc;
         __syncthreads();
     }
     __syncthreads();
     // the blocks are now as full as the items allow
-    for (int k = threadIdx.x; k < K; k += 256) {
+    for (int k = threadIdx.x; k < K; k += kLeftThreads) {
         int c = 0;
         for (int j = 0; j < bf; ++j) c += slots[((size_t)t * K + k) * bf + j] >= 0;
         fill[(size_t)t * K + k] = c;
@@ -734,7 +735,7 @@ static int build_impl(const HiraTree* t, const void* keys_in, const void* values
             hipLaunchKernelGGL(k_accept, g_cent, dim3(64), 0, s, w.sorted, w.offsets, n_c, Kl, bf,
                                w.fill, w.slots[l], w.placed);
         }
-        hipLaunchKernelGGL(k_leftover, dim3(NT), dim3(256), 0, s, n_c, Kl, bf, w.fill, w.slots[l],
+        hipLaunchKernelGGL(k_leftover, dim3(NT), dim3(kLeftThreads), 0, s, n_c, Kl, bf, w.fill, w.slots[l],
                            w.placed, w.scratch);
         // block centre = mean of what is in the block, rounded to the storage type
         hipLaunchKernelGGL((k_mean<T>), g_cent, dim3(64), 0, s, x, xs, n_c, Kl, D, nullptr, nullptr,
