@@ -459,12 +459,31 @@ __global__ void k_compose_order(const int32_t* order_parent, int size_parent, in
     order_child[(size_t)t * size_parent * bf + i] = v;
 }
 
-// dst[t][s] = src[t][order[t][s]] (zero row for -1); one wave per 64/(D/...) rows: thread
-// per element.  perm_out != NULL: also writes perm.
+// dst[t][s] = src[t][order[t][s]] (zero row for -1), a thread per 16-byte chunk of a row (a chunk
+// is contiguous in either layout).  perm_out != NULL: also writes perm.
 template <typename T>
 __global__ void k_gather_rows(const void* src, size_t src_tree_stride, const int32_t* order,
                               int size, int D, void* dst, size_t dst_tree_stride, int dst_layout,
                               int32_t* perm_out, size_t perm_tree_stride) {
+    constexpr int EPL = Elem<T>::kPerChunk;
+    const int t = blockIdx.y;
+    const int chunks = D / EPL;
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)size * chunks) return;
+    const int s = (int)(i / chunks), c = (int)(i % chunks);
+    const int o = order[(size_t)t * size + s];
+    uint4 v = make_uint4(0, 0, 0, 0);
+    if (o >= 0) v = load_chunk<T>(src, ((size_t)t * src_tree_stride + o) * D, c);
+    T* out = reinterpret_cast<T*>(dst) + (size_t)t * dst_tree_stride * D +
+             elem_index(dst_layout, D, (size_t)s, c * EPL);
+    *reinterpret_cast<uint4*>(out) = v;
+    if (perm_out && c == 0) perm_out[(size_t)t * perm_tree_stride + s] = o;
+}
+
+// the same, a thread per element: value rows whose length is not a multiple of 16 bytes
+template <typename T>
+__global__ void k_gather_elems(const void* src, size_t src_tree_stride, const int32_t* order,
+                               int size, int D, void* dst, size_t dst_tree_stride) {
     const int t = blockIdx.y;
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= (size_t)size * D) return;
@@ -472,8 +491,7 @@ __global__ void k_gather_rows(const void* src, size_t src_tree_stride, const int
     const int o = order[(size_t)t * size + s];
     float v = 0.0f;
     if (o >= 0) v = load_elem<T>(src, ((size_t)t * src_tree_stride + o) * D + j);
-    store_elem<T>(dst, (size_t)t * dst_tree_stride * D + elem_index(dst_layout, D, (size_t)s, j), v);
-    if (perm_out && j == 0) perm_out[(size_t)t * perm_tree_stride + s] = o;
+    store_elem<T>(dst, ((size_t)t * dst_tree_stride + s) * D + j, v);
 }
 
 // counts[p] = children in use; radii[p] = max over them of (||child - centre|| + r_child),
@@ -759,18 +777,25 @@ static int build_impl(const HiraTree* t, const void* keys_in, const void* values
     }
     // gathers
     {
-        const size_t tot = (size_t)t->size[0] * D;
+        const size_t tot = (size_t)t->size[0] * (D / Elem<T>::kPerChunk);
         hipLaunchKernelGGL((k_gather_rows<T>), dim3((unsigned)((tot + 255) / 256), NT), dim3(256),
                            0, s, keys_in, (size_t)n, w.order[0], t->size[0], D, t->keys,
                            (size_t)t->cap[0], key_layout_of(t->layout), t->perm, (size_t)t->cap[0]);
         if (values_in && t->values) {
-            const size_t totv = (size_t)t->size[0] * t->vdim;
-            hipLaunchKernelGGL((k_gather_rows<T>), dim3((unsigned)((totv + 255) / 256), NT),
-                               dim3(256), 0, s, values_in, (size_t)n, w.order[0], t->size[0],
-                               t->vdim, t->values, (size_t)t->cap[0], (int)HIRA_ROW_MAJOR, nullptr, (size_t)0);
+            if (t->vdim % Elem<T>::kPerChunk == 0) {
+                const size_t totv = (size_t)t->size[0] * (t->vdim / Elem<T>::kPerChunk);
+                hipLaunchKernelGGL((k_gather_rows<T>), dim3((unsigned)((totv + 255) / 256), NT),
+                                   dim3(256), 0, s, values_in, (size_t)n, w.order[0], t->size[0],
+                                   t->vdim, t->values, (size_t)t->cap[0], (int)HIRA_ROW_MAJOR, nullptr, (size_t)0);
+            } else {
+                const size_t totv = (size_t)t->size[0] * t->vdim;
+                hipLaunchKernelGGL((k_gather_elems<T>), dim3((unsigned)((totv + 255) / 256), NT),
+                                   dim3(256), 0, s, values_in, (size_t)n, w.order[0], t->size[0],
+                                   t->vdim, t->values, (size_t)t->cap[0]);
+            }
         }
         for (int l = 1; l < L; ++l) {
-            const size_t totc = (size_t)t->size[l] * D;
+            const size_t totc = (size_t)t->size[l] * (D / Elem<T>::kPerChunk);
             hipLaunchKernelGGL((k_gather_rows<T>), dim3((unsigned)((totc + 255) / 256), NT),
                                dim3(256), 0, s, w.cent_t[l], (size_t)K[l], w.order[l], t->size[l], D,
                                t->centers[l], (size_t)t->cap[l], center_layout_of(t->layout), nullptr, (size_t)0);

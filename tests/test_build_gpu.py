@@ -246,3 +246,25 @@ def test_build_of_trees_with_different_numbers_of_keys(dtype, d, bf, gpu_device)
     assert_same_selection(out != 0, s, th)
     with pytest.raises(ValueError):
         HIPIndexer(3, 1, bf).build(torch.from_numpy(keys)[None].to(dtype), key_counts=kc)
+
+
+@pytest.mark.parametrize("dtype,dv", [(torch.bfloat16, 8), (torch.float32, 12), (torch.bfloat16, 40)])
+def test_value_rows_of_any_width_follow_their_keys(dtype, dv, gpu_device):
+    """Value rows narrower and wider than the keys, of one to five 16-byte chunks: every slot
+    holds the value of the key it holds."""
+    from hira_amd.indexer.hip import HIPIndexer
+
+    t, n, d, bf = 2, 700, 64, 8
+    rnd = bf16_round if dtype == torch.bfloat16 else (lambda x: x)
+    keys = rnd(clustered_keys(t, n, d, seed=77, clusters=20))
+    vals = rnd(np.random.default_rng(dv).normal(size=(t, n, dv)).astype(np.float32))
+    idx = HIPIndexer(3, 1, bf).build(torch.from_numpy(keys)[None].to(dtype),
+                                     torch.from_numpy(vals)[None].to(dtype))
+    perm = idx.perm.cpu().numpy()
+    got_v = idx.values_buf[:, : idx.size[0]].float().cpu().numpy()
+    got_k = idx.keys_rowmajor()[:, : idx.size[0]].float().cpu().numpy()
+    for h in range(t):
+        ok = perm[h, : idx.size[0]] >= 0
+        assert ok.sum() == n
+        assert np.array_equal(got_v[h][ok], vals[h][perm[h, : idx.size[0]][ok]])
+        assert np.array_equal(got_k[h][ok], keys[h][perm[h, : idx.size[0]][ok]])
