@@ -5,6 +5,7 @@ the two loaders the reference leaves unimplemented (``from_dict`` / ``from_yaml`
 from __future__ import annotations
 
 import dataclasses
+import warnings
 from typing import Any, Dict
 
 
@@ -19,6 +20,9 @@ class DeviceMode:
 
 
 _THRESHOLD_METHODS = ("sample_max", "sample_mean_topk", "exact_topk", "none")
+# sections a configuration file may group its settings under
+_SECTIONS = {"indexing": ("num_levels", "max_iterations", "branching_factor"),
+             "thresholds": ("threshold_method", "sample_size", "threshold_topk")}
 
 
 @dataclasses.dataclass
@@ -50,13 +54,40 @@ class HiraConfig:
     # ------------------------------------------------------------------ loaders
     @classmethod
     def from_dict(cls, config_dict: Dict[str, Any]) -> "HiraConfig":
+        """Settings from a mapping: the field names flat, or grouped the way the reference's
+        sample file groups them (examples/configs/1_example_config.yml:1-8: the index's three
+        settings under ``indexing:``; likewise ``thresholds:``).  ``cuda_memory_limit`` (the
+        sample file's budget for the reference's unbuilt "cpu-cuda" mode, which nothing reads
+        there either) is accepted and ignored with a warning.  Any other unknown key, a key in
+        the wrong section or a key given twice is a ``ValueError``."""
         names = {f.name for f in dataclasses.fields(cls)}
-        extra = sorted(k for k in config_dict if k not in names and k != "chunk_size")
-        if extra:
-            raise ValueError(f"unknown HiraConfig keys: {extra}")
-        cfg = cls(**{k: config_dict[k] for k in config_dict if k in names})
-        if "chunk_size" in config_dict:
-            cfg.chunk_size = int(config_dict["chunk_size"])
+        flat: Dict[str, Any] = {}
+
+        def take(key, value, where):
+            if key not in names and key != "chunk_size":
+                raise ValueError(f"unknown HiraConfig key {where}{key!r}")
+            if key in flat:
+                raise ValueError(f"HiraConfig key {key!r} is given twice")
+            flat[key] = value
+
+        for key, value in config_dict.items():
+            if key in _SECTIONS:
+                if not isinstance(value, dict):
+                    raise ValueError(f"section {key!r} must be a mapping, got {type(value).__name__}")
+                for sub, sub_value in value.items():
+                    if sub not in _SECTIONS[key]:
+                        raise ValueError(f"{sub!r} is not a setting of section {key!r} "
+                                         f"(which holds {_SECTIONS[key]})")
+                    take(sub, sub_value, f"{key}.")
+            elif key == "cuda_memory_limit":
+                warnings.warn("HiraConfig: 'cuda_memory_limit' only concerns a mixed host/GPU "
+                              "mode that does not exist here; ignored", stacklevel=2)
+            else:
+                take(key, value, "")
+        chunk_size = flat.pop("chunk_size", None)
+        cfg = cls(**flat)
+        if chunk_size is not None:
+            cfg.chunk_size = int(chunk_size)
         return cfg
 
     @classmethod

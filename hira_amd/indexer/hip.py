@@ -920,3 +920,7 @@ class HIPIndexer(BaseIndexer):
         self._tree_struct = None
         self.quantize(s0, nsub)
         return self
+
+
+# the class name the reference's indexer/cuda.py defines (PyTorch-ROCm calls the device "cuda")
+CUDAIndexer = HIPIndexer

@@ -469,3 +469,7 @@ class StreamingStep:
         self.indexer.note_unsynced(1)
         self.left -= 1
         return self.out
+
+
+# the class name the reference's searcher/cuda.py defines (PyTorch-ROCm calls the device "cuda")
+CUDASearcher = HIPSearcher

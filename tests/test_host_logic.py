@@ -101,11 +101,73 @@ def test_config_kwargs_and_loaders(tmp_path):
     d = hira_config.HiraConfig.from_dict({"num_levels": 4, "update_every": 64})
     assert d.num_levels == 4 and d.update_every == 64 and d.branching_factor == 10
     with pytest.raises(ValueError):
-        hira_config.HiraConfig.from_dict({"cuda_memory_limit": 1})
+        hira_config.HiraConfig.from_dict({"no_such_setting": 1})
     p = tmp_path / "c.yml"
     p.write_text("device_mode: cuda_only\nnum_levels: 3\nbranching_factor: 16\n")
     y = hira_config.HiraConfig.from_yaml(str(p))
     assert (y.device_mode, y.num_levels, y.branching_factor) == ("cuda_only", 3, 16)
+
+
+def test_config_file_in_the_layout_of_the_reference_sample(tmp_path):
+    """The one configuration file the reference ships (examples/configs/1_example_config.yml:1-8)
+    groups the index's settings under ``indexing:`` and carries a ``cuda_memory_limit`` nothing
+    reads; a file of that structure must load."""
+    p = tmp_path / "sample.yml"
+    p.write_text('device_mode: "cuda_only" # "cpu_only" or "cuda_only" or "cpu-cuda"\n\n'
+                 'cuda_memory_limit: 4096  # MB\n\n'
+                 'indexing:\n  num_levels: 3\n  max_iterations: 2 # k-means\n'
+                 '  branching_factor: 32\n')
+    with pytest.warns(UserWarning, match="cuda_memory_limit"):
+        cfg = hira_config.HiraConfig.from_yaml(str(p))
+    assert cfg.device_mode == "cuda_only"
+    assert cfg.get_indexer_kwargs() == {"num_levels": 3, "max_iterations": 2,
+                                        "branching_factor": 32}
+    assert cfg.update_every == 1 and cfg.sample_size == 1000      # untouched defaults
+    both = hira_config.HiraConfig.from_dict(
+        {"update_every": 64, "indexing": {"num_levels": 4},
+         "thresholds": {"threshold_method": "sample_max", "sample_size": 256}})
+    assert (both.update_every, both.num_levels, both.threshold_method, both.sample_size) == \
+        (64, 4, "sample_max", 256)
+    for bad in ({"indexing": {"update_every": 2}},            # a setting in the wrong section
+                {"indexing": {"num_level": 3}},               # a misspelt one
+                {"indexing": 3},                              # a section that is no mapping
+                {"num_levels": 3, "indexing": {"num_levels": 4}}):   # given twice
+        with pytest.raises(ValueError):
+            hira_config.HiraConfig.from_dict(bad)
+
+
+def test_reference_import_paths_resolve_to_this_package():
+    """The reference installs as ``hira`` (setup.py:14-15) and its modules import each other as
+    ``hira.indexer``, ``hira.searcher``, ``hira.cache.*`` (cache/hira_cache.py:7-10,
+    tests/test_hira_cache.py:17-19): the same paths give this package's modules, the very
+    objects, so a patch through one name is seen through the other."""
+    import importlib
+
+    import hira
+    import hira.indexer
+    import hira.searcher
+    import hira.cache.hira_cache as by_old_name
+    import hira_amd.cache.hira_cache as by_new_name
+    import hira_amd.indexer
+    from hira.attention.hira_attention import hira_attention_forward
+    from hira.cache.hira_cache import CacheOutput, HiraCache, HiraCacheLayer  # noqa: F401
+    from hira.cache.hira_config import DeviceMode, HiraConfig
+    from hira.cache.threshold_finder import THRESHOLD_METHODS
+    from hira.indexer import BaseIndexer, CUDAIndexer
+    from hira.indexer.cuda import CUDAIndexer as from_cuda_module
+    from hira.searcher import BaseSearcher, CUDASearcher
+    from hira.searcher.cuda import CUDASearcher as searcher_from_cuda_module
+
+    assert hira.indexer is hira_amd.indexer and by_old_name is by_new_name
+    assert CUDAIndexer is from_cuda_module is HIPIndexer and issubclass(CUDAIndexer, BaseIndexer)
+    assert CUDASearcher is searcher_from_cuda_module is HIPSearcher
+    assert issubclass(CUDASearcher, BaseSearcher)
+    assert HiraConfig is hira_config.HiraConfig and DeviceMode.CUDA_ONLY == "cuda_only"
+    assert THRESHOLD_METHODS is threshold_finder.THRESHOLD_METHODS
+    assert callable(hira_attention_forward)
+    assert by_new_name.__spec__.name == "hira_amd.cache.hira_cache"   # its own spec is kept
+    with pytest.raises(ModuleNotFoundError):
+        importlib.import_module("hira.no_such_module")
 
 
 def test_threshold_rules():
