@@ -316,6 +316,77 @@ def streaming(a, w, index, plan, q_d, taus, out, dev):
     return res
 
 
+# columns of a workgroup's row of time stamps (hira_amd/csrc/search_mfma_timeline.h)
+TL_STAMPS = ["start", "arguments in registers", "gate operands asked for", "wave 0 gated",
+             "barrier behind the gates", "first key tiles asked for", "wave 0: first products done",
+             "wave 0: first round listed", "wave 0: first round gathered", "wave 0 at the merge",
+             "all waves at the merge", "partial on its way", "partial arrived", "ticket drawn",
+             "fold: partials listed", "fold: output written"]
+TL_ROWS, TL_ROUNDS, TL_XCC, TL_LOCAL = 16, 17, 18, 19
+TL_WAVE_END, TL_WAVE_ROWS, TL_WAVE_SCANNED, TL_WAVE_ISSUED, TL_WAVE_CONSUMED, TL_COLS = 24, 32, 40, 48, 56, 64
+
+
+def timeline_report(a, w, index, searcher, q_d, taus, outs, W, total, scale):
+    """Steps on the library built with time stamps: per phase, when the workgroups of a step
+    reach it (microseconds after the step's first workgroup started; mean over the steps of the
+    minimum / mean / maximum over the workgroups), and the differences between consecutive
+    phases on the path of the workgroup that finishes last (the one that folds last)."""
+    import numpy as np
+    import torch
+
+    dev = q_d.device
+    h_all = w.batch * w.h_q
+    # a row per workgroup: a tree is walked by at most 128 workgroups plus one for a queue, per
+    # pass of 16 heads
+    passes = (-(-h_all // index.num_trees) + 15) // 16
+    nwg = index.num_trees * 129 * max(passes, 1)
+    tl = torch.zeros((nwg, TL_COLS), dtype=torch.int64, device=dev)
+    plan = searcher.plan_attention(index, h_all, scaling=torch.full((h_all,), scale), stats=tl)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+    per_step, lens, wave_rows, wave_end, crit = [], [], [], [], []
+    for i in range(W, total):
+        tl.zero_()
+        torch.cuda.synchronize()
+        ev[0].record()
+        plan.run(q_d[i], taus[i], outs[i])
+        ev[1].record()
+        torch.cuda.synchronize()
+        t = tl.cpu().numpy()
+        t = t[t[:, 0] != 0]
+        t0 = t[:, 0].min()
+        r = (t[:, :16] - t0) / 100.0  # the clock runs at 100 MHz
+        r[t[:, :16] == 0] = np.nan
+        per_step.append(np.stack([np.nanmin(r, 0), np.nanmean(r, 0), np.nanmax(r, 0)]))
+        lens.append(ev[0].elapsed_time(ev[1]) * 1e3)
+        we = (t[:, TL_WAVE_END:TL_WAVE_END + 8] - t0) / 100.0
+        ok = t[:, TL_WAVE_END:TL_WAVE_END + 8] != 0
+        wave_end.append(we[ok])
+        wave_rows.append(t[:, TL_WAVE_ROWS:TL_WAVE_ROWS + 8][ok])
+        # the workgroup whose fold ends last: its own stamps, phase by phase
+        last = np.nanargmax(np.where(np.isnan(r[:, 15]), -1.0, r[:, 15]))
+        crit.append(r[last])
+    m = np.nanmean(np.stack(per_step), 0)
+    c = np.nanmean(np.stack(crit), 0)
+    print(f"# where a decode step goes: {w.name}, {total - W} steps, library with time stamps")
+    print(f"# step between HIP events (eager launch, stamps on): mean {np.mean(lens):.2f} us")
+    print("# microseconds after the first workgroup's start; min / mean / max over the "
+          "workgroups, mean over the steps; last column: the workgroup that folds last")
+    print(f"{'phase':34s} {'min':>7s} {'mean':>7s} {'max':>7s} {'last folder':>12s} {'its step':>9s}")
+    prev = 0.0
+    for k, name in enumerate(TL_STAMPS):
+        step = c[k] - prev if not np.isnan(c[k]) else float('nan')
+        print(f"{name:34s} {m[0, k]:7.2f} {m[1, k]:7.2f} {m[2, k]:7.2f} {c[k]:12.2f} {step:9.2f}")
+        if not np.isnan(c[k]):
+            prev = c[k]
+    we, wr = np.concatenate(wave_end), np.concatenate(wave_rows)
+    print("# waves by the rows they listed: count per step, when they arrive at the merge (mean, max)")
+    for lo, hi in ((0, 1), (1, 9), (9, 17), (17, 33), (33, 65), (65, 1 << 30)):
+        sel = (wr >= lo) & (wr < hi)
+        if sel.any():
+            print(f"rows {lo:3d}..{min(hi - 1, 9999):4d}: {sel.sum() / len(lens):8.1f} waves  "
+                  f"mean {we[sel].mean():6.2f}  max {we[sel].max():6.2f}")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -327,9 +398,6 @@ def main():
     ap.add_argument("--block-threads", type=int, default=0)
     ap.add_argument("--nodes-per-wave", type=int, default=0)
     ap.add_argument("--kernel", type=int, default=0)
-    ap.add_argument("--share", type=int, default=0,
-                    help="MFMA kernel: workgroups that gate the same tiles and split the survivors "
-                         "(0 = chosen by the library, 1 = no sharing)")
     ap.add_argument("--kmeans-iters", type=int, default=-1)
     ap.add_argument("--layout", default="auto", choices=["auto", "tiled", "q8", "row_major"],
                     help="index layout (q8: an 8-bit shadow of the keys is scanned first)")
@@ -352,6 +420,13 @@ def main():
     ap.add_argument("--npz", default=None,
                     help="keys and queries captured from a model (the reference sampler's .npz: "
                          "keys (N,D), queries (N,D)) instead of the synthetic ones")
+    ap.add_argument("--taus", default=None,
+                    help="file that keeps the steps' thresholds: written when absent, read when "
+                         "present (so that a run under a profiler's counters need not launch "
+                         "the sort kernels that find them)")
+    ap.add_argument("--timeline", action="store_true",
+                    help="run the steps on the library built with time stamps "
+                         "(`make -C hira_amd/csrc timeline`) and print where a step's time goes")
     ap.add_argument("--counters", action="store_true",
                     help="run the steps once, untimed, plus a kernel of known traffic "
                          "(for rocprofv3 --pmc runs)")
@@ -372,6 +447,8 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     dev = torch.device("cuda:0")
+    if a.timeline:
+        _lib.use_library(_lib.CSRC / "libhira_hip_timeline.so")
     w = synth.WORKLOADS[a.config]
     if a.context > 0:
         import dataclasses
@@ -404,13 +481,24 @@ def main():
     q_d = queries.to(dev).reshape(total, w.batch * w.h_q, w.d).contiguous()
     taus = torch.empty((total, w.batch * w.h_q), dtype=torch.float32, device=dev)
     ksel = [int(np.ceil(float(fr[b]) * w.n)) for b in range(w.batch)]
-    for b in range(w.batch):
-        hs = slice(b * w.h_q, (b + 1) * w.h_q)
-        for i in range(total):
-            taus[i, hs] = exact_topk(keys_d[b], q_d[i, hs], ksel[b])
+    if a.taus and os.path.exists(a.taus):
+        kept = torch.load(a.taus, weights_only=True)
+        if tuple(kept.shape) != tuple(taus.shape):
+            raise SystemExit(f"{a.taus} holds thresholds of shape {tuple(kept.shape)}, this run "
+                             f"needs {tuple(taus.shape)}: made with other --steps/--warmup/--config?")
+        taus.copy_(kept)
+        log(f"[bench] thresholds read from {a.taus}")
+    else:
+        for b in range(w.batch):
+            hs = slice(b * w.h_q, (b + 1) * w.h_q)
+            for i in range(total):
+                taus[i, hs] = exact_topk(keys_d[b], q_d[i, hs], ksel[b])
+        if a.taus:
+            torch.save(taus.cpu(), a.taus)
+            log(f"[bench] thresholds written to {a.taus}")
     scale = w.d ** -0.5
     searcher = HIPSearcher(block_threads=a.block_threads, nodes_per_wave=a.nodes_per_wave,
-                           kernel=a.kernel, separate_merge=a.separate_merge, share=a.share)
+                           kernel=a.kernel, separate_merge=a.separate_merge)
     h_all = w.batch * w.h_q
     plan = searcher.plan_attention(index, h_all, scaling=torch.full((h_all,), scale))
     outs = torch.empty((total, h_all, w.d), dtype=torch.float32, device=dev)
@@ -419,6 +507,10 @@ def main():
     for i in range(W):
         plan.run(q_d[i], taus[i], outs[i])
     torch.cuda.synchronize()
+
+    if a.timeline:
+        timeline_report(a, w, index, searcher, q_d, taus, outs, W, total, scale)
+        return
 
     if a.counters:
         # For `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`: K plain launches of the

@@ -17,7 +17,7 @@ HIRA_MAX_LEVELS = 8
 HIRA_STATS_COLS = HIRA_MAX_LEVELS + 3  # counters per tree a search can fill in
 HIRA_F32, HIRA_BF16 = 0, 1
 HIRA_ROW_MAJOR, HIRA_TILE16, HIRA_TILE16_Q8 = 0, 1, 2
-HIRA_ABI_VERSION = 4
+HIRA_ABI_VERSION = 5
 
 _vp = C.c_void_p
 
@@ -83,7 +83,6 @@ class HiraLaunch(C.Structure):
         ("nodes_per_wave", C.c_int32),
         ("kernel", C.c_int32),
         ("separate_merge", C.c_int32),
-        ("share", C.c_int32),
     ]
 
 
@@ -145,6 +144,16 @@ def build_library(verbose: bool = False) -> None:
         print(r.stdout[-4000:], r.stderr[-4000:])
     if r.returncode != 0:
         raise RuntimeError("building libhira_hip.so failed")
+
+
+def use_library(path) -> None:
+    """Load another build of the library than the default one (the build with time stamps that
+    `make -C hira_amd/csrc timeline` makes, for looking at a decode step): call before anything
+    else has used the library."""
+    global LIB_PATH
+    if _lib is not None:
+        raise RuntimeError("the library is already loaded")
+    LIB_PATH = Path(path).resolve()
 
 
 def lib() -> C.CDLL:

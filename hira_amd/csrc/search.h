@@ -38,8 +38,6 @@ struct SearchParams {
     // work split
     int32_t nodes_per_wave;  // level-1 nodes (or pseudo blocks) per wave; MFMA kernel: tiles per workgroup
     int32_t tree_blocks;     // workgroups that walk the tree; the rest scan the queue
-    int32_t share;           // MFMA kernel: workgroups that gate the same tiles and split what
-                             // survives (tree_blocks is a multiple of it)
     int32_t key_policy;      // MFMA kernel: which cache policy the scan's loads use (0: default,
                              // 1: key tiles non-temporal, 2: value rows too), by the launch's size
     int32_t num_nodes;       // level-1 nodes (or pseudo blocks over the keys when L == 1)
@@ -71,7 +69,6 @@ struct SearchPlan {
     int nodes_per_wave;
     int num_nodes, num_queue_blocks;
     int tree_blocks, queue_blocks, head_chunks;
-    int share;        // MFMA kernel: see SearchParams
     int gate_steps;   // vector-ALU kernel: steps of gates a wave batches (1 or 4)
     size_t smem;
 };

@@ -24,17 +24,19 @@ static int round_pow2(int v) {
     return r;
 }
 
-// compute units of the current device (asked once)
+// compute units of the current device (asked once per device: the launch plan depends on it)
 static int compute_units() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess ||
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+    constexpr int kMaxDev = 64;
+    static int cus[kMaxDev];  // 0: not asked yet (written once per entry, the same value from any thread)
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) return 256;
+    int n = __atomic_load_n(&cus[dev], __ATOMIC_RELAXED);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
             n = 256;
-        cus = n;
+        __atomic_store_n(&cus[dev], n, __ATOMIC_RELAXED);
     }
-    return cus;
+    return n;
 }
 
 // attn: the launch writes attention partials (the plan then also weighs what folding them costs)
@@ -137,21 +139,10 @@ static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* que
                 }
             }
         }
-        // groups of `share` workgroups may gate the same share*tpw tiles (at most 16: two a wave)
-        // and split the survivors evenly.  Off unless asked for: measured at the benchmark's
-        // shapes the spread between workgroups comes from the burst of key reads draining
-        // through the memory system, not from uneven node counts, and the longer gate costs
-        // more than the even deal gains.
-        int share = launch ? launch->share : 0;
-        HIRA_CHECK_ARG(share >= 0 && share * tpw <= kMfmaMaxTilesPerWg,
-                       "MFMA kernel: share %d x %d tiles per workgroup (at most %d tiles gated)",
-                       share, tpw, kMfmaMaxTilesPerWg);
-        if (share == 0) share = 1;
-        plan->share = share;
         plan->nodes_per_wave = tpw;
         plan->num_nodes = t->size[1];
-        plan->tree_blocks = (tiles + tpw * share - 1) / (tpw * share) * share;
-        if (!(launch && launch->nodes_per_wave) && share == 1) {
+        plan->tree_blocks = (tiles + tpw - 1) / tpw;
+        if (!(launch && launch->nodes_per_wave)) {
             // a launch that fits one round: as many workgroups a tree as there are compute units
             // for it, each with `tpw` tiles or one less (the tiles are dealt out a stride apart),
             // rather than fewer workgroups that all hold `tpw` (66 tiles a tree on 32 compute units
@@ -164,6 +155,10 @@ static int make_plan(const HiraTree* t, const HiraQuery* q, const HiraQueue* que
         }
         plan->queue_blocks = plan->num_queue_blocks > 0 ? 1 : 0;  // one workgroup takes the whole queue
         plan->smem = 0;
+        // every workgroup that walks the tree must own at least one tile: one without a tile
+        // leaves the kernel before it draws its ticket, and the fold would never run
+        if (plan->tree_blocks > tiles)
+            return fail(HIRA_EINVAL, "launch plan: %d workgroups for %d tiles", plan->tree_blocks, tiles);
         return HIRA_OK;
     }
     plan->gmax = q->max_group <= 1 ? 1 : (q->max_group <= 4 ? 4 : 8);
@@ -305,7 +300,6 @@ static int search_impl(const HiraTree* tree, const HiraQuery* query, const HiraQ
     }
     p.nodes_per_wave = plan.nodes_per_wave;
     p.tree_blocks = plan.tree_blocks;
-    p.share = plan.kernel == 2 ? plan.share : 1;
     {   // up to what the eight L2s hold together (32 MiB) the default policy; up to 512 MiB the
         // key tiles and the value rows non-temporal; beyond, the key tiles only
         const size_t key_bytes = (size_t)tree->num_trees * (size_t)tree->size[0] * (size_t)tree->dim * 2;

@@ -38,6 +38,7 @@
 #pragma once
 
 #include "search.h"
+#include "search_mfma_timeline.h"
 
 namespace hira {
 
@@ -278,38 +279,23 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     const int tree = blockIdx.x;
     const int L = p.num_levels, bf = p.bf;
     const bool want_attn = p.part_acc != nullptr;
-    // The tree's workgroups come in groups of `share`.  The workgroups of a group gate the same
-    // tiles -- grp, grp + (groups), ... : a stride apart, since neighbouring tiles hold sibling
-    // nodes, which tend to survive (and be selected from) together -- so each of them knows the
-    // group's whole ordered list of surviving nodes without a word exchanged, and member `rep`
-    // takes entries rep, rep + share, ... of it.  Gating a tile costs a wave one 16 x D read
-    // that the L2 serves; what it buys is that the keys to scan are dealt out evenly however
-    // unevenly the query's hits are spread over the tree.
+    // Workgroup y of a tree owns the tree's tiles y, y + (workgroups of the tree), ...: a stride
+    // apart, since neighbouring tiles hold sibling nodes, which tend to survive (and be selected
+    // from) together.
     const int wg_tiles = (p.size[1] + 15) >> 4;
-    const int share = p.share, n_groups = p.tree_blocks / share;
-    const int grp = (int)blockIdx.y % n_groups, rep = (int)blockIdx.y / n_groups;
+    const int n_groups = p.tree_blocks;
+    const int grp = (int)blockIdx.y;
     const int ntile = (int)blockIdx.y < p.tree_blocks
-                          ? min(p.nodes_per_wave * share, (wg_tiles - grp + n_groups - 1) / n_groups)
+                          ? min(p.nodes_per_wave, (wg_tiles - grp + n_groups - 1) / n_groups)
                           : 0;
     auto tile_of = [&](int tl) { return grp + tl * n_groups; };
     // level-1 node behind entry n (tile n / 16 of mine, node n % 16 of the tile)
     auto node_of = [&](int n) { return tile_of(n >> 4) * 16 + (n & 15); };
     const bool is_queue = (int)blockIdx.y >= p.tree_blocks;  // the workgroup after the tree's
-#ifdef HIRA_TIMELINE  // experiment builds only: p.stats receives 32 entries per workgroup: 16
-                      // time stamps of its first thread, then per wave the time its rounds
-                      // ended and the rows it listed
-    unsigned long long* stats = nullptr;
-    unsigned long long* tl =
-        p.stats + (((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 64;
-    unsigned long long tl_rows = 0;
-#define HIRA_TLW(k) do { if ((threadIdx.x & 63) == 0) tl[(k) + (threadIdx.x >> 6)] = wall_clock64(); } while (0)
-#define HIRA_TL(k) do { if (threadIdx.x == 0) tl[k] = wall_clock64(); } while (0)
-#else
-    unsigned long long* stats = p.stats ? p.stats + (size_t)tree * HIRA_STATS_COLS : nullptr;
-#define HIRA_TL(k) do { } while (0)
-#define HIRA_TLW(k) do { } while (0)
-#endif
-    HIRA_TL(0);
+    Timeline tline(p);  // (empty unless the library is built with time stamps)
+    unsigned long long* stats =
+        (p.stats && !Timeline::kOn) ? p.stats + (size_t)tree * HIRA_STATS_COLS : nullptr;
+    tline.stamp(kTlStart);
 
     // ---- heads of this pass ----------------------------------------------------------
     int hoff, G;
@@ -322,6 +308,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     }
     if (G <= 0 || (ntile <= 0 && !is_queue)) return;  // uniform
     G = min(G, GS);
+    tline.stamp(kTlArgs);
     const bool head_ok = col < G;
     int qh = 0;
     if (head_ok) qh = p.group_size > 0 ? hoff + col : p.tree_q_heads[hoff + col];
@@ -414,6 +401,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         const float sc = head_ok ? p.scaling[qh] : 0.0f;
         GateLoads<KS> gl;
         if (tl_mine < ntile) gate_issue<KS, Q8>(p, tree, tile_of(tl_mine), lane, kb, gl);
+        tline.stamp(kTlGateIssued);
         if constexpr (Q8) {
             // ---- the queries in steps of the shadow (the last wave, which has the fewest tiles to
             // gate, for all): lane (kb, head) takes
@@ -510,7 +498,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         // ---- gate: one tile per wave at a time ------------------------------------------------
         while (tl_mine < ntile) {  // uniform in the wave
             const int t1 = tile_of(tl_mine);
-            const bool count_nodes = stats != nullptr && lane == 0 && rep == 0;  // once per group
+            const bool count_nodes = stats != nullptr && lane == 0;
             size_t span = 1;  // level-1 nodes under one node of the current level
             for (int l = 2; l < L; ++l) span *= (size_t)bf;
             int lcur = L - 1;
@@ -587,12 +575,11 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
             tl_mine += nw;
             if (tl_mine < ntile) gate_issue<KS, Q8>(p, tree, tile_of(tl_mine), lane, kb, gl);
         }
-        HIRA_TL(7);
+        tline.stamp(kTlGated);
         __syncthreads();
-        HIRA_TL(1);
+        tline.stamp(kTlBarrier);
 
-        // ---- the surviving nodes of the group's tiles in order; mine are entries rep, rep +
-        // share, ... of them, dealt round-robin to the waves ----------------------------------------
+        // ---- the surviving nodes of my tiles in order, dealt round-robin to the waves ----------
         int rounds, alive = 0;
         {
             const int n_info = ntile * 16;
@@ -617,8 +604,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 alive += __popcll(all);
             }
             alive *= HV;
-            const int mine = alive > rep ? (alive - rep + share - 1) / share : 0;
-            rounds = ((mine + nw - 1) / nw + NB - 1) / NB;
+            rounds = ((alive + nw - 1) / nw + NB - 1) / NB;
         }
 
         const float sc2 = sc * kLog2e;
@@ -650,13 +636,12 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         float nx_eps[Q8 ? NB : 1];
         uint4 a[NB][MT][KA];
         auto fetch = [&](int round, int u_only) {  // u_only < 0: all NB nodes of the round
-            // my nodes of the round: entries ((round*NB + u) * nw + wave) * share + rep of the
-            // group's survivors
+            // my nodes of the round: entries (round*NB + u) * nw + wave of the survivors
             uint32_t ent[NB];
 #pragma unroll
             for (int u = 0; u < NB; ++u) {
                 if (u_only >= 0 && u != u_only) continue;
-                const int k = ((round * NB + u) * nw + wave) * share + rep;
+                const int k = (round * NB + u) * nw + wave;
                 ent[u] = k < alive ? s_order[wave][k] : 0xFFu;
             }
 #pragma unroll
@@ -687,6 +672,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
             }
         };
         if (rounds > 0) fetch(0, -1);
+        tline.stamp(kTlFetched);
 
         constexpr int KB0 = KS <= 4 ? 2 : 1;      // batches of 16 key rows asked for ahead
         constexpr int RP = 64 / GS;               // rows whose weights one pass over the lanes computes
@@ -701,7 +687,6 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
             // ---- scan: the key tiles of this round's nodes were asked for a round ago; node by
             // node: the products, at once the request for the node that takes its place in the
             // next round, then the node's bookkeeping while the other tiles arrive -------------------
-            if (r == 0) HIRA_TL(8);
             // The bookkeeping below derives everything per-lane from this copy, which the compiler
             // cannot see through: otherwise it computes those values once, ahead of the loop, and
             // they crowd out the registers that the loads above need.
@@ -829,6 +814,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
 #pragma unroll
                 for (int tt = 0; tt < MT; ++tt)  // (only read where it is written: under this condition)
                     if (tt * 16 < cnt[u]) sco_u[tt] = tile_scores_lds<KS>(a[u][tt], s_bq, lane);
+                if (r == 0 && u == 0) tline.stamp(kTlTiles);
                 if (r + 1 < rounds) fetch(r + 1, u);
                 // a head for which the node did not survive selects nothing
                 const float tau_u = ((nmask[u] >> col) & 1u) ? tau : INFINITY;
@@ -876,9 +862,14 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 }
                 }  // shadow or bf16 tiles
             }
-            if (r == 0) HIRA_TLW(32);
             const int tot = nsel;  // rows on my list
-            if (r == 0) HIRA_TL(10);
+            if (r == 0) {
+                tline.stamp_wave(kTlWaveScanned);
+                tline.stamp(kTlListed);
+                tline.set(kTlRows, (unsigned long long)tot);
+                tline.set(kTlRounds, (unsigned long long)rounds);
+            }
+            tline.add_rows(tot);
 
             // ---- value rows: kVBatch in flight; the rows of a batch in the score table (lane =
             // (row of the pass, head)), their key slots, and the loads ---------------------------------
@@ -1015,10 +1006,6 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                     }
                 }
             };
-#ifdef HIRA_TIMELINE
-            if (threadIdx.x == 0 && r == 0) { tl[6] = (unsigned long long)tot; tl[12] = (unsigned long long)rounds; }
-            tl_rows += (unsigned long long)tot;
-#endif
             if constexpr (Q8) {
                 // The listed rows go kVBatch at a time: the value rows of the batch (most rows that
                 // the shadow lets through are selected) and their key rows are asked for together,
@@ -1054,13 +1041,12 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                         rows16(e0, at, slot, kr);
                         exact16(at, slot, kr);
                     }
-                    if (r == 0) HIRA_TL(9);
-                    if (r == 0) HIRA_TLW(40);
+                    if (r == 0) tline.stamp_wave(kTlWaveIssued);
                     if (want_attn && tot > 0) {  // uniform
                         raise_max();
                         consume(0, at_v0, vraw0);
                     }
-                    if (r == 0) HIRA_TLW(48);
+                    if (r == 0) tline.stamp_wave(kTlWaveConsumed);
                 }
                 for (int e0 = kVBatch; e0 < tot; e0 += kVBatch) {  // uniform in the wave; a hot wave
                     int at_v[NPASS], at_k[KB0];
@@ -1083,33 +1069,25 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                     }
                 }
             } else {
-                if (r == 0) HIRA_TL(9);
                 if (want_attn && tot > 0) {  // uniform in the launch / in the wave
                     raise_max();
                     for (int e0 = 0; e0 < tot; e0 += kVBatch) {  // uniform in the wave
                         int at_v[NPASS];
                         uint32_t vraw[kVBatch][VW];
                         issue(e0, at_v, vraw);
-                        if (r == 0 && e0 == 0) HIRA_TLW(40);
+                        if (r == 0 && e0 == 0) tline.stamp_wave(kTlWaveIssued);
                         consume(e0, at_v, vraw);
-                        if (r == 0 && e0 == 0) HIRA_TLW(48);
+                        if (r == 0 && e0 == 0) tline.stamp_wave(kTlWaveConsumed);
                     }
                 }
             }
-            if (r == 0) HIRA_TL(11);
-            if (r == 1) HIRA_TL(13);
-            if (r == 2) HIRA_TL(14);
-            if (r == 3) HIRA_TL(15);
+            if (r == 0) tline.stamp(kTlGathered);
         }
     }  // tree or queue
     if (!want_attn) return;  // uniform
-#ifdef HIRA_TIMELINE
-    if (lane == 0) {
-        tl[16 + wave] = wall_clock64();
-        tl[24 + wave] = tl_rows;
-    }
-#endif
-    HIRA_TL(2);
+    tline.stamp_wave(kTlWaveEnd);
+    tline.set_wave(kTlWaveRows, tline.rows);
+    tline.stamp(kTlWave0Done);
 
     // ---- merge the waves: first one maximum per head for the workgroup, to which every wave
     // brings its sums (m_run: lane = head col; l_mine: head lane % GS); then l and acc add up ---
@@ -1145,7 +1123,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
 #pragma unroll
             for (int e = 0; e < VPL; ++e) macc[(wave * 4 + gi) * D + (tid & 63) * VPL + e] = acc[c * 4 + gi][e];
         __syncthreads();
-        if (c == 0) HIRA_TL(3);
+        if (c == 0) tline.stamp(kTlMerged);
         for (int t = tid; t < 4 * D; t += blockDim.x) {
             const int gi = t / D, e = t % D, g = c * 4 + gi;
             if (g >= G) break;
@@ -1168,10 +1146,12 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
             }
         }
     }
+    tline.stamp(kTlStoresIssued);
     if (p.done == nullptr) return;  // the caller folds the partials in a second launch
 
     // ---- the last workgroup of this tree (and pass) to arrive folds the tree's partials ----
     hand_off_release();
+    tline.stamp(kTlStored);
     __syncthreads();
     if (threadIdx.x == 0) {
         int* ctr = p.done + (size_t)tree * gridDim.z + blockIdx.z;
@@ -1180,7 +1160,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         if (s_last) __hip_atomic_store(ctr, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
-    HIRA_TL(4);
+    tline.stamp(kTlTicket);
     if (!s_last) return;
 
     auto ld = [](const float* q) {
@@ -1226,6 +1206,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         }
     }
     __syncthreads();
+    tline.stamp(kTlFoldListed);
     // phase 2, only partials that hold something.  Where the heads of the tree are consecutive and
     // the workgroup has threads to spare: a thread owns four output columns of a head and every
     // n_grp-th listed partial, eight 16-byte loads in flight (one or two trips to memory for the
@@ -1273,7 +1254,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
             for (int r = 0; r < n_grp; ++r) sum += red[(size_t)r * G * D + t];
             p.attn_out[(size_t)(hoff + g) * D + (t % D)] = Lg > 0.0f ? sum / Lg : 0.0f;
         }
-        HIRA_TL(5);
+        tline.stamp(kTlFoldDone);
         return;
     }
     // otherwise: thread t owns output column e of head g
@@ -1321,7 +1302,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         const float inv = Lg > 0.0f ? 1.0f / Lg : 0.0f;
         p.attn_out[(size_t)head * D + e] = (s0 + s1) * inv;
     }
-    HIRA_TL(5);
+    tline.stamp(kTlFoldDone);
 }
 
 template <int KS, int MT, bool Q8, int POL, int HV = 1>

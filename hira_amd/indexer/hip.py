@@ -133,6 +133,10 @@ class HIPIndexer(BaseIndexer):
         # self.size holds upper bounds and _exact_size the sizes as of the last read-back
         self._pending = 0
         self._exact_size: Optional[List[int]] = None
+        self._unsynced_room = 0  # appends a stretch opened by begin_unsynced still has room for
+        # whether a decode step has looked at its attention mask for this index (padding cannot be
+        # honoured by the sparse step: the attention function checks once per built index)
+        self._decode_mask_checked = False
         self.dtype: Optional[torch.dtype] = None
         self.size: List[int] = []
         self.cap: List[int] = []
@@ -234,6 +238,8 @@ class HIPIndexer(BaseIndexer):
         self.batch, self.num_heads = batch, heads
         self.num_trees = batch * heads
         self.dim, self.vdim, self.dtype = dim, vdim, dtype
+        self._decode_mask_checked = False  # a new index: maybe a new, padded batch
+        self._pending, self._exact_size, self._unsynced_room = 0, None, 0
         bf, nl = self.branching_factor, self.num_levels
         self.size = level_sizes(n, bf, nl)
         want = max(n, int(self.capacity or 0))
@@ -546,7 +552,7 @@ class HIPIndexer(BaseIndexer):
             caps.append(-(-c2 // 16) * 16 if self.tiled else c2)
         if caps == self.cap:
             return
-        if getattr(self, "_unsynced_room", 0) > 0:
+        if self._unsynced_room > 0:
             # a launch captured by begin_unsynced holds the current pointers
             raise RuntimeError(
                 "the index would have to re-allocate while a stretch of unsynced updates is open "
@@ -719,7 +725,7 @@ class HIPIndexer(BaseIndexer):
 
     def note_unsynced(self, m: int) -> None:
         """`m` keys per tree were appended by a launch outside ``update`` (a graph replay)."""
-        if m > getattr(self, "_unsynced_room", 0):
+        if m > self._unsynced_room:
             raise RuntimeError("more appends than begin_unsynced made room for")
         self._unsynced_room -= m
         self._pending += m
@@ -798,6 +804,8 @@ class HIPIndexer(BaseIndexer):
                 if where is not None:
                     return self._graft(new_keys, new_values, m, nl - 1, where)
                 return self._graft(new_keys, new_values, m, nl, None)
+        if not sync and 0 < self._unsynced_room < m:  # (checked before anything is launched)
+            raise RuntimeError("more appends than begin_unsynced made room for")
         need = self._needed_caps(m)
         self._grow(need)
         t = self.num_trees
@@ -819,10 +827,13 @@ class HIPIndexer(BaseIndexer):
             self._adopt_state(self._state.cpu())
             self._unsynced_room = 0
             return self
-        if self._pending == 0:
+        if self._exact_size is None:  # (inside a stretch self.size already holds bounds)
             self._exact_size = list(self.size)
+        if self._unsynced_room > 0:   # a stretch opened by begin_unsynced: its room is used up
+            self._unsynced_room -= m
         self._pending += m
         bound = [need[1] * self.branching_factor] + list(need[1:])
+        bound = [max(a, b) for a, b in zip(bound, self.size)]  # (bounds never shrink)
         if bound != self.size:
             self.size = bound
             self._tree_struct = None

@@ -39,7 +39,7 @@ def _on(t: torch.Tensor, device) -> bool:
 class HIPSearcher(BaseSearcher):
     def __init__(self, block_c=None, output_fill_value: float = DEFAULT_OUTPUT_FILL_VALUE,
                  *, index_space: str = "slot", block_threads: int = 0, nodes_per_wave: int = 0,
-                 kernel: int = 0, separate_merge: bool = False, share: int = 0):
+                 kernel: int = 0, separate_merge: bool = False):
         super().__init__()
         if index_space not in ("slot", "position"):
             raise ValueError("index_space must be 'slot' or 'position'")
@@ -47,7 +47,7 @@ class HIPSearcher(BaseSearcher):
         self.output_fill_value = float(output_fill_value)
         self.index_space = index_space
         self.launch = _lib.HiraLaunch(int(block_threads), int(nodes_per_wave), int(kernel),
-                                      int(bool(separate_merge)), int(share))
+                                      int(bool(separate_merge)))
         self._tmp_out: Optional[torch.Tensor] = None
         self._map_cache = {}
         self._workspace: Optional[torch.Tensor] = None

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define HIRA_ABI_VERSION 4
+#define HIRA_ABI_VERSION 5
 #define HIRA_MAX_LEVELS 8
 #define HIRA_STATS_COLS (HIRA_MAX_LEVELS + 3) /* counters per tree a search can fill in */
 
@@ -151,9 +151,6 @@ typedef struct HiraLaunch {
     int32_t kernel;         /* 0 = auto, 1 = vector-ALU kernel, 2 = MFMA kernel (bf16) */
     int32_t separate_merge; /* != 0: fold the attention partials in a second launch even
                                where the search kernel could do it itself */
-    int32_t share;          /* MFMA kernel: workgroups of a tree that gate the same tiles and
-                               split the surviving nodes among them (share * nodes_per_wave at
-                               most 16); 0 or 1 = every workgroup keeps to its own tiles */
 } HiraLaunch;
 
 int hira_abi_version(void);
@@ -197,7 +194,10 @@ int hira_search(const HiraTree* tree, const HiraQuery* query, const HiraQueue* q
  * that may overlap on one GPU (different streams) race -- order them, or give the others a
  * workspace of their own through hira_search.  The counters are left at zero by every
  * completed call; the partials keep the last call's contents and are overwritten before they
- * are read.
+ * are read.  The first call on a device looks the buffer's address up (a symbol lookup that may
+ * load the library's code object -- not a stream operation): make one call on the device, at
+ * set-up, before a stream capture begins; every later call, under capture too, records nothing
+ * but the kernel launch.
  */
 int hira_search_noalloc(const HiraTree* tree, const HiraQuery* query, const HiraQueue* queue,
                         const HiraSearchOut* out, const HiraLaunch* launch, void* stream);

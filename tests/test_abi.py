@@ -56,7 +56,7 @@ def test_struct_layout_matches_header():
     """ctypes mirrors of the header structs: field order and sizes."""
     assert ctypes.sizeof(_lib.HiraTree) == 8 * 4 + 2 * 8 * 4 + 3 * 8 + 3 * 8 * 8 + 3 * 8
     assert ctypes.sizeof(_lib.HiraQueue) == 24
-    assert ctypes.sizeof(_lib.HiraLaunch) == 20
+    assert ctypes.sizeof(_lib.HiraLaunch) == 16
     assert _lib.HiraQuery.max_group.offset == 48 and _lib.HiraQuery.group_size.offset == 52
     assert _lib.HiraSearchOut.attn_out.offset == 56
 

@@ -380,3 +380,37 @@ def test_unsynced_updates_keep_search_exact(gpu_device):
     assert b.size == a.size
     with pytest.raises(ValueError):
         HIPIndexer(1, 1, bf).build(K[:, :, :n0]).update(K[:, :, n0:n0 + 1], sync=False)
+
+
+def test_updates_inside_an_open_unsynced_stretch(gpu_device):
+    """begin_unsynced(M) then update(sync=False) calls: the sizes of the last read-back stay the
+    base of the capacity bound (so the bound does not creep up call by call), the stretch's room
+    is debited, an append beyond it is refused, and the index stays valid and exact."""
+    from hira_amd.indexer.hip import HIPIndexer
+    from hira_amd.searcher.hip import HIPSearcher
+
+    t, d, bf, n0 = 2, 64, 16, 600
+    keys = clustered_keys(t, n0 + 40, d, seed=5, clusters=12)
+    K = torch.from_numpy(keys)[None]
+    idx = HIPIndexer(3, 1, bf).build(K[:, :, :n0], K[:, :, :n0])
+    exact = list(idx.size)
+    idx.begin_unsynced(8)
+    held, caps = list(idx.size), list(idx.cap)
+    assert idx._exact_size == exact and idx._unsynced_room == 8
+    at = n0
+    for m in (3, 3):
+        idx.update(K[:, :, at:at + m], K[:, :, at:at + m], sync=False)
+        at += m
+        assert idx._exact_size == exact              # not overwritten by the bounds
+        assert idx.size == held and idx.cap == caps  # bounds and pointers of the stretch hold
+    assert idx._unsynced_room == 2 and idx._pending == 6
+    with pytest.raises(RuntimeError):
+        idx.update(K[:, :, at:at + 3], K[:, :, at:at + 3], sync=False)
+    idx.sync_sizes()
+    assert idx._exact_size is None and idx._pending == 0 and idx.num_keys == at
+    _check_tree(idx, keys[:, :at], keys[:, :at])
+    q = random_query(t, d, seed=3)
+    s = ho.scores(keys[:, :at], q, ho.default_q2kv(t, t))
+    th = midpoint_threshold(s, 20)
+    out = HIPSearcher(index_space="position").search(torch.from_numpy(q), torch.from_numpy(th), idx)
+    assert_same_selection(out.cpu().numpy()[:, :at] != 0, s, th)

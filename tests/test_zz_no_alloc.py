@@ -119,3 +119,49 @@ def test_noalloc_refuses_what_does_not_fit(gpu_device):
     assert "scratch buffer" in msg, msg
     with pytest.raises(RuntimeError):
         _lib.check(rc)
+
+
+def test_noalloc_under_graph_capture_after_a_warm_up(gpu_device):
+    """One eager call resolves the scratch buffer's address; after it the call records nothing
+    but the kernel launch, so it can be captured: the graph is replayed for three different
+    queries, with eager work and synchronisations between the replays, and every replay equals
+    hira_search with a caller's workspace bit for bit."""
+    from hira_amd import _lib
+    from hira_amd.cache.threshold_finder import exact_topk
+    from hira_amd.searcher import HIPSearcher
+
+    idx, keys = _index(4, 4096, 128, 32, 3, seed=11)
+    h_q, d = 16, 128
+    _both(idx, keys, h_q, seed=12, keep=40)                     # the warm-up call, eager
+    lib, se = _lib.lib(), HIPSearcher()
+    scale = torch.full((h_q,), d ** -0.5)
+    q = torch.zeros((h_q, d), dtype=torch.bfloat16, device="cuda")      # fixed buffers the graph reads
+    tau = torch.zeros((h_q,), dtype=torch.float32, device="cuda")
+    out = torch.zeros((h_q, d), dtype=torch.float32, device="cuda")
+    qs, keep_alive = se._query_struct(q, tau, idx, None, scale)
+    assert qs.q == q.data_ptr() and qs.tau == tau.data_ptr()    # the launch reads the fixed buffers
+    so = _lib.HiraSearchOut()
+    so.attn_out = out.data_ptr()
+    tree = idx.tree_struct()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            _lib.check(lib.hira_search_noalloc(C.byref(tree), C.byref(qs), None, C.byref(so),
+                                               C.byref(se.launch),
+                                               torch.cuda.current_stream().cuda_stream))
+    torch.cuda.current_stream().wait_stream(side)
+    g = torch.Generator().manual_seed(13)
+    for step in range(3):
+        qn = torch.randn((h_q, d), generator=g).to(torch.bfloat16).cuda()
+        tn = exact_topk(keys[0].cuda(), qn, 30 + 25 * step)
+        want = se.search_attention(qn, tn, idx, scaling=scale).clone()  # eager work between replays
+        q.copy_(qn)
+        tau.copy_(tn)
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), f"replay {step}"
+    del keep_alive
