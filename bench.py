@@ -322,7 +322,7 @@ TL_STAMPS = ["start", "arguments in registers", "gate operands asked for", "wave
              "wave 0: first round listed", "wave 0: first round gathered", "wave 0 at the merge",
              "all waves at the merge", "partial on its way", "partial arrived", "ticket drawn",
              "fold: partials listed", "fold: output written"]
-TL_ROWS, TL_ROUNDS, TL_XCC, TL_LOCAL = 16, 17, 18, 19
+TL_ROWS, TL_ROUNDS, TL_ALIVE = 16, 17, 18
 TL_WAVE_END, TL_WAVE_ROWS, TL_WAVE_SCANNED, TL_WAVE_ISSUED, TL_WAVE_CONSUMED, TL_COLS = 24, 32, 40, 48, 56, 64
 
 
@@ -378,6 +378,41 @@ def timeline_report(a, w, index, searcher, q_d, taus, outs, W, total, scale):
         print(f"{name:34s} {m[0, k]:7.2f} {m[1, k]:7.2f} {m[2, k]:7.2f} {c[k]:12.2f} {step:9.2f}")
         if not np.isnan(c[k]):
             prev = c[k]
+    print("# workgroups of the last step by when all their waves are at the merge: nodes that "
+          "survived the gates, rows listed, the waves' arrival times")
+    merged = np.where(np.isnan(r[:, 10]), -1.0, r[:, 10])
+    alive_n = t[:, TL_ALIVE].astype(float)
+    rows_wg = t[:, TL_WAVE_ROWS:TL_WAVE_ROWS + 8].sum(1).astype(float)
+    for k in np.argsort(-merged)[:8]:
+        ends = (t[k, TL_WAVE_END:TL_WAVE_END + 8] - t0) / 100.0
+        print(f"  merged {merged[k]:6.2f}  tiles asked {r[k, 5]:5.2f}  alive {int(alive_n[k]):3d}  rows {int(rows_wg[k]):4d}  "
+              f"waves {' '.join(f'{x:5.1f}' for x in ends)}  rows/wave {t[k, TL_WAVE_ROWS:TL_WAVE_ROWS + 8].tolist()}")
+    okm = merged > 0
+    print(f"# correlation of a workgroup's merge time with its surviving nodes "
+          f"{np.corrcoef(merged[okm], alive_n[okm])[0, 1]:.2f}, with its rows "
+          f"{np.corrcoef(merged[okm], rows_wg[okm])[0, 1]:.2f}; surviving nodes mean "
+          f"{alive_n[okm].mean():.1f} max {alive_n[okm].max():.0f}; rows mean {rows_wg[okm].mean():.1f} "
+          f"max {rows_wg[okm].max():.0f}")
+    for lo, hi in ((0, 9), (9, 17), (17, 25), (25, 33), (33, 1 << 30)):
+        sel = okm & (alive_n >= lo) & (alive_n < hi)
+        if sel.any():
+            print(f"  workgroups with {lo:2d}..{min(hi - 1, 999):3d} surviving nodes: {int(sel.sum()):4d}  merged at mean "
+                  f"{merged[sel].mean():6.2f} max {merged[sel].max():6.2f}  rows mean {rows_wg[sel].mean():6.1f}")
+    # (last step) per wave with rows: when its scan ended, its first batch of value rows was asked
+    # for and was in the sums
+    wsc = (t[:, TL_WAVE_SCANNED:TL_WAVE_SCANNED + 8] - t0) / 100.0
+    wis = (t[:, TL_WAVE_ISSUED:TL_WAVE_ISSUED + 8] - t0) / 100.0
+    wco = (t[:, TL_WAVE_CONSUMED:TL_WAVE_CONSUMED + 8] - t0) / 100.0
+    wrl = t[:, TL_WAVE_ROWS:TL_WAVE_ROWS + 8]
+    has = (t[:, TL_WAVE_ISSUED:TL_WAVE_ISSUED + 8] != 0) & (wrl > 0)
+    print("# waves of the last step with rows, by when their scan ended: scan end -> first batch asked "
+          "for -> in the sums (mean microseconds), rows")
+    for lo, hi in ((0, 6), (6, 8), (8, 10), (10, 12), (12, 99)):
+        sel = has & (wsc >= lo) & (wsc < hi)
+        if sel.any():
+            print(f"  scan ended {lo:2d}..{hi:2d}: {int(sel.sum()):4d} waves  scanned {wsc[sel].mean():6.2f}  asked "
+                  f"{wis[sel].mean():6.2f}  in the sums {wco[sel].mean():6.2f}  (trip + sums "
+                  f"{(wco[sel] - wis[sel]).mean():5.2f})  rows {wrl[sel].mean():5.1f}")
     we, wr = np.concatenate(wave_end), np.concatenate(wave_rows)
     print("# waves by the rows they listed: count per step, when they arrive at the merge (mean, max)")
     for lo, hi in ((0, 1), (1, 9), (9, 17), (17, 33), (33, 65), (65, 1 << 30)):
@@ -424,6 +459,9 @@ def main():
                     help="file that keeps the steps' thresholds: written when absent, read when "
                          "present (so that a run under a profiler's counters need not launch "
                          "the sort kernels that find them)")
+    ap.add_argument("--lib", default=None,
+                    help="another build of libhira_hip.so to load instead of the one in hira_amd/csrc "
+                         "(to compare two builds on one machine)")
     ap.add_argument("--timeline", action="store_true",
                     help="run the steps on the library built with time stamps "
                          "(`make -C hira_amd/csrc timeline`) and print where a step's time goes")
@@ -449,6 +487,8 @@ def main():
     dev = torch.device("cuda:0")
     if a.timeline:
         _lib.use_library(_lib.CSRC / "libhira_hip_timeline.so")
+    elif a.lib:
+        _lib.use_library(a.lib)
     w = synth.WORKLOADS[a.config]
     if a.context > 0:
         import dataclasses

@@ -30,8 +30,7 @@ enum TlStamp {
     kTlFoldDone,      // fold: output written
     kTlRows,          // (a count, not a time) rows wave 0 listed in the first round
     kTlRounds,        // (a count) rounds of the workgroup
-    kTlXcc,           // (an id) the XCD the workgroup ran on
-    kTlLocal,         // (a flag) the partial went through the XCD's own L2
+    kTlAlive,         // (a count) nodes of the workgroup's tiles that survived the gates
     kTlWaveEnd = 24,       // + wave: the wave arrives at the merge
     kTlWaveRows = 32,      // + wave: (a count) rows the wave listed over all rounds
     kTlWaveScanned = 40,   // + wave: the wave's first round is scanned
