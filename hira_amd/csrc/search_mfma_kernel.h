@@ -269,7 +269,12 @@ __device__ __forceinline__ void touch_kernel_arguments() {
 // head; their bf16 rows (row-major) are fetched, 16 at a time as one MFMA operand, and take the
 // exact test -- with the very products of the other layout, so the selected set and the scores
 // are the same bit for bit.
-template <int KS, int MT, int GS, bool OUT, bool Q8, int POL, int HV>
+// ONE: every workgroup of the launch scans in a single round (the host knows: its tiles hold no
+// more nodes than its waves take at once).  The round is then straight-line code without a loop
+// around it, in which the compiler's waits count the loads still in flight and a node's products
+// start when ITS tiles have arrived; at the head of a loop they fall back to waiting for
+// everything asked for so far.
+template <int KS, int MT, int GS, bool OUT, bool Q8, int POL, int HV, bool ONE>
 __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const SearchParams p) {
     using S = MfmaShape<KS, MT, GS, Q8>;
     constexpr int D = S::D;
@@ -649,7 +654,10 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
             tline.set(kTlAlive, (unsigned long long)alive);
         }
 
-        const float sc2 = sc * kLog2e;
+        float sc2 = sc * kLog2e;
+        asm volatile("" : "+v"(sc2));  // (computed here, where its load has long arrived, and not
+                                       // behind the key tiles' requests, where it would be waited
+                                       // for with all of them)
         const size_t row0 = (size_t)tree * p.cap[0];
 
         // (8-bit shadow: krsrc = the bf16 rows of the exact test, row-major; k8rsrc = the tiles
@@ -706,9 +714,11 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                         load_tile_buf<KA, false>(k8rsrc, (unsigned)lane * 16u + (tt * 16 < nx_cnt[u] ? 0u : 0x80000000u),
                                           (tile_first + tt) * (unsigned)(KA * 1024), a[u][tt]);
                     } else {
-                        if (tt * 16 < nx_cnt[u])
-                            load_tile_buf<KA, POL != 0>(krsrc, (unsigned)lane * 16u,
-                                              (tile_first + tt) * (unsigned)(KA * 1024), a[u][tt]);
+                        // (every load is issued, a tile that is not there beyond the end of the
+                        // buffer -- zeros, no memory access: straight-line code, in which the waits
+                        // further down can count the loads behind them)
+                        load_tile_buf<KA, POL != 0>(krsrc, (unsigned)lane * 16u + (tt * 16 < nx_cnt[u] ? 0u : 0x80000000u),
+                                          (tile_first + tt) * (unsigned)(KA * 1024), a[u][tt]);
                     }
                 }
             }
@@ -719,7 +729,9 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         constexpr int KB0 = KS <= 4 ? 2 : 1;      // batches of 16 key rows asked for ahead
         constexpr int RP = 64 / GS;               // rows whose weights one pass over the lanes computes
         constexpr int NPASS = kVBatch / RP;       // GS = 4: 2, GS = 8: 4, GS = 16: 8
-        for (int r = 0; r < rounds; ++r) {  // uniform in the workgroup
+        // one round of a wave
+        auto do_round = [&](const int r) {
+            constexpr bool SINGLE = ONE;
             // the round's score table and row list; every wave has a stretch of ROWS * NB rows of
             // its own and nobody else looks at it: no barrier inside the rounds
             uint32_t* lst_row = s_words;                                        // (LIST) listed row -> table row
@@ -854,10 +866,10 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 } else {
                 f32x4_t sco_u[MT];
 #pragma unroll
-                for (int tt = 0; tt < MT; ++tt)  // (only read where it is written: under this condition)
-                    if (tt * 16 < cnt[u]) sco_u[tt] = tile_scores_lds<KS>(a[u][tt], s_bq, lane);
+                for (int tt = 0; tt < MT; ++tt)  // (a tile that is not there came as zeros)
+                    sco_u[tt] = tile_scores_lds<KS>(a[u][tt], s_bq, lane);
                 if (r == 0 && u == 0) tline.stamp(kTlTiles);
-                if (r + 1 < rounds) fetch(r + 1, u);
+                if constexpr (!SINGLE) fetch(r + 1, u);  // (past the last round: no node, nothing read)
                 // a head for which the node did not survive selects nothing
                 const float tau_u = ((nmask[u] >> col) & 1u) ? tau : INFINITY;
                 if (stats && lane == 0) stat_add(stats, 0, (unsigned)cnt[u]);
@@ -1124,6 +1136,11 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                 }
             }
             if (r == 0) tline.stamp(kTlGathered);
+        };
+        if constexpr (ONE) {
+            if (rounds > 0) do_round(0);
+        } else {
+            for (int r = 0; r < rounds; ++r) do_round(r);  // uniform in the workgroup
         }
     }  // tree or queue
     if (!want_attn) return;  // uniform
@@ -1347,20 +1364,29 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     tline.stamp(kTlFoldDone);
 }
 
-template <int KS, int MT, bool Q8, int POL, int HV = 1>
-void launch_mfma_gs(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s) {
+// the attention-only scan of bf16 tiles has an instantiation for launches of a single round
+template <int KS, int MT, int GS, bool Q8, int POL, int HV>
+void launch_mfma_one(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s) {
     const dim3 block(plan.threads);
     const bool out = p.dense != nullptr || p.sel_count != nullptr;
-    if (plan.gmax <= 4) {
-        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 4, true, Q8, POL, HV>), grid, block, 0, s, p);
-        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 4, false, Q8, POL, HV>), grid, block, 0, s, p);
-    } else if (plan.gmax <= 8) {
-        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 8, true, Q8, POL, HV>), grid, block, 0, s, p);
-        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 8, false, Q8, POL, HV>), grid, block, 0, s, p);
+    // nodes (entries of the survivors' list) a workgroup's tiles hold at most, against those its
+    // waves take in one round
+    const bool one = plan.nodes_per_wave * 16 * HV <= (plan.threads / 64) * MfmaShape<KS, MT, GS, Q8>::NB;
+    if (out) {
+        hipLaunchKernelGGL((search_mfma_kernel<KS, MT, GS, true, Q8, POL, HV, false>), grid, block, 0, s, p);
+    } else if constexpr (!Q8) {
+        if (one) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, GS, false, Q8, POL, HV, true>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, GS, false, Q8, POL, HV, false>), grid, block, 0, s, p);
     } else {
-        if (out) hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 16, true, Q8, POL, HV>), grid, block, 0, s, p);
-        else hipLaunchKernelGGL((search_mfma_kernel<KS, MT, 16, false, Q8, POL, HV>), grid, block, 0, s, p);
+        hipLaunchKernelGGL((search_mfma_kernel<KS, MT, GS, false, Q8, POL, HV, false>), grid, block, 0, s, p);
     }
+}
+
+template <int KS, int MT, bool Q8, int POL, int HV = 1>
+void launch_mfma_gs(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s) {
+    if (plan.gmax <= 4) launch_mfma_one<KS, MT, 4, Q8, POL, HV>(plan, p, grid, s);
+    else if (plan.gmax <= 8) launch_mfma_one<KS, MT, 8, Q8, POL, HV>(plan, p, grid, s);
+    else launch_mfma_one<KS, MT, 16, Q8, POL, HV>(plan, p, grid, s);
 }
 
 template <int KS, bool Q8, int POL>
