@@ -283,7 +283,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     constexpr int KS8 = Q8 ? KS / 2 : 1;
     constexpr int VPL = KS / 2;        // value elements per lane: Dv = D = 64 * VPL
     constexpr int VW = (VPL + 1) / 2;  // dwords of a value row per lane
-    __shared__ uint32_t s_words[S::WORDS];  // the round's list; the merge; the fold
+    __shared__ __align__(16) uint32_t s_words[S::WORDS];  // the round's list; the merge; the fold
     // a node of my tiles: heads for which it survives (16 bits) | child count << 16
     __shared__ uint32_t s_ninfo[kMfmaMaxTilesPerWg * 16];
     // the surviving ones in order, a copy per wave (each wave makes its own: no barrier):
@@ -354,6 +354,21 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     for (int g = 0; g < GS; ++g)
 #pragma unroll
         for (int e = 0; e < VPL; ++e) acc[g][e] = 0.0f;
+    // The gather of the single-round instantiations (up to 8 heads a pass, rows of 256 bytes)
+    // fetches value rows 16 bytes a lane: LR lanes share a row, one load instruction brings RPI
+    // rows, and lane (row group rg, chunk cc) sums columns 8 cc .. 8 cc + 7 of the rows of its
+    // group in acc8; the row groups' sums meet before the merge.  (A quarter of the load
+    // instructions and half the instructions per row of the gather below, which holds a row in
+    // 4 bytes a lane and has the registers that the tiles in flight of several rounds leave.)
+    constexpr bool WIDE = ONE && !Q8 && GS <= 8 && KS == 4;
+    constexpr int LR = D / 8;     // lanes per value row
+    constexpr int RPI = 64 / LR;  // rows per load instruction
+    const int rg = lane / LR, cc = lane % LR;
+    float acc8[WIDE ? GS : 1][8];
+#pragma unroll
+    for (int g = 0; g < (WIDE ? GS : 1); ++g)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc8[g][j] = 0.0f;
 
     if (is_queue) {
         // ---- the queue of keys appended since the last update of the tree: row-major, every
@@ -1012,8 +1027,13 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
 #pragma unroll
                     for (int g = 0; g < GS; ++g) {
                         const float fg = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), g));
+                        if constexpr (WIDE) {
 #pragma unroll
-                        for (int e = 0; e < VPL; ++e) acc[g][e] *= fg;
+                            for (int j = 0; j < 8; ++j) acc8[g][j] *= fg;
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < VPL; ++e) acc[g][e] *= fg;
+                        }
                     }
                 }
             };
@@ -1123,6 +1143,72 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
                     }
                 }
             } else {
+                if constexpr (WIDE) {
+                    if (want_attn && tot > 0) {  // uniform in the launch / in the wave
+                        raise_max();
+                        constexpr int NLD = kVBatch / RPI;  // load instructions of a batch
+                        for (int e0 = 0; e0 < tot; e0 += kVBatch) {  // uniform in the wave
+                            // the batch's rows in the score table: for the weights (lane = (row of
+                            // the pass, head)) and for the loads (lane = (row group, chunk))
+                            int at_w[NPASS], at_r[NLD];
+#pragma unroll
+                            for (int ps = 0; ps < NPASS; ++ps) {
+                                const int le = e0 + ps * RP + lane_o / GS;
+                                at_w[ps] = le < tot ? (int)lst_row[zrow0 + le] : -1;  // (-1: past the end)
+                            }
+#pragma unroll
+                            for (int i = 0; i < NLD; ++i) {
+                                const int le = e0 + i * RPI + rg;
+                                at_r[i] = le < tot ? (int)lst_row[zrow0 + le] : -1;
+                            }
+                            uint4 vr[NLD];
+#pragma unroll
+                            for (int i = 0; i < NLD; ++i) {  // (rows past the end: slot 0, weight 0)
+                                const unsigned slot =
+                                    at_r[i] >= 0 ? lst_tslot[at_r[i] >> 4] + (unsigned)(at_r[i] & 15) : 0u;
+                                vr[i] = __builtin_bit_cast(
+                                    uint4, __builtin_amdgcn_raw_buffer_load_b128(
+                                               vrsrc, slot * (unsigned)(D * 2) + (unsigned)cc * 16u, 0,
+                                               POL == 2 ? kReadOnce : 0));
+                            }
+                            if (r == 0 && e0 == 0) tline.stamp_wave(kTlWaveIssued);
+                            __builtin_amdgcn_sched_barrier(0);
+                            // scores -> weights, in place, 64 (row, head) pairs at a time
+#pragma unroll
+                            for (int ps = 0; ps < NPASS; ++ps) {
+                                if (at_w[ps] >= 0) {
+                                    float* zp = lst_z + at_w[ps] * GS + (lane_o & (GS - 1));
+                                    const float w = __builtin_amdgcn_exp2f(*zp - m_lane);
+                                    l_mine += w;
+                                    *zp = w;
+                                }
+                            }
+#pragma unroll
+                            for (int i = 0; i < NLD; ++i) {
+                                if (e0 + i * RPI >= tot) break;  // uniform
+                                float wv[GS];
+#pragma unroll
+                                for (int g4 = 0; g4 < GS / 4; ++g4) {
+                                    float4 w4 = make_float4(0.f, 0.f, 0.f, 0.f);
+                                    if (at_r[i] >= 0)
+                                        w4 = *reinterpret_cast<const float4*>(lst_z + at_r[i] * GS + 4 * g4);
+                                    wv[4 * g4 + 0] = w4.x;
+                                    wv[4 * g4 + 1] = w4.y;
+                                    wv[4 * g4 + 2] = w4.z;
+                                    wv[4 * g4 + 3] = w4.w;
+                                }
+                                const uint4 raw = at_r[i] >= 0 ? vr[i] : make_uint4(0, 0, 0, 0);
+                                float vf[8];
+                                unpack<bf16_t>(raw, vf);
+#pragma unroll
+                                for (int g = 0; g < GS; ++g)
+#pragma unroll
+                                    for (int j = 0; j < 8; ++j) acc8[g][j] += wv[g] * vf[j];
+                            }
+                            if (r == 0 && e0 == 0) tline.stamp_wave(kTlWaveConsumed);
+                        }
+                    }
+                } else
                 if (want_attn && tot > 0) {  // uniform in the launch / in the wave
                     raise_max();
                     for (int e0 = 0; e0 < tot; e0 += kVBatch) {  // uniform in the wave
@@ -1151,6 +1237,7 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     // ---- merge the waves: first one maximum per head for the workgroup, to which every wave
     // brings its sums (m_run: lane = head col; l_mine: head lane % GS); then l and acc add up ---
     if (kb == 0) s_mxw[wave * 16 + col] = m_run;
+    const bool wide = WIDE && !is_queue;  // uniform: my sums are in acc8
     __syncthreads();
     {
         float m_all = -INFINITY;
@@ -1162,6 +1249,10 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
             const float fg = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(fw), g));
 #pragma unroll
             for (int e = 0; e < VPL; ++e) acc[g][e] *= fg;
+            if constexpr (WIDE) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc8[g][j] *= fg;
+            }
         }
         m_run = m_all;
     }
@@ -1177,10 +1268,34 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     for (int c = 0; c < GS / 4; ++c) {
         if (c * 4 >= G) continue;  // uniform (no break: the loop has to unroll)
         __syncthreads();           // the list (or the previous four heads) is not needed any more
+        if (wide) {
+            if constexpr (WIDE) {
+                // The four row groups' sums of the four heads meet so that group rg ends up with
+                // head rg: the halves of the wave trade heads (0,1) against (2,3) -- one swap
+                // leaves, in the lower half, both halves' sums of head 0 or 1, in the upper half
+                // those of head 2 or 3 --, then the rows of 16 lanes trade (0,2) against (1,3).
+                float mine[8];
 #pragma unroll
-        for (int gi = 0; gi < 4; ++gi)
+                for (int j = 0; j < 8; ++j) {
+                    const auto s02 = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc8[c * 4 + 0][j]),
+                                                                      __float_as_uint(acc8[c * 4 + 2][j]), false, false);
+                    const auto s13 = __builtin_amdgcn_permlane32_swap(__float_as_uint(acc8[c * 4 + 1][j]),
+                                                                      __float_as_uint(acc8[c * 4 + 3][j]), false, false);
+                    const float r02 = __uint_as_float(s02[0]) + __uint_as_float(s02[1]);
+                    const float r13 = __uint_as_float(s13[0]) + __uint_as_float(s13[1]);
+                    const auto t = __builtin_amdgcn_permlane16_swap(__float_as_uint(r02), __float_as_uint(r13), false, false);
+                    mine[j] = __uint_as_float(t[0]) + __uint_as_float(t[1]);
+                }
+                float4* dst = reinterpret_cast<float4*>(macc + (wave * 4 + ((tid & 63) / LR)) * D + ((tid & 63) % LR) * 8);
+                dst[0] = make_float4(mine[0], mine[1], mine[2], mine[3]);
+                dst[1] = make_float4(mine[4], mine[5], mine[6], mine[7]);
+            }
+        } else {
 #pragma unroll
-            for (int e = 0; e < VPL; ++e) macc[(wave * 4 + gi) * D + (tid & 63) * VPL + e] = acc[c * 4 + gi][e];
+            for (int gi = 0; gi < 4; ++gi)
+#pragma unroll
+                for (int e = 0; e < VPL; ++e) macc[(wave * 4 + gi) * D + (tid & 63) * VPL + e] = acc[c * 4 + gi][e];
+        }
         __syncthreads();
         if (c == 0) tline.stamp(kTlMerged);
         for (int t = tid; t < 4 * D; t += blockDim.x) {
