@@ -99,6 +99,34 @@ def cpu_index_build(w, keys_slots, perm):
                       "where it holds more), built once"}
 
 
+def host_cpu():
+    """The host this process runs on: model name, logical CPUs of the machine, physical cores,
+    and the logical CPUs this process may use (the box's share of a shared machine)."""
+    model, cores = "unknown", set()
+    try:
+        phys = core = None
+        for line in open("/proc/cpuinfo", encoding="utf-8", errors="replace"):
+            key, _, val = line.partition(":")
+            key, val = key.strip(), val.strip()
+            if key == "model name" and model == "unknown":
+                model = val
+            elif key == "physical id":
+                phys = val
+            elif key == "core id":
+                core = val
+            elif not key and phys is not None and core is not None:
+                cores.add((phys, core))
+                phys = core = None
+    except OSError:
+        pass
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count() or 1
+    return {"cpu_model": model, "nproc": os.cpu_count() or 1, "physical_cores": len(cores) or None,
+            "usable_cpus": usable}
+
+
 def cpu_baseline(w, index, queries, taus, scale, budget_s=20.0, gpu_out=None, gpu_sel=None):
     """Reference CPU search (+ host softmax-V) on the same trees, first steps of the same
     queries, for about `budget_s` seconds of CPU work; one sequence after the other when the
@@ -225,6 +253,7 @@ def cpu_baseline(w, index, queries, taus, scale, budget_s=20.0, gpu_out=None, gp
                       f"thresholds); median; p99 {float(np.percentile(times, 99) * 1e6):.0f} us; "
                       f"search = reference v3 C++ kernel, attention = numpy fp32",
                one_thread_us=float(np.median(times1) * 1e6), one_thread_steps=len(times1))
+    res.update(host_cpu())  # (`cores` above: the threads the timed kernel used)
     res["index_build"] = cpu_index_build(w, keys_all, perm_all)
     if gpu_out is not None:
         res["gpu_vs_cpu"] = {"steps_compared": compared, "attn_max_rel_err": attn_err,

@@ -171,3 +171,57 @@ def test_large_fp32_trees_on_the_vector_kernel(gpu_device):
     ref = torch.einsum("tgk,tgkd->tgd", w, vsel).reshape(t * grp, d)
     err = ((out.double() - ref).abs().max(dim=1).values / ref.abs().max(dim=1).values).max()
     assert float(err) <= 1e-5, float(err)
+
+
+FOLD_CASES = [
+    # trees, keys per tree, heads a tree, keys kept per head, tiles per workgroup (0 = plan's choice)
+    (8, 32768, 4, 328, 0),      # the benchmark's shape: 32 partials a head, single round
+    (1, 131072, 4, 655, 0),     # a lone tree: 128 partials a head
+    (1, 200000, 8, 1000, 0),    # 8 heads a tree, 98 workgroups of unequal tile counts
+    (32, 32768, 4, 200, 0),     # more workgroups than compute units: several rounds of them
+    (8, 16384, 4, 160, 1),      # one tile a workgroup by request: 32 partials, every wave one node
+    (4, 8192, 16, 80, 0),       # 16 heads a tree
+]
+
+
+@pytest.mark.parametrize("t,n,g,keep,tpw", FOLD_CASES)
+def test_fused_fold_equals_the_fold_of_a_second_launch(t, n, g, keep, tpw, gpu_device):
+    """The search kernel's last workgroup of a tree folds the tree's attention partials inside the
+    launch, behind a hand-off that rests on the completion of write-through stores; asked for
+    (`separate_merge`), the partials are folded by a second launch instead, which sees them behind
+    the kernel boundary.  Both must give the same output: a partial that the in-launch fold read
+    too early (stale, or not yet there) would show as a difference far above rounding.  The two
+    folds add the partials up in different orders, so the comparison is to 2e-6 of a head's
+    largest output, not bit for bit; each path must repeat its own result bit for bit."""
+    from hira_amd.cache.threshold_finder import exact_topk
+    from hira_amd.indexer import HIPIndexer
+    from hira_amd.searcher import HIPSearcher
+
+    gen = torch.Generator().manual_seed(1000 * t + g)
+    d, h = 128, t * g
+    K = torch.randn(1, t, n, d, generator=gen).bfloat16().cuda()
+    V = torch.randn(1, t, n, d, generator=gen).bfloat16().cuda()
+    idx = HIPIndexer(3, 1, 32).build(K, V)
+    sc = torch.full((h,), d ** -0.5)
+    fused = HIPSearcher(kernel=2, nodes_per_wave=tpw)
+    apart = HIPSearcher(kernel=2, nodes_per_wave=tpw, separate_merge=True)
+    for step in range(3):   # fresh queries: the workspace's partials are overwritten every time
+        q = torch.randn(h, d, generator=gen).bfloat16().cuda()
+        tau = exact_topk(K[0], q, keep)
+        a = fused.search_attention(q, tau, idx, scaling=sc).clone()
+        b = apart.search_attention(q, tau, idx, scaling=sc).clone()
+        scale = b.abs().max(dim=1, keepdim=True).values
+        assert float(((a - b).abs() / scale).max()) <= 2e-6, (step, float(((a - b).abs() / scale).max()))
+        assert torch.equal(a, fused.search_attention(q, tau, idx, scaling=sc))
+        assert torch.equal(b, apart.search_attention(q, tau, idx, scaling=sc))
+    # against the definition, once (the last step's queries, a few trees): softmax over exactly
+    # the kept keys
+    for i in range(min(t, 3)):
+        qi = q[i * g:(i + 1) * g].double()
+        s = qi @ K[0, i].double().T
+        top = s.topk(keep, dim=-1)
+        w = torch.softmax(top.values * d ** -0.5, dim=-1)
+        ref = torch.einsum("hk,hkd->hd", w, V[0, i].double()[top.indices])
+        got = a[i * g:(i + 1) * g].double()
+        err = ((got - ref).abs().max(dim=1).values / ref.abs().max(dim=1).values).max()
+        assert float(err) <= 2e-3, (i, float(err))

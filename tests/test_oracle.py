@@ -9,7 +9,7 @@ import torch
 
 from oracle import hira_oracle as ho
 from oracle.build_ref import load_ref
-from helpers import midpoint_threshold, normalized_keys, random_query
+from helpers import clustered_keys, midpoint_threshold, normalized_keys, random_query
 
 GOLDEN = sorted(glob.glob(str(Path(__file__).parent / "golden" / "*.npz")))
 
@@ -214,3 +214,49 @@ def test_attention_matches_torch_softmax_and_full_selection_is_sdpa():
         Q.view(2, 2, 1, 16), K.view(2, 1, 64, 16).expand(2, 2, 64, 16),
         V.view(2, 1, 64, 24).expand(2, 2, 64, 24), scale=0.25).reshape(4, 24)
     np.testing.assert_allclose(full, sdpa.numpy(), atol=1e-10)
+
+
+def test_group_traffic_equals_a_numpy_union_on_a_tiny_tree():
+    """The numerator of every roofline figure: per KV head and level, the nodes that at least one
+    head of the group evaluates (a maximum or a sum over the heads would pass the bounds of the
+    test above), restated here level by level with numpy sets on a tree small enough to follow."""
+    h_kv, g, n, d, bf = 2, 3, 96, 16, 4
+    keys = clustered_keys(h_kv, n, d, seed=21, clusters=6)
+    q = random_query(h_kv * g, d, seed=22)
+    ff = ho.fixed_fanout_tree(keys, bf, 3, niter=4)
+    tree, csr = ho.fixed_fanout_as_cpu_tree(ff)
+    q2kv = ho.default_q2kv(h_kv * g, h_kv)
+    s = ho.scores(ff.keys, q, q2kv)
+    th = midpoint_threshold(np.where(ff.perm[q2kv] >= 0, s, -1e30), 9)
+    tr = ho.group_traffic(tree, q, th, q2kv=q2kv, csr=csr)
+    assert tr.shape == (h_kv, 4)
+    strict = False
+    for kv in range(h_kv):
+        heads = [h for h in range(h_kv * g) if q2kv[h] == kv]
+        seen = {0: set(), 1: set(), 2: set()}   # level -> nodes (keys at level 0) evaluated by some head
+        picked = set()
+        for h in heads:
+            alive = []
+            for p in range(ff.sizes[2]):        # the root level: every node that holds children
+                if ff.counts[2][kv, p] > 0:
+                    seen[2].add(p)
+                    if ff.centers[2][kv, p] @ q[h] + ff.radii[2][kv, p] >= th[h]:
+                        alive.append(p)
+            nxt = []
+            for p in alive:
+                for c in range(p * bf, p * bf + ff.counts[2][kv, p]):
+                    seen[1].add(c)
+                    if ff.centers[1][kv, c] @ q[h] + ff.radii[1][kv, c] >= th[h]:
+                        nxt.append(c)
+            for p in nxt:
+                for i in range(p * bf, p * bf + ff.counts[1][kv, p]):
+                    seen[0].add(i)
+                    if ff.keys[kv, i] @ q[h] >= th[h]:
+                        picked.add(i)
+        want = [len(seen[0]), len(seen[1]), len(seen[2]), len(picked)]
+        assert tr[kv].tolist() == want, (kv, tr[kv].tolist(), want)
+        # the heads do differ here: the union is neither one head's count nor the sum of them
+        _, st = ho.search_v3(tree, q, th, q2kv=q2kv, csr=csr, want_stats=True)
+        assert st[heads, 0].max() <= want[0] <= st[heads, 0].sum()
+        strict = strict or st[heads, 0].max() < want[0] < st[heads, 0].sum()
+    assert strict
