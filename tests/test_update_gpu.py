@@ -414,3 +414,44 @@ def test_updates_inside_an_open_unsynced_stretch(gpu_device):
     th = midpoint_threshold(s, 20)
     out = HIPSearcher(index_space="position").search(torch.from_numpy(q), torch.from_numpy(th), idx)
     assert_same_selection(out.cpu().numpy()[:, :at] != 0, s, th)
+
+
+@pytest.mark.parametrize("t,n0,m,d,bf,nl,dtype,layout", [
+    (2, 2048, 100, 128, 32, 3, torch.bfloat16, "auto"),   # every node full: a node opens every 32 keys
+    (2, 2048, 255, 128, 32, 4, torch.bfloat16, "q8"),     # with the 8-bit shadow, 4 levels
+    (3, 1000, 70, 64, 16, 3, torch.bfloat16, "auto"),     # free slots here and there
+    (2, 5000, 130, 32, 8, 3, torch.float32, "auto"),      # fp32 rows; more nodes with room than the list holds
+    (1, 300, 40, 256, 16, 2, torch.float32, "auto"),      # wide rows (a short chunk), two levels
+])
+def test_a_window_placed_at_once_equals_key_by_key(t, n0, m, d, bf, nl, dtype, layout, gpu_device):
+    """update() with a window of several keys (the kernel that reads the nodes with room into LDS
+    once and places key after key from there) against the same keys appended one call each (the
+    general kernel): the same slots, counts, centres and radii bit for bit, and a valid tree."""
+    from hira_amd.indexer.hip import HIPIndexer
+
+    keys = clustered_keys(t, n0 + m + 7, d, seed=31 + m, clusters=20)
+    if dtype == torch.bfloat16:
+        keys = bf16_round(keys)
+    K = torch.from_numpy(keys)[None].to(dtype)
+    mk = lambda: HIPIndexer(nl, 1, bf, layout=layout, graft_min=1 << 30).build(K[:, :, :n0], K[:, :, :n0])
+    a, b = mk(), mk()
+    a.update(K[:, :, n0:n0 + m], K[:, :, n0:n0 + m])
+    for i in range(m):
+        b.update(K[:, :, n0 + i:n0 + i + 1], K[:, :, n0 + i:n0 + i + 1])
+    # and a second, short window on top (the list is read anew)
+    a.update(K[:, :, n0 + m:n0 + m + 7], K[:, :, n0 + m:n0 + m + 7])
+    for i in range(m, m + 7):
+        b.update(K[:, :, n0 + i:n0 + i + 1], K[:, :, n0 + i:n0 + i + 1])
+    assert a.size == b.size and a.num_keys == b.num_keys == n0 + m + 7
+    n = a.size[0]
+    assert torch.equal(a.perm[:, :n], b.perm[:, :n])
+    assert torch.equal(a.keys_buf[:, :a.cap[0]], b.keys_buf[:, :b.cap[0]])
+    assert torch.equal(a.values_buf[:, :n], b.values_buf[:, :n])
+    for l in range(1, nl):
+        k = a.size[l]
+        assert torch.equal(a.counts[l][:, :k], b.counts[l][:, :k]), f"counts level {l}"
+        assert torch.equal(a.radii[l][:, :k], b.radii[l][:, :k]), f"radii level {l}"
+        assert torch.equal(a.centers[l][:, :a.cap[l]], b.centers[l][:, :b.cap[l]]), f"centres level {l}"
+    if layout == "q8":
+        assert torch.equal(a.keys8, b.keys8) and torch.equal(a.keps[:, :a.size[1]], b.keps[:, :b.size[1]])
+    _check_tree(a, keys[:, :n0 + m + 7], keys[:, :n0 + m + 7])
