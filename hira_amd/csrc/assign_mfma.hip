@@ -18,7 +18,7 @@
 //               the products of its centroid column n with rows 4*kb + j, keeps the best
 //               (value, index) per row, and the 16 columns are merged at the end
 //               (lowest index on ties).
-#include "common.hip.h"
+#include "assign.h"
 
 namespace hira {
 
@@ -31,10 +31,6 @@ constexpr int kAssignStage = 4;    // centroid tiles staged together: the time t
                                    // matrix cores busy covers the latency of fetching the next
                                    // four (two for D = 256, whose tiles are twice as large)
 constexpr int assign_stage(int KS) { return KS <= 4 ? kAssignStage : kAssignStage / 2; }
-
-__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
-    return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
-}
 
 template <int KS>
 __global__ __launch_bounds__(64) void k_cent_prep(const float* cent, int K, const int32_t* fill,
@@ -75,7 +71,7 @@ template <int KS>
 __global__ __launch_bounds__(kAssignThreads, 2) void k_assign_mfma(
     const void* x, int n_c, size_t x_tree_stride, const uint4* tiles, const float* cn2, int Kt,
     const int32_t* list, const int32_t* list_count, size_t list_stride, int32_t* assign,
-    float* dist) {
+    float* dist, int K, AssignCounting ac) {
     constexpr int D = 32 * KS;
     constexpr int RI = kAssignRI;
     constexpr int TILE_CHUNKS = 2 * KS * 64;                 // hi and lo halves of 16 centroids
@@ -93,7 +89,11 @@ __global__ __launch_bounds__(kAssignThreads, 2) void k_assign_mfma(
     const int t = blockIdx.y;
     const int n_items = list ? list_count[t] : n_c;
     const int first = (blockIdx.x * (kAssignThreads / 64) + wave) * (RI * 16);
-    if ((int)blockIdx.x * (kAssignThreads / 64) * (RI * 16) >= n_items) return;  // uniform
+    // (a launch that counts: a workgroup without items still draws its ticket at the end)
+    const bool active = (int)blockIdx.x * (kAssignThreads / 64) * (RI * 16) < n_items;  // uniform
+    if (ac.counts == nullptr && !active) return;
+    if (ac.zero != nullptr && blockIdx.x == 0 && threadIdx.x == 0) ac.zero[t] = 0;
+    if (active) {
 
     // ---- my items: operand tiles in registers, ||x||^2 of row lane % 16 ------------------
     int item[RI];
@@ -195,7 +195,12 @@ __global__ __launch_bounds__(kAssignThreads, 2) void k_assign_mfma(
         __syncthreads();
     }
 
-    // ---- merge the 16 centroid columns of a row group; column 0 writes -----------------------
+    // ---- merge the 16 centroid columns of a row group; the wave's 64 results pass through LDS
+    // (free behind the loop's last barrier) so that every lane ends up with one item: one store
+    // instruction, and one counting instruction, for the whole wave -----------------------------
+    static_assert(RI * 16 == 64, "one result per lane");
+    int* s_g = reinterpret_cast<int*>(s_dyn) + wave * 128;
+    float* s_b = reinterpret_cast<float*>(s_g + 64);
 #pragma unroll
     for (int ri = 0; ri < RI; ++ri)
 #pragma unroll
@@ -211,14 +216,27 @@ __global__ __launch_bounds__(kAssignThreads, 2) void k_assign_mfma(
                     g = og;
                 }
             }
-            // row 4*kb + j of the operand tile: its item and ||x||^2 live in lane 4*kb + j
-            const int it = __shfl(item[ri], 4 * kb + j, 64);
-            const float xx = __shfl(x2[ri], 4 * kb + j, 64);
-            if (n == 0 && it >= 0) {
-                assign[(size_t)t * n_c + it] = g;
-                dist[(size_t)t * n_c + it] = fmaxf(b + xx, 0.0f);
+            if (n == 0) {  // row 4*kb + j of operand tile ri
+                s_g[ri * 16 + 4 * kb + j] = g;
+                s_b[ri * 16 + 4 * kb + j] = b;
             }
         }
+    __builtin_amdgcn_wave_barrier();
+    {
+        // lane (kb, n) takes row n of operand tile kb: its item and ||x||^2 are its own
+        const int g = s_g[lane];
+        const float b = s_b[lane];
+        const int it = kb == 0 ? item[0] : kb == 1 ? item[1] : kb == 2 ? item[2] : item[3];
+        const float xx = kb == 0 ? x2[0] : kb == 1 ? x2[1] : kb == 2 ? x2[2] : x2[3];
+        if (it >= 0) {
+            assign[(size_t)t * n_c + it] = g;
+            dist[(size_t)t * n_c + it] = fmaxf(b + xx, 0.0f);
+            if (ac.counts != nullptr && g >= 0)
+                ac.pos[(size_t)t * n_c + it] = atomicAdd(&ac.counts[(size_t)t * K + g], 1);
+        }
+    }
+    }  // active
+    if (ac.counts != nullptr) finish_counts(ac, t, K, (int)gridDim.x);
 }
 
 // centroid tiles per tree, in whole stages
@@ -246,7 +264,7 @@ int launch_cent_prep(int dim, const float* cent, int K, int num_trees, const int
 int launch_assign_mfma(int dim, const void* x, int n_c, size_t x_tree_stride, const void* tiles,
                        const float* cn2, int K, int num_trees, const int32_t* list,
                        const int32_t* list_count, size_t list_stride, int32_t* assign, float* dist,
-                       hipStream_t s) {
+                       const AssignCounting& counting, hipStream_t s) {
     const int Kt = assign_tiles(K);
     const int per_block = (kAssignThreads / 64) * kAssignRI * 16;
     const int tps = assign_stage(dim / 32);
@@ -261,7 +279,8 @@ int launch_assign_mfma(int dim, const void* x, int n_c, size_t x_tree_stride, co
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) \
             return fail(HIRA_ELAUNCH, "MFMA assignment: %zu bytes of LDS refused", smem);              \
         hipLaunchKernelGGL((k_assign_mfma<KS>), grid, dim3(kAssignThreads), smem, s, x, n_c,        \
-                           x_tree_stride, tl, cn2, Kt, list, list_count, list_stride, assign, dist); \
+                           x_tree_stride, tl, cn2, Kt, list, list_count, list_stride, assign, dist, \
+                           K, counting);                                                            \
     }                                                                                               \
     break;
         case 64: HIRA_ASSIGN_MFMA(2)

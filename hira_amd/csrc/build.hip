@@ -18,6 +18,7 @@
 // layout: r_p = max over children (||c_child - c_p|| + r_child), the bound of
 // indexer/cpu.py:286-309 / indexer/cuda.py:114-198, against the ROUNDED centres and
 // nudged up by a few ulp so that rounding never makes a ball too small.
+#include "assign.h"
 #include "rows.h"
 
 namespace hira {
@@ -38,12 +39,58 @@ __global__ void k_fill_i32(int32_t* p, size_t n, int32_t v) {
 }
 
 // ------------------------------------------------------------------------------------
+// 0. what a level starts from, in one launch: nothing placed, empty blocks, zero counters; the
+//    centroid columns that pad the last stage of operand tiles are zeros that take no items.
+//    n_live != NULL: tree t holds n_live[t] <= n_c items, the first ones of its rows; the items
+//    it does not hold count as placed from the start (no phase ever touches them), and it uses
+//    its first ceil(n_t / bf) centroids only: the others count as full.
+// ------------------------------------------------------------------------------------
+__global__ void k_level_init(int n_c, int K, int bf, int D, int Kt, const int32_t* n_live,
+                             int32_t* placed, int32_t* fill, int32_t* slots, int32_t* counts,
+                             int32_t* done, int32_t* list_count /* (2, T) */, uint4* tiles,
+                             float* cn2) {
+    const int t = blockIdx.y, T = gridDim.y;
+    const int n_t = n_live ? min(max(n_live[t], 0), n_c) : n_c;
+    const int K_t = n_live ? max((n_t + bf - 1) / bf, 1) : K;
+    const int stride = gridDim.x * blockDim.x;
+    const int i0 = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i0 == 0) {
+        done[t] = 0;
+        list_count[t] = 0;
+        list_count[T + t] = 0;
+    }
+    for (int i = i0; i < n_c; i += stride) placed[(size_t)t * n_c + i] = i >= n_t ? 1 : 0;
+    for (int i = i0; i < K; i += stride) {
+        fill[(size_t)t * K + i] = i >= K_t ? bf : 0;
+        counts[(size_t)t * K + i] = 0;
+    }
+    for (size_t i = i0; i < (size_t)K * bf; i += stride) slots[(size_t)t * K * bf + i] = -1;
+    if (tiles != nullptr) {
+        const int pad = Kt * 16 - K, cpc = D / 4;  // chunks of a column: hi and lo halves
+        const int KS = D / 32;
+        for (int i = i0; i < pad * cpc; i += stride) {
+            const int k = K + i / cpc, c = i % cpc;
+            const int half = c / (D / 8), j = c % (D / 8);
+            tiles[((size_t)t * Kt + (k >> 4)) * (size_t)(2 * KS * 64) + half * KS * 64 + (j >> 2) * 64 +
+                  (j & 3) * 16 + (k & 15)] = make_uint4(0, 0, 0, 0);
+        }
+        for (int i = i0; i < pad; i += stride) cn2[(size_t)t * Kt * 16 + K + i] = INFINITY;
+    }
+}
+
+// ------------------------------------------------------------------------------------
 // 1. initial centroids: item floor((k + u_k) * n_c / K), u_k in [0,1) from the seed
 // ------------------------------------------------------------------------------------
 //    (n_live != NULL: tree t holds n_live[t] <= n_c items, the first ones of its rows)
+//    tiles != NULL: the centroid also goes into its operand tile (fill: the centroids that
+//    count as full from the start take no items)
 template <typename T>
-__global__ void k_init_centroids(const void* x, int n_c, size_t x_tree_stride, int K, int D,
-                                 uint64_t seed, float* cent, const int32_t* n_live, int bf) {
+__global__ __launch_bounds__(64) void k_init_centroids(const void* x, int n_c, size_t x_tree_stride,
+                                                       int K, int D, uint64_t seed, float* cent,
+                                                       const int32_t* n_live, int bf, int Kt,
+                                                       const int32_t* fill, uint4* tiles,
+                                                       float* cn2) {
+    __shared__ float s_c[256];
     const int k = blockIdx.x, t = blockIdx.y;
     const uint64_t h = mix64(seed ^ mix64((uint64_t)t * 0x100000001b3ull + (uint64_t)k));
     const double u = (double)(h >> 11) * (1.0 / 9007199254740992.0);
@@ -54,7 +101,15 @@ __global__ void k_init_centroids(const void* x, int n_c, size_t x_tree_stride, i
     if (idx >= n_t) idx = n_t - 1;
     const size_t src = ((size_t)t * x_tree_stride + (size_t)idx) * D;
     float* dst = cent + ((size_t)t * K + k) * D;
-    for (int j = threadIdx.x; j < D; j += blockDim.x) dst[j] = load_elem<T>(x, src + j);
+    for (int j = threadIdx.x; j < D; j += blockDim.x) {
+        const float v = load_elem<T>(x, src + j);
+        dst[j] = v;
+        if (tiles != nullptr) s_c[j] = v;  // (the matrix-core path has D <= 256)
+    }
+    if (tiles != nullptr) {
+        __syncthreads();
+        emit_centroid(s_c, D, Kt, t, k, fill[(size_t)t * K + k] < bf, tiles, cn2);
+    }
 }
 
 // ------------------------------------------------------------------------------------
@@ -62,6 +117,7 @@ __global__ void k_init_centroids(const void* x, int n_c, size_t x_tree_stride, i
 //    LPR lanes hold one item row; each lane group keeps PPG items in registers and walks
 //    all centroids.  fill != NULL: centroids with fill[k] >= bf are skipped.
 //    list != NULL: only the items list[0 .. *list_count) are processed.
+//    ac: the items a centroid takes are counted as they are assigned (assign.h).
 // ------------------------------------------------------------------------------------
 constexpr int kPPG = 4;
 
@@ -69,7 +125,7 @@ template <typename T, int LPR>
 __global__ __launch_bounds__(256) void k_assign_simple(
     const void* x, int n_c, size_t x_tree_stride, const float* cent, int K, int D,
     const int32_t* fill, int bf, const int32_t* list, const int32_t* list_count, size_t list_stride,
-    int32_t* assign, float* dist) {
+    int32_t* assign, float* dist, AssignCounting ac) {
     constexpr int EPL = Elem<T>::kPerChunk;
     constexpr int RPW = kWave / LPR;
     const int lane = lane_id();
@@ -78,234 +134,291 @@ __global__ __launch_bounds__(256) void k_assign_simple(
     const int n_items = list ? list_count[t] : n_c;
     const int wave_global = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     const int first = wave_global * (RPW * kPPG);
-    if (first >= n_items) return;
+    if (ac.counts == nullptr && first >= n_items) return;
+    if (ac.zero != nullptr && blockIdx.x == 0 && threadIdx.x == 0) ac.zero[t] = 0;
     const bool chunk_ok = ch * EPL < D;
 
-    int item[kPPG];
-    float xf[kPPG][EPL];
-    float best[kPPG];
-    int arg[kPPG];
-#pragma unroll
-    for (int p = 0; p < kPPG; ++p) {
-        const int pos = first + p * RPW + rg;
-        item[p] = -1;
-        if (pos < n_items) item[p] = list ? list[(size_t)t * list_stride + pos] : pos;
-        uint4 raw = make_uint4(0, 0, 0, 0);
-        if (item[p] >= 0 && chunk_ok)
-            raw = load_chunk<T>(x, ((size_t)t * x_tree_stride + item[p]) * D, ch);
-        unpack<T>(raw, xf[p]);
-        best[p] = INFINITY;
-        arg[p] = -1;
-    }
-    const float* ct = cent + (size_t)t * K * D;
-    const int32_t* ft = fill ? fill + (size_t)t * K : nullptr;
-    for (int k = 0; k < K; ++k) {
-        if (ft && ft[k] >= bf) continue;  // wave-uniform
-        float cf[4] = {0.f, 0.f, 0.f, 0.f};
-        float cf2[4] = {0.f, 0.f, 0.f, 0.f};
-        if (chunk_ok) {
-            const float4 a = *reinterpret_cast<const float4*>(ct + (size_t)k * D + ch * EPL);
-            cf[0] = a.x, cf[1] = a.y, cf[2] = a.z, cf[3] = a.w;
-            if (EPL == 8) {
-                const float4 b =
-                    *reinterpret_cast<const float4*>(ct + (size_t)k * D + ch * EPL + 4);
-                cf2[0] = b.x, cf2[1] = b.y, cf2[2] = b.z, cf2[3] = b.w;
-            }
-        }
+    if (first < n_items) {  // (wave-uniform; no barrier inside)
+        int item[kPPG];
+        float xf[kPPG][EPL];
+        float best[kPPG];
+        int arg[kPPG];
 #pragma unroll
         for (int p = 0; p < kPPG; ++p) {
-            float ss = 0.0f;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float df = xf[p][e] - cf[e];
-                ss += df * df;
+            const int pos = first + p * RPW + rg;
+            item[p] = -1;
+            if (pos < n_items) item[p] = list ? list[(size_t)t * list_stride + pos] : pos;
+            uint4 raw = make_uint4(0, 0, 0, 0);
+            if (item[p] >= 0 && chunk_ok)
+                raw = load_chunk<T>(x, ((size_t)t * x_tree_stride + item[p]) * D, ch);
+            unpack<T>(raw, xf[p]);
+            best[p] = INFINITY;
+            arg[p] = -1;
+        }
+        const float* ct = cent + (size_t)t * K * D;
+        const int32_t* ft = fill ? fill + (size_t)t * K : nullptr;
+        for (int k = 0; k < K; ++k) {
+            if (ft && ft[k] >= bf) continue;  // wave-uniform
+            float cf[4] = {0.f, 0.f, 0.f, 0.f};
+            float cf2[4] = {0.f, 0.f, 0.f, 0.f};
+            if (chunk_ok) {
+                const float4 a = *reinterpret_cast<const float4*>(ct + (size_t)k * D + ch * EPL);
+                cf[0] = a.x, cf[1] = a.y, cf[2] = a.z, cf[3] = a.w;
+                if (EPL == 8) {
+                    const float4 b =
+                        *reinterpret_cast<const float4*>(ct + (size_t)k * D + ch * EPL + 4);
+                    cf2[0] = b.x, cf2[1] = b.y, cf2[2] = b.z, cf2[3] = b.w;
+                }
             }
-            if (EPL == 8) {
+#pragma unroll
+            for (int p = 0; p < kPPG; ++p) {
+                float ss = 0.0f;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const float df = xf[p][4 + e] - cf2[e];
+                    const float df = xf[p][e] - cf[e];
                     ss += df * df;
                 }
-            }
-            ss = group_sum<LPR>(ss);
-            if (ss < best[p]) {
-                best[p] = ss;
-                arg[p] = k;
-            }
-        }
-    }
-    if (ch == 0) {
+                if (EPL == 8) {
 #pragma unroll
-        for (int p = 0; p < kPPG; ++p) {
-            if (item[p] >= 0) {
-                assign[(size_t)t * n_c + item[p]] = arg[p];
-                dist[(size_t)t * n_c + item[p]] = best[p];
+                    for (int e = 0; e < 4; ++e) {
+                        const float df = xf[p][4 + e] - cf2[e];
+                        ss += df * df;
+                    }
+                }
+                ss = group_sum<LPR>(ss);
+                if (ss < best[p]) {
+                    best[p] = ss;
+                    arg[p] = k;
+                }
+            }
+        }
+        if (ch == 0) {
+#pragma unroll
+            for (int p = 0; p < kPPG; ++p) {
+                if (item[p] >= 0) {
+                    assign[(size_t)t * n_c + item[p]] = arg[p];
+                    dist[(size_t)t * n_c + item[p]] = best[p];
+                    if (ac.counts != nullptr && arg[p] >= 0)
+                        ac.pos[(size_t)t * n_c + item[p]] =
+                            atomicAdd(&ac.counts[(size_t)t * K + arg[p]], 1);
+                }
             }
         }
     }
+    if (ac.counts != nullptr) finish_counts(ac, t, K, (int)gridDim.x);
 }
 
 // ------------------------------------------------------------------------------------
-// 3. bucket the processed items by assigned centroid, each bucket sorted by (dist, item)
+// 3. the items of a round bucketed by the centroid they were assigned to: item i of bucket a
+//    goes to members[offsets[a] + pos[i]] (offsets and pos come out of the assignment launch)
 // ------------------------------------------------------------------------------------
-__global__ void k_bucket_count(const int32_t* assign, int n_c, const int32_t* list,
-                               const int32_t* list_count, size_t list_stride, int K,
-                               int32_t* counts) {
+__global__ void k_bucket_fill(const int32_t* assign, const int32_t* pos, const int32_t* offsets,
+                              int n_c, const int32_t* list, const int32_t* list_count,
+                              size_t list_stride, int K, int32_t* members) {
     const int t = blockIdx.y;
     const int n_items = list ? list_count[t] : n_c;
-    const int pos = blockIdx.x * blockDim.x + threadIdx.x;
-    if (pos >= n_items) return;
-    const int i = list ? list[(size_t)t * list_stride + pos] : pos;
-    const int a = assign[(size_t)t * n_c + i];
-    if (a >= 0) atomicAdd(&counts[(size_t)t * K + a], 1);
-}
-
-// exclusive scan of counts (K entries) per tree -> offsets (K+1 entries); cursor := offsets
-__global__ __launch_bounds__(256) void k_scan(const int32_t* counts, int K, int32_t* offsets,
-                                              int32_t* cursor) {
-    __shared__ int32_t wsum[4];
-    __shared__ int32_t carry;
-    const int t = blockIdx.x;
-    const int lane = lane_id(), wave = threadIdx.x >> 6;
-    if (threadIdx.x == 0) carry = 0;
-    __syncthreads();
-    for (int base = 0; base < K; base += 256) {
-        const int k = base + threadIdx.x;
-        const int v = k < K ? counts[(size_t)t * K + k] : 0;
-        int inc = v;  // inclusive scan in the wave
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const int o = __shfl_up(inc, off, 64);
-            if (lane >= off) inc += o;
-        }
-        if (lane == 63) wsum[wave] = inc;
-        __syncthreads();
-        int before = carry;
-        for (int w = 0; w < wave; ++w) before += wsum[w];
-        const int excl = before + inc - v;
-        if (k < K) {
-            offsets[(size_t)t * (K + 1) + k] = excl;
-            cursor[(size_t)t * K + k] = excl;
-        }
-        __syncthreads();
-        if (threadIdx.x == 255) carry = excl + v;
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) offsets[(size_t)t * (K + 1) + K] = carry;
-}
-
-__global__ void k_bucket_fill(const int32_t* assign, int n_c, const int32_t* list,
-                              const int32_t* list_count, size_t list_stride, int K,
-                              int32_t* cursor, int32_t* members) {
-    const int t = blockIdx.y;
-    const int n_items = list ? list_count[t] : n_c;
-    const int pos = blockIdx.x * blockDim.x + threadIdx.x;
-    if (pos >= n_items) return;
-    const int i = list ? list[(size_t)t * list_stride + pos] : pos;
+    const int p = blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= n_items) return;
+    const int i = list ? list[(size_t)t * list_stride + p] : p;
     const int a = assign[(size_t)t * n_c + i];
     if (a < 0) return;
-    const int at = atomicAdd(&cursor[(size_t)t * K + a], 1);
-    members[(size_t)t * n_c + at] = i;
+    members[(size_t)t * n_c + offsets[(size_t)t * (K + 1) + a] + pos[(size_t)t * n_c + i]] = i;
 }
 
-// one workgroup per bucket: rank every member by (dist, item id) and write it to its rank (four
-// waves: nearest-centroid buckets of seeds drawn from the keys are very uneven in 128 dimensions,
-// and a bucket of m members costs m * m / threads comparisons)
-constexpr int kSortTile = 1024;
-constexpr int kSortThreads = 256;
-__global__ __launch_bounds__(kSortThreads) void k_bucket_sort(const int32_t* members,
-                                                              const int32_t* offsets,
-                                                              const float* dist, int n_c, int K,
-                                                              int32_t* sorted) {
-    __shared__ uint64_t keys[kSortTile];
-    const int k = blockIdx.x, t = blockIdx.y;
-    const int tid = threadIdx.x;
-    const int b0 = offsets[(size_t)t * (K + 1) + k], b1 = offsets[(size_t)t * (K + 1) + k + 1];
-    const int m = b1 - b0;
+// The order in which a bucket's members arrive depends on the run; everything that follows works
+// on them in a fixed order, which a workgroup per bucket establishes in LDS:
+//   up to 256 members   every thread ranks its member against all others
+//   more                a bitonic sorting network over the next power of two
+constexpr int kBucketThreads = 256;
+
+template <typename Key>
+__device__ __forceinline__ void bitonic_sort(Key* a, int P) {  // (a barrier ahead of the first step)
+    for (int k = 2; k <= P; k <<= 1)
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            __syncthreads();
+            for (int i = threadIdx.x; i < P; i += kBucketThreads) {
+                const int x = i ^ j;
+                if (x > i) {
+                    const Key u = a[i], v = a[x];
+                    if ((u > v) == ((i & k) == 0)) {
+                        a[i] = v;
+                        a[x] = u;
+                    }
+                }
+            }
+        }
+    __syncthreads();
+}
+
+__device__ __forceinline__ int pow2_at_least(int n) {
+    int p = 1;
+    while (p < n) p <<= 1;
+    return p;
+}
+
+// (what every workgroup of the per-bucket kernels does for the round after it)
+__device__ __forceinline__ void reset_counters(int t, int k, int K, int32_t* counts, int32_t* done) {
+    if (threadIdx.x == 0) {
+        counts[(size_t)t * K + k] = 0;
+        if (k == 0) done[t] = 0;
+    }
+}
+
+// ------------------------------------------------------------------------------------
+// 4. Lloyd round: centroid = mean of the member rows.  One workgroup per centroid: the members
+//    in the order of their item ids, row e summed by row group e % R, the R sums added in order:
+//    the result does not depend on the order of arrival.  An empty centroid keeps its value.
+//    tiles != NULL: the new centroid also goes into its operand tile.
+// ------------------------------------------------------------------------------------
+constexpr int kMeanSort = 4096;      // members ordered in LDS; more: through a bit map of item ids
+constexpr int kMeanMapBits = kMeanSort * 32;
+
+template <typename T>
+__global__ __launch_bounds__(kBucketThreads) void k_bucket_mean(
+    const void* x, size_t x_tree_stride, int n_c, int K, int D, const int32_t* offsets,
+    const int32_t* members, int32_t* ordered /* (T, n_c): buckets too large for LDS */,
+    const int32_t* fill, int bf, float* cent, int Kt, uint4* tiles, float* cn2, int32_t* counts,
+    int32_t* done) {
+    constexpr int EPL = Elem<T>::kPerChunk;
+    __shared__ uint32_t s_ord[kMeanSort];            // (as a bit map: kMeanMapBits ids)
+    __shared__ float s_part[kBucketThreads * EPL];   // (R, D) partial sums, R * D <= 256 * EPL
+    __shared__ int32_t s_small[kBucketThreads];
+    const int k = blockIdx.x, t = blockIdx.y, tid = threadIdx.x;
+    reset_counters(t, k, K, counts, done);
+    const int b0 = offsets[(size_t)t * (K + 1) + k];
+    const int m = offsets[(size_t)t * (K + 1) + k + 1] - b0;
     if (m <= 0) return;
     const int32_t* mem = members + (size_t)t * n_c + b0;
-    const float* dt = dist + (size_t)t * n_c;
-    for (int e0 = 0; e0 < m; e0 += kSortThreads) {
-        const int e = e0 + tid;
-        uint64_t mykey = 0;
-        int myitem = -1;
-        if (e < m) {
-            myitem = mem[e];
-            mykey = ((uint64_t)__float_as_uint(dt[myitem]) << 32) | (uint32_t)myitem;
-        }
+    const int32_t* ord_g = nullptr;  // the ordered members: in LDS, or here
+    if (m <= kBucketThreads) {
+        const int mine = tid < m ? mem[tid] : 0x7fffffff;
+        s_small[tid] = mine;
+        __syncthreads();
         int rank = 0;
-        for (int tile = 0; tile < m; tile += kSortTile) {
-            const int tn = min(kSortTile, m - tile);
+        for (int j = 0; j < m; ++j) rank += s_small[j] < mine;
+        if (tid < m) s_ord[rank] = (uint32_t)mine;
+        __syncthreads();
+    } else if (m <= kMeanSort) {
+        const int P = pow2_at_least(m);
+        for (int e = tid; e < P; e += kBucketThreads) s_ord[e] = e < m ? (uint32_t)mem[e] : 0xffffffffu;
+        bitonic_sort(s_ord, P);
+    } else {
+        // ids in ranges of kMeanMapBits: a bit per member, then the set bits in order
+        int32_t* out = ordered + (size_t)t * n_c + b0;
+        int written = 0;
+        for (int lo = 0; lo < n_c; lo += kMeanMapBits) {
             __syncthreads();
-            for (int j = tid; j < tn; j += kSortThreads) {
-                const int it = mem[tile + j];
-                keys[j] = ((uint64_t)__float_as_uint(dt[it]) << 32) | (uint32_t)it;
+            for (int w = tid; w < kMeanSort; w += kBucketThreads) s_ord[w] = 0;
+            __syncthreads();
+            for (int e = tid; e < m; e += kBucketThreads) {
+                const int d = mem[e] - lo;
+                if (d >= 0 && d < kMeanMapBits) atomicOr(&s_ord[d >> 5], 1u << (d & 31));
             }
             __syncthreads();
-            if (e < m)
-                for (int j = 0; j < tn; ++j) rank += keys[j] < mykey;
+            // thread `tid` owns the words [tid * W, (tid + 1) * W)
+            constexpr int W = kMeanSort / kBucketThreads;
+            const int in_range = block_exclusive_scan(
+                kBucketThreads, [&](int i) {
+                    int c = 0;
+                    for (int w = 0; w < W; ++w) c += __popc(s_ord[i * W + w]);
+                    return c;
+                },
+                [&](int i, int v) { s_small[i] = v; });
+            __syncthreads();
+            int at = written + s_small[tid];
+            for (int w = 0; w < W; ++w) {
+                uint32_t bits = s_ord[tid * W + w];
+                while (bits) {
+                    const int b = __ffs(bits) - 1;
+                    bits &= bits - 1;
+                    out[at++] = lo + (tid * W + w) * 32 + b;
+                }
+            }
+            written += in_range;
         }
-        if (e < m) sorted[(size_t)t * n_c + b0 + rank] = myitem;
+        __threadfence_block();
+        __syncthreads();
+        ord_g = out;
+    }
+    // ---- sums: CPR threads a row, R rows at a time -------------------------------------------
+    const int CPR = D / EPL, R = kBucketThreads / CPR;
+    const int r = tid / CPR, c = tid % CPR;
+    float acc[EPL];
+#pragma unroll
+    for (int e = 0; e < EPL; ++e) acc[e] = 0.0f;
+    if (r < R) {
+        for (int e = r; e < m; e += R) {
+            const int it = ord_g ? ord_g[e] : (int)s_ord[e];
+            float f[EPL];
+            unpack<T>(load_chunk<T>(x, ((size_t)t * x_tree_stride + it) * D, c), f);
+#pragma unroll
+            for (int q = 0; q < EPL; ++q) acc[q] += f[q];
+        }
+#pragma unroll
+        for (int q = 0; q < EPL; ++q) s_part[r * D + c * EPL + q] = acc[q];
+    }
+    __syncthreads();
+    float v = 0.0f;
+    for (int j = tid; j < D; j += kBucketThreads) {  // (D <= 512: at most two columns a thread)
+        float s = 0.0f;
+        const int rows = min(R, m);
+        for (int q = 0; q < rows; ++q) s += s_part[q * D + j];
+        v = s / (float)m;
+        cent[((size_t)t * K + k) * D + j] = v;
+    }
+    if (tiles != nullptr) {  // (D <= 256: column tid)
+        __syncthreads();
+        if (tid < D) s_part[tid] = v;
+        __syncthreads();
+        if (tid < 64)
+            emit_centroid(s_part, D, Kt, t, k, !(fill != nullptr && fill[(size_t)t * K + k] >= bf),
+                          tiles, cn2);
     }
 }
 
-// ------------------------------------------------------------------------------------
-// 4. centroid = mean of the member rows, summed in list order.  One wave per centroid.
-//    Lists: CSR (offsets/members) when slots == NULL, else the bf slots of the block.
-//    An empty centroid keeps its value.  out_t != NULL: also store rounded to T.
-// ------------------------------------------------------------------------------------
+// block centre = mean of the items in the bf slots of the block, stored in fp32 and rounded to the
+// storage type.  One wave per block: `lpr` lanes (a power of two) hold a row in 16-byte chunks,
+// the 64 / lpr lane groups take every (64 / lpr)-th slot, and their sums are added pairwise in a
+// fixed order.  An empty block keeps its value.
 template <typename T>
-__global__ __launch_bounds__(256) void k_mean(const void* x, size_t x_tree_stride, int n_c, int K,
-                                              int D, const int32_t* offsets,
-                                              const int32_t* members, const int32_t* slots, int bf,
-                                              float* cent, void* out_t) {
-    // launched with one wave (the sums then run in list order) or four (wave w sums members
-    // w, w + 4, ..., the four sums are added in wave order: large buckets, still reproducible)
-    __shared__ float s_part[3][64];
-    __shared__ int s_cnt[3];
+__global__ __launch_bounds__(64) void k_block_mean(const void* x, size_t x_tree_stride, int K,
+                                                   int D, const int32_t* slots, int bf, int lpr,
+                                                   float* cent, void* out_t) {
+    constexpr int EPL = Elem<T>::kPerChunk;
     const int k = blockIdx.x, t = blockIdx.y;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
-    const int32_t* lst;
-    int m;
-    if (slots) {
-        lst = slots + ((size_t)t * K + k) * bf;
-        m = bf;
-    } else {
-        const int b0 = offsets[(size_t)t * (K + 1) + k];
-        m = offsets[(size_t)t * (K + 1) + k + 1] - b0;
-        lst = members + (size_t)t * n_c + b0;
+    const int lane = threadIdx.x;
+    const int rg = lane / lpr, ch = lane % lpr, groups = 64 / lpr;
+    const bool chunk_ok = ch * EPL < D;
+    const int32_t* lst = slots + ((size_t)t * K + k) * bf;
+    float acc[EPL];
+#pragma unroll
+    for (int q = 0; q < EPL; ++q) acc[q] = 0.0f;
+    int cnt = 0;
+    for (int e = rg; e < bf; e += groups) {
+        const int it = lst[e];
+        if (it < 0) continue;
+        ++cnt;
+        if (!chunk_ok) continue;
+        float f[EPL];
+        unpack<T>(load_chunk<T>(x, ((size_t)t * x_tree_stride + it) * D, ch), f);
+#pragma unroll
+        for (int q = 0; q < EPL; ++q) acc[q] += f[q];
     }
-    for (int j0 = 0; j0 < D; j0 += 64) {
-        const int j = j0 + lane;
-        float s = 0.0f;
-        int cnt = 0;
-        for (int e = wave; e < m; e += nw) {
-            const int it = lst[e];
-            if (it < 0) continue;
-            ++cnt;
-            if (j < D) s += load_elem<T>(x, ((size_t)t * x_tree_stride + it) * D + j);
-        }
-        if (nw > 1) {  // uniform
-            __syncthreads();
-            if (wave > 0) {
-                s_part[wave - 1][lane] = s;
-                if (lane == 0) s_cnt[wave - 1] = cnt;
-            }
-            __syncthreads();
-            if (wave == 0)
-                for (int w = 1; w < nw; ++w) {
-                    s += s_part[w - 1][lane];
-                    cnt += s_cnt[w - 1];
-                }
-        }
-        if (wave == 0 && j < D) {
-            const size_t o = ((size_t)t * K + k) * D + j;
+    for (int off = lpr; off < 64; off <<= 1) {
+        cnt += __shfl_xor(cnt, off, 64);
+#pragma unroll
+        for (int q = 0; q < EPL; ++q) acc[q] += __shfl_xor(acc[q], off, 64);
+    }
+    if (rg == 0 && chunk_ok) {
+#pragma unroll
+        for (int q = 0; q < EPL; ++q) {
+            const size_t o = ((size_t)t * K + k) * D + ch * EPL + q;
             float v = cent[o];
             if (cnt > 0) {
-                v = s / (float)cnt;
+                v = acc[q] / (float)cnt;
                 cent[o] = v;
             }
-            if (out_t) store_elem<T>(out_t, o, v);
+            store_elem<T>(out_t, o, v);
         }
     }
 }
@@ -313,35 +426,82 @@ __global__ __launch_bounds__(256) void k_mean(const void* x, size_t x_tree_strid
 // ------------------------------------------------------------------------------------
 // 5. capacity packing
 // ------------------------------------------------------------------------------------
-// one wave per bucket: the closest proposers take the free slots of the block
-__global__ __launch_bounds__(64) void k_accept(const int32_t* sorted, const int32_t* offsets,
-                                               int n_c, int K, int bf, int32_t* fill,
-                                               int32_t* slots, int32_t* placed) {
-    const int k = blockIdx.x, t = blockIdx.y;
-    const int lane = threadIdx.x;
+// One workgroup per bucket: the closest proposers (by distance, then item id) take the free
+// slots of the block in that order; the others go on the list of the next round.  A block that
+// is full now takes no more items: its norm in the operand tiles becomes +inf.
+constexpr int kAcceptSort = 2048;  // keys sorted at a time; larger buckets in several goes, the
+                                   // best `take` so far carried along
+
+__global__ __launch_bounds__(kBucketThreads) void k_bucket_accept(
+    const int32_t* members, const int32_t* offsets, const float* dist, int n_c, int K, int bf,
+    int32_t* fill, int32_t* slots, int32_t* placed, int32_t* next_list, int32_t* next_count,
+    int Kt, float* cn2, int32_t* counts, int32_t* done) {
+    __shared__ uint64_t s_keys[kAcceptSort];
+    __shared__ int32_t s_base, s_rej;
+    const int k = blockIdx.x, t = blockIdx.y, tid = threadIdx.x;
+    reset_counters(t, k, K, counts, done);
     const int b0 = offsets[(size_t)t * (K + 1) + k];
     const int m = offsets[(size_t)t * (K + 1) + k + 1] - b0;
     if (m <= 0) return;
+    const int32_t* mem = members + (size_t)t * n_c + b0;
+    const float* dt = dist + (size_t)t * n_c;
     const int f = fill[(size_t)t * K + k];
-    const int take = min(m, bf - f);
-    for (int r = lane; r < take; r += 64) {
-        const int it = sorted[(size_t)t * n_c + b0 + r];
-        slots[((size_t)t * K + k) * bf + f + r] = it;
-        placed[(size_t)t * n_c + it] = 1;
+    const int take = max(min(m, bf - f), 0);
+    int32_t* my_slots = slots + ((size_t)t * K + k) * bf + f;
+    int32_t* pl = placed + (size_t)t * n_c;
+    int32_t* nl = next_list + (size_t)t * n_c;
+    __syncthreads();  // (every thread has read the block's fill)
+    if (tid == 0) {
+        s_base = m > take ? atomicAdd(&next_count[t], m - take) : 0;
+        s_rej = 0;
+        fill[(size_t)t * K + k] = f + take;
+        if (cn2 != nullptr && f + take >= bf) cn2[(size_t)t * Kt * 16 + k] = INFINITY;
     }
-    __syncthreads();
-    if (lane == 0) fill[(size_t)t * K + k] = f + take;
-}
-
-// items a tree does not hold count as placed from the start: no phase ever touches them; and
-// a tree with n_t items uses its first ceil(n_t / bf) centroids only: the others count as full
-__global__ void k_mark_absent(const int32_t* n_live, int n_c, int K, int bf, int32_t* placed,
-                              int32_t* fill) {
-    const int t = blockIdx.y;
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    const int n_t = min(max(n_live[t], 0), n_c);
-    if (i < n_c) placed[(size_t)t * n_c + i] = i >= n_t ? 1 : 0;
-    if (i < K) fill[(size_t)t * K + i] = i >= max((n_t + bf - 1) / bf, 1) ? bf : 0;
+    auto key_of = [&](int it) { return ((uint64_t)__float_as_uint(dt[it]) << 32) | (uint32_t)it; };
+    if (m <= kBucketThreads) {
+        int it = -1;
+        uint64_t mine = ~0ull;
+        if (tid < m) {
+            it = mem[tid];
+            mine = key_of(it);
+        }
+        s_keys[tid] = mine;
+        __syncthreads();
+        int rank = 0;
+        for (int j = 0; j < m; ++j) rank += s_keys[j] < mine;
+        if (tid < m) {
+            if (rank < take) {
+                my_slots[rank] = it;
+                pl[it] = 1;
+            } else {
+                nl[s_base + rank - take] = it;
+            }
+        }
+        return;
+    }
+    int kept = 0;  // s_keys[0 .. kept): the best so far, in order
+    for (int e0 = 0; e0 < m;) {
+        const int cn = min(kAcceptSort - kept, m - e0);
+        const int P = pow2_at_least(kept + cn);
+        __syncthreads();
+        for (int e = kept + tid; e < P; e += kBucketThreads)
+            s_keys[e] = e < kept + cn ? key_of(mem[e0 + e - kept]) : ~0ull;
+        bitonic_sort(s_keys, P);
+        kept = min(take, kept + cn);
+        e0 += cn;
+    }
+    for (int r = tid; r < take; r += kBucketThreads) {
+        const int it = (int)(uint32_t)s_keys[r];
+        my_slots[r] = it;
+        pl[it] = 1;
+    }
+    if (m > take) {  // whoever lies behind the last one taken tries again
+        const uint64_t last = take > 0 ? s_keys[take - 1] : 0ull;
+        for (int e = tid; e < m; e += kBucketThreads) {
+            const int it = mem[e];
+            if (take == 0 || key_of(it) > last) nl[s_base + atomicAdd(&s_rej, 1)] = it;
+        }
+    }
 }
 
 // (one atomic per workgroup of 256 items, not per wave: the tree's counter is one address)
@@ -367,77 +527,69 @@ __global__ __launch_bounds__(256) void k_collect_unplaced(const int32_t* placed,
 }
 
 // Whatever is still unplaced goes to the free slots in order: the u-th unplaced item (by
-// item id) takes the u-th free slot (by block, then slot).  One workgroup per tree.
-constexpr int kLeftThreads = 1024;  // (the walk over a tree's items is serial in steps of this many)
-__global__ __launch_bounds__(kLeftThreads) void k_leftover(int n_c, int K, int bf, int32_t* fill,
-                                                  int32_t* slots, int32_t* placed,
-                                                  int32_t* scratch /* (T, K+1) */) {
-    __shared__ int32_t wsum[kLeftThreads / 64];
-    __shared__ int32_t carry;
-    const int t = blockIdx.x;
-    const int lane = lane_id(), wave = threadIdx.x >> 6;
-    int32_t* freepre = scratch + (size_t)t * (K + 1);  // exclusive prefix of free slots
-    if (threadIdx.x == 0) carry = 0;
+// item id) takes the u-th free slot (by block, then slot).  Two launches: the unplaced items of
+// every 256 are counted, and the tree's last workgroup turns the counts, and the free slots
+// of the blocks, into prefix sums; then every item finds its slot by itself.
+__global__ __launch_bounds__(256) void k_leftover_count(const int32_t* placed, int n_c, int K,
+                                                        int bf, const int32_t* fill,
+                                                        int32_t* chunk_pre /* (T, chunks + 1) */,
+                                                        int32_t* free_pre /* (T, K + 1) */,
+                                                        int32_t* done) {
+    __shared__ int32_t s_cnt[4];
+    __shared__ int32_t s_last;
+    const int t = blockIdx.y, nb = gridDim.x;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    const bool mine = i < n_c && placed[(size_t)t * n_c + i] == 0;
+    const unsigned long long bal = __ballot(mine);
+    if (lane_id() == 0) s_cnt[threadIdx.x >> 6] = __popcll(bal);
     __syncthreads();
-    for (int base = 0; base < K; base += kLeftThreads) {
-        const int k = base + threadIdx.x;
-        const int v = k < K ? bf - fill[(size_t)t * K + k] : 0;
-        int inc = v;
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const int o = __shfl_up(inc, off, 64);
-            if (lane >= off) inc += o;
-        }
-        if (lane == 63) wsum[wave] = inc;
-        __syncthreads();
-        int before = carry;
-        for (int w = 0; w < wave; ++w) before += wsum[w];
-        if (k < K) freepre[k] = before + inc - v;
-        __syncthreads();
-        if (threadIdx.x == kLeftThreads - 1) carry = before + inc;
-        __syncthreads();
-    }
+    int32_t* cp = chunk_pre + (size_t)t * (nb + 1);
     if (threadIdx.x == 0) {
-        freepre[K] = carry;
-        carry = 0;
+        __hip_atomic_store(&cp[blockIdx.x], s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3],
+                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        hand_off_release();  // (the count is where every workgroup sees it before the ticket)
+        s_last = atomicAdd(&done[t], 1) == nb - 1 ? 1 : 0;
     }
     __syncthreads();
-    for (int base = 0; base < n_c; base += kLeftThreads) {
-        const int i = base + threadIdx.x;
-        const int v = (i < n_c && placed[(size_t)t * n_c + i] == 0) ? 1 : 0;
-        int inc = v;
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const int o = __shfl_up(inc, off, 64);
-            if (lane >= off) inc += o;
-        }
-        if (lane == 63) wsum[wave] = inc;
-        __syncthreads();
-        int before = carry;
-        for (int w = 0; w < wave; ++w) before += wsum[w];
-        if (v) {
-            const int u = before + inc - 1;  // rank among the unplaced
-            // block k with freepre[k] <= u < freepre[k+1]
-            int lo = 0, hi = K;
-            while (hi - lo > 1) {
-                const int mid = (lo + hi) >> 1;
-                if (freepre[mid] <= u) lo = mid; else hi = mid;
-            }
-            const int j = fill[(size_t)t * K + lo] + (u - freepre[lo]);
-            slots[((size_t)t * K + lo) * bf + j] = i;
-            placed[(size_t)t * n_c + i] = 1;
-        }
-        __syncthreads();
-        if (threadIdx.x == kLeftThreads - 1) carry = before + inc;
-        __syncthreads();
+    if (!s_last) return;
+    const int unplaced = block_exclusive_scan(
+        nb, [&](int b) { return load_agent(cp + b); }, [&](int b, int v) { cp[b] = v; });
+    int32_t* fp = free_pre + (size_t)t * (K + 1);
+    const int32_t* ft = fill + (size_t)t * K;
+    const int room = block_exclusive_scan(
+        K, [&](int k) { return bf - ft[k]; }, [&](int k, int v) { fp[k] = v; });
+    if (threadIdx.x == 0) {
+        cp[nb] = unplaced;
+        fp[K] = room;
+        done[t] = 0;
     }
+}
+
+__global__ __launch_bounds__(256) void k_leftover_place(int n_c, int K, int bf, const int32_t* fill,
+                                                        const int32_t* chunk_pre,
+                                                        const int32_t* free_pre, int32_t* slots,
+                                                        int32_t* placed) {
+    __shared__ int32_t s_cnt[4];
+    const int t = blockIdx.y, nb = gridDim.x;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    const bool mine = i < n_c && placed[(size_t)t * n_c + i] == 0;
+    const unsigned long long bal = __ballot(mine);
+    const int lane = lane_id(), wave = threadIdx.x >> 6;
+    if (lane == 0) s_cnt[wave] = __popcll(bal);
     __syncthreads();
-    // the blocks are now as full as the items allow
-    for (int k = threadIdx.x; k < K; k += kLeftThreads) {
-        int c = 0;
-        for (int j = 0; j < bf; ++j) c += slots[((size_t)t * K + k) * bf + j] >= 0;
-        fill[(size_t)t * K + k] = c;
+    if (!mine) return;
+    int u = chunk_pre[(size_t)t * (nb + 1) + blockIdx.x] + __popcll(bal & ((1ull << lane) - 1ull));
+    for (int w = 0; w < wave; ++w) u += s_cnt[w];
+    // block k with free_pre[k] <= u < free_pre[k + 1]
+    const int32_t* fp = free_pre + (size_t)t * (K + 1);
+    int lo = 0, hi = K;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (fp[mid] <= u) lo = mid; else hi = mid;
     }
+    const int j = fill[(size_t)t * K + lo] + (u - fp[lo]);
+    slots[((size_t)t * K + lo) * bf + j] = i;
+    placed[(size_t)t * n_c + i] = 1;
 }
 
 // ------------------------------------------------------------------------------------
@@ -495,36 +647,61 @@ __global__ void k_gather_elems(const void* src, size_t src_tree_stride, const in
 }
 
 // counts[p] = children in use; radii[p] = max over them of (||child - centre|| + r_child),
-// -inf when there is none.  One wave per node.
+// -inf when there is none.  One wave per node: `lpr` lanes (a power of two) hold a row in
+// 16-byte chunks (a chunk is contiguous in either layout), 64 / lpr children at a time.
 template <typename T>
 __global__ __launch_bounds__(64) void k_radii(const void* child, size_t child_tree_stride,
                                               const float* child_radii,
                                               size_t child_radii_stride,
                                               const int32_t* child_order, int size_child,
                                               const void* centers, size_t center_tree_stride,
-                                              int size, int bf, int D, int child_layout,
+                                              int size, int bf, int D, int lpr, int child_layout,
                                               int layout, float* radii, int32_t* counts,
                                               size_t out_stride) {
+    constexpr int EPL = Elem<T>::kPerChunk;
     const int p = blockIdx.x, t = blockIdx.y;
     const int lane = threadIdx.x;
+    const int rg = lane / lpr, ch = lane % lpr, groups = 64 / lpr;
+    const bool chunk_ok = ch * EPL < D;
+    float cf[EPL];
+    {
+        uint4 raw = make_uint4(0, 0, 0, 0);
+        if (chunk_ok)
+            raw = *reinterpret_cast<const uint4*>(
+                reinterpret_cast<const T*>(centers) + (size_t)t * center_tree_stride * D +
+                elem_index(layout, D, (size_t)p, ch * EPL));
+        unpack<T>(raw, cf);
+    }
     float r = -INFINITY;
     int c = 0;
-    for (int j = 0; j < bf; ++j) {
+    for (int j0 = 0; j0 < bf; j0 += groups) {  // (uniform trip count: the sums meet in shuffles)
+        const int j = j0 + rg;
         const int s = p * bf + j;
-        if (s >= size_child) break;
-        if (child_order[(size_t)t * size_child + s] < 0) continue;
-        ++c;
+        const bool have = j < bf && s < size_child && child_order[(size_t)t * size_child + s] >= 0;
+        uint4 raw = make_uint4(0, 0, 0, 0);
+        if (have && chunk_ok)
+            raw = *reinterpret_cast<const uint4*>(
+                reinterpret_cast<const T*>(child) + (size_t)t * child_tree_stride * D +
+                elem_index(child_layout, D, (size_t)s, ch * EPL));
+        float f[EPL];
+        unpack<T>(raw, f);
         float ss = 0.0f;
-        for (int e = lane; e < D; e += 64) {
-            const float df =
-                load_elem<T>(child, (size_t)t * child_tree_stride * D + elem_index(child_layout, D, (size_t)s, e)) -
-                load_elem<T>(centers, (size_t)t * center_tree_stride * D + elem_index(layout, D, (size_t)p, e));
+#pragma unroll
+        for (int q = 0; q < EPL; ++q) {
+            const float df = f[q] - cf[q];
             ss += df * df;
         }
-        ss = group_sum<64>(ss);
-        float v = sqrtf(ss);
-        if (child_radii) v += child_radii[(size_t)t * child_radii_stride + s];
-        r = fmaxf(r, v);
+        for (int off = 1; off < lpr; off <<= 1) ss += __shfl_xor(ss, off, 64);
+        if (have) {
+            ++c;
+            float v = sqrtf(ss);
+            if (child_radii) v += child_radii[(size_t)t * child_radii_stride + s];
+            r = fmaxf(r, v);
+        }
+    }
+    for (int off = lpr; off < 64; off <<= 1) {
+        r = fmaxf(r, __shfl_xor(r, off, 64));
+        c += __shfl_xor(c, off, 64);
     }
     if (lane == 0) {
         // a few ulp of head room: the bound must survive fp32 rounding of this sum
@@ -553,9 +730,11 @@ struct BuildWs {
     float* cent_f32;
     void* cent_tiles;  // centroids as bf16 operand tiles (matrix-core assignment), or NULL
     float* cent_n2;
-    int32_t *assign, *placed, *members, *sorted, *list, *list_count;
+    int32_t *assign, *pos, *placed, *members, *ordered;
+    int32_t* list[2];     // the items of a packing round, and those of the round after it
+    int32_t* list_count;  // (2, T)
     float* dist;
-    int32_t *counts, *offsets, *cursor, *fill, *scratch;
+    int32_t *counts, *offsets, *done, *fill, *free_pre, *chunk_pre;
     int32_t* slots[HIRA_MAX_LEVELS];
     void* cent_t[HIRA_MAX_LEVELS];
     int32_t* order[HIRA_MAX_LEVELS];
@@ -563,15 +742,6 @@ struct BuildWs {
 };
 
 static int ceil_div(int a, int b) { return (a + b - 1) / b; }
-
-// assign_mfma.hip
-int assign_tiles(int K);
-int launch_cent_prep(int dim, const float* cent, int K, int num_trees, const int32_t* fill, int bf,
-                     void* tiles, float* cn2, hipStream_t s);
-int launch_assign_mfma(int dim, const void* x, int n_c, size_t x_tree_stride, const void* tiles,
-                       const float* cn2, int K, int num_trees, const int32_t* list,
-                       const int32_t* list_count, size_t list_stride, int32_t* assign, float* dist,
-                       hipStream_t s);
 
 // bf16 rows of 64, 128 or 256 columns are assigned on the matrix cores
 static bool assign_on_mfma(const HiraTree* t) {
@@ -600,17 +770,20 @@ static void carve(const HiraTree* t, int n, void* ws, BuildWs* b) {
         b->cent_n2 = c.take<float>((size_t)T * kpad);
     }
     b->assign = c.take<int32_t>((size_t)T * n);
+    b->pos = c.take<int32_t>((size_t)T * n);
     b->placed = c.take<int32_t>((size_t)T * n);
     b->members = c.take<int32_t>((size_t)T * n);
-    b->sorted = c.take<int32_t>((size_t)T * n);
-    b->list = c.take<int32_t>((size_t)T * n);
-    b->list_count = c.take<int32_t>((size_t)T);
+    b->ordered = c.take<int32_t>((size_t)T * n);
+    b->list[0] = c.take<int32_t>((size_t)T * n);
+    b->list[1] = c.take<int32_t>((size_t)T * n);
+    b->list_count = c.take<int32_t>((size_t)T * 2);
     b->dist = c.take<float>((size_t)T * n);
     b->counts = c.take<int32_t>((size_t)T * k1);
     b->offsets = c.take<int32_t>((size_t)T * (k1 + 1));
-    b->cursor = c.take<int32_t>((size_t)T * k1);
+    b->done = c.take<int32_t>((size_t)T);
     b->fill = c.take<int32_t>((size_t)T * k1);
-    b->scratch = c.take<int32_t>((size_t)T * (k1 + 1));
+    b->free_pre = c.take<int32_t>((size_t)T * (k1 + 1));
+    b->chunk_pre = c.take<int32_t>((size_t)T * ((size_t)ceil_div(n, 256) + 1));
     for (int l = 0; l < HIRA_MAX_LEVELS; ++l) {
         b->slots[l] = nullptr;
         b->cent_t[l] = nullptr;
@@ -628,11 +801,13 @@ template <typename T>
 static int launch_assign(int lpr, dim3 grid, hipStream_t s, const void* x, int n_c,
                          size_t x_stride, const float* cent, int K, int D, const int32_t* fill,
                          int bf, const int32_t* list, const int32_t* list_count,
-                         size_t list_stride, int32_t* assign, float* dist) {
+                         size_t list_stride, int32_t* assign, float* dist,
+                         const AssignCounting& counting) {
 #define HIRA_ASSIGN_CASE(N)                                                                   \
     case N:                                                                                   \
         hipLaunchKernelGGL((k_assign_simple<T, N>), grid, dim3(256), 0, s, x, n_c, x_stride,   \
-                           cent, K, D, fill, bf, list, list_count, list_stride, assign, dist); \
+                           cent, K, D, fill, bf, list, list_count, list_stride, assign, dist, \
+                           counting);                                                          \
         break;
     switch (lpr) {
         HIRA_ASSIGN_CASE(2)
@@ -664,100 +839,80 @@ static int build_impl(const HiraTree* t, const void* keys_in, const void* values
     int K[HIRA_MAX_LEVELS];
     cluster_counts(n, bf, L, K);
 
+    const bool on_mfma = w.cent_tiles != nullptr;
+    uint4* tiles = reinterpret_cast<uint4*>(w.cent_tiles);
     for (int l = 1; l < L; ++l) {
         const void* x = l == 1 ? keys_in : w.cent_t[l - 1];
         const int n_c = K[l - 1];
         const size_t xs = (size_t)n_c;  // rows per tree in x
         const int Kl = K[l];
+        const int Kt = on_mfma ? assign_tiles(Kl) : 0;
         const int items_per_block = 4 * (64 / lpr) * kPPG;
         const dim3 g_assign(ceil_div(n_c, items_per_block), NT);
         const dim3 g_items(ceil_div(n_c, 256), NT);
         const dim3 g_cent(Kl, NT);
 
-        // Trees with fewer items than rows (n_live): the items a tree does not hold are marked
-        // placed before anything else, and every phase walks the list of the unplaced ones.
+        // Trees with fewer items than rows (n_live): every phase walks the list of the items
+        // the tree holds, and the first packing round does too.
         const bool ragged = n_live != nullptr && l == 1;
+        hipLaunchKernelGGL(k_level_init, dim3(min(ceil_div(max(n_c, Kl * bf), 256), 2048), NT),
+                           dim3(256), 0, s, n_c, Kl, bf, D, Kt, ragged ? n_live : nullptr, w.placed,
+                           w.fill, w.slots[l], w.counts, w.done, w.list_count, tiles, w.cent_n2);
         const int32_t* live = nullptr;
         const int32_t* live_cnt = nullptr;
-        const size_t live_stride = ragged ? (size_t)n_c : 0;
         if (ragged) {
-            hipLaunchKernelGGL(k_mark_absent, dim3(ceil_div(n_c > Kl ? n_c : Kl, 256), NT), dim3(256),
-                               0, s, n_live, n_c, Kl, bf, w.placed, w.fill);
-            fill_i32(w.list_count, (size_t)NT, 0, s);
-            hipLaunchKernelGGL(k_collect_unplaced, g_items, dim3(256), 0, s, w.placed, n_c, w.list,
-                               w.list_count);
-            live = w.list;
+            hipLaunchKernelGGL(k_collect_unplaced, g_items, dim3(256), 0, s, w.placed, n_c,
+                               w.list[0], w.list_count);
+            live = w.list[0];
             live_cnt = w.list_count;
         }
         hipLaunchKernelGGL((k_init_centroids<T>), g_cent, dim3(64), 0, s, x, n_c, xs, Kl, D,
-                           seed + 7919ull * (uint64_t)l, w.cent_f32, ragged ? n_live : nullptr, bf);
+                           seed + 7919ull * (uint64_t)l, w.cent_f32, ragged ? n_live : nullptr, bf,
+                           Kt, w.fill, tiles, w.cent_n2);
+        // a round: the assignment (which also counts the items of every centroid and turns the
+        // counts into offsets), the buckets, and what the round does with every bucket
+        auto assign_round = [&](const int32_t* list, const int32_t* lcnt, const int32_t* fill,
+                                int32_t* zero) -> int {
+            const AssignCounting ac{w.counts, w.pos, w.done, w.offsets, zero};
+            int rc;
+            if (on_mfma)
+                rc = launch_assign_mfma(D, x, n_c, xs, w.cent_tiles, w.cent_n2, Kl, NT, list, lcnt,
+                                        (size_t)n_c, w.assign, w.dist, ac, s);
+            else
+                rc = launch_assign<T>(lpr, g_assign, s, x, n_c, xs, w.cent_f32, Kl, D, fill, bf, list,
+                                      lcnt, (size_t)n_c, w.assign, w.dist, ac);
+            if (rc != HIRA_OK) return rc;
+            hipLaunchKernelGGL(k_bucket_fill, g_items, dim3(256), 0, s, w.assign, w.pos, w.offsets,
+                               n_c, list, lcnt, (size_t)n_c, Kl, w.members);
+            return HIRA_OK;
+        };
         for (int it = 0; it < niter; ++it) {
-            int rc;
-            if (w.cent_tiles != nullptr) {
-                rc = launch_cent_prep(D, w.cent_f32, Kl, NT, ragged ? w.fill : nullptr, bf,
-                                      w.cent_tiles, w.cent_n2, s);
-                if (rc == HIRA_OK)
-                    rc = launch_assign_mfma(D, x, n_c, xs, w.cent_tiles, w.cent_n2, Kl, NT, live,
-                                            live_cnt, live_stride, w.assign, w.dist, s);
-            } else {
-                rc = launch_assign<T>(lpr, g_assign, s, x, n_c, xs, w.cent_f32, Kl, D,
-                                      ragged ? w.fill : nullptr, bf, live, live_cnt, live_stride,
-                                      w.assign, w.dist);
-            }
+            const int rc = assign_round(live, live_cnt, ragged ? w.fill : nullptr, nullptr);
             if (rc != HIRA_OK) return rc;
-            fill_i32(w.counts, (size_t)NT * Kl, 0, s);
-            hipLaunchKernelGGL(k_bucket_count, g_items, dim3(256), 0, s, w.assign, n_c, live,
-                               live_cnt, live_stride, Kl, w.counts);
-            hipLaunchKernelGGL(k_scan, dim3(NT), dim3(256), 0, s, w.counts, Kl, w.offsets, w.cursor);
-            hipLaunchKernelGGL(k_bucket_fill, g_items, dim3(256), 0, s, w.assign, n_c, live,
-                               live_cnt, live_stride, Kl, w.cursor, w.members);
-            hipLaunchKernelGGL(k_bucket_sort, g_cent, dim3(kSortThreads), 0, s, w.members, w.offsets, w.dist,
-                               n_c, Kl, w.sorted);
-            hipLaunchKernelGGL((k_mean<T>), g_cent, dim3(256), 0, s, x, xs, n_c, Kl, D, w.offsets,
-                               w.sorted, nullptr, bf, w.cent_f32, nullptr);
+            hipLaunchKernelGGL((k_bucket_mean<T>), g_cent, dim3(kBucketThreads), 0, s, x, xs, n_c,
+                               Kl, D, w.offsets, w.members, w.ordered, ragged ? w.fill : nullptr, bf,
+                               w.cent_f32, Kt, tiles, w.cent_n2, w.counts, w.done);
         }
-        // capacity packing
-        if (!ragged) {  // (ragged: both were set up ahead of the Lloyd rounds)
-            fill_i32(w.fill, (size_t)NT * Kl, 0, s);
-            fill_i32(w.placed, (size_t)NT * n_c, 0, s);
-        }
-        fill_i32(w.slots[l], (size_t)NT * Kl * bf, -1, s);
+        // capacity packing: round r walks list r % 2 (the first one all items, or the items the
+        // trees hold) and leaves those it could not place on the other list
         for (int r = 0; r < pack_rounds; ++r) {
-            // (ragged: the first round walks the list of the items the trees hold, made above)
-            const int32_t* list = r == 0 && !ragged ? nullptr : w.list;
-            const int32_t* lcnt = r == 0 && !ragged ? nullptr : w.list_count;
-            if (r > 0) {
-                fill_i32(w.list_count, (size_t)NT, 0, s);
-                hipLaunchKernelGGL(k_collect_unplaced, g_items, dim3(256), 0, s, w.placed, n_c,
-                                   w.list, w.list_count);
-            }
-            int rc;
-            if (w.cent_tiles != nullptr) {  // full centroids get an infinite norm: never nearest
-                rc = launch_cent_prep(D, w.cent_f32, Kl, NT, w.fill, bf, w.cent_tiles, w.cent_n2, s);
-                if (rc == HIRA_OK)
-                    rc = launch_assign_mfma(D, x, n_c, xs, w.cent_tiles, w.cent_n2, Kl, NT, list,
-                                            lcnt, (size_t)n_c, w.assign, w.dist, s);
-            } else {
-                rc = launch_assign<T>(lpr, g_assign, s, x, n_c, xs, w.cent_f32, Kl, D, w.fill, bf,
-                                      list, lcnt, (size_t)n_c, w.assign, w.dist);
-            }
+            const int32_t* list = r == 0 ? live : w.list[r & 1];
+            const int32_t* lcnt = r == 0 ? live_cnt : w.list_count + (size_t)(r & 1) * NT;
+            int32_t* next_cnt = w.list_count + (size_t)((r + 1) & 1) * NT;
+            const int rc = assign_round(list, lcnt, w.fill, next_cnt);
             if (rc != HIRA_OK) return rc;
-            fill_i32(w.counts, (size_t)NT * Kl, 0, s);
-            hipLaunchKernelGGL(k_bucket_count, g_items, dim3(256), 0, s, w.assign, n_c, list, lcnt,
-                               (size_t)n_c, Kl, w.counts);
-            hipLaunchKernelGGL(k_scan, dim3(NT), dim3(256), 0, s, w.counts, Kl, w.offsets, w.cursor);
-            hipLaunchKernelGGL(k_bucket_fill, g_items, dim3(256), 0, s, w.assign, n_c, list, lcnt,
-                               (size_t)n_c, Kl, w.cursor, w.members);
-            hipLaunchKernelGGL(k_bucket_sort, g_cent, dim3(kSortThreads), 0, s, w.members, w.offsets, w.dist,
-                               n_c, Kl, w.sorted);
-            hipLaunchKernelGGL(k_accept, g_cent, dim3(64), 0, s, w.sorted, w.offsets, n_c, Kl, bf,
-                               w.fill, w.slots[l], w.placed);
+            hipLaunchKernelGGL(k_bucket_accept, g_cent, dim3(kBucketThreads), 0, s, w.members,
+                               w.offsets, w.dist, n_c, Kl, bf, w.fill, w.slots[l], w.placed,
+                               w.list[(r + 1) & 1], next_cnt, Kt, on_mfma ? w.cent_n2 : nullptr,
+                               w.counts, w.done);
         }
-        hipLaunchKernelGGL(k_leftover, dim3(NT), dim3(kLeftThreads), 0, s, n_c, Kl, bf, w.fill, w.slots[l],
-                           w.placed, w.scratch);
+        hipLaunchKernelGGL(k_leftover_count, g_items, dim3(256), 0, s, w.placed, n_c, Kl, bf, w.fill,
+                           w.chunk_pre, w.free_pre, w.done);
+        hipLaunchKernelGGL(k_leftover_place, g_items, dim3(256), 0, s, n_c, Kl, bf, w.fill,
+                           w.chunk_pre, w.free_pre, w.slots[l], w.placed);
         // block centre = mean of what is in the block, rounded to the storage type
-        hipLaunchKernelGGL((k_mean<T>), g_cent, dim3(64), 0, s, x, xs, n_c, Kl, D, nullptr, nullptr,
-                           w.slots[l], bf, w.cent_f32, w.cent_t[l]);
+        hipLaunchKernelGGL((k_block_mean<T>), g_cent, dim3(64), 0, s, x, xs, Kl, D, w.slots[l], bf,
+                           lpr, w.cent_f32, w.cent_t[l]);
         HIRA_CHECK_LAUNCH("build level");
     }
 
@@ -807,7 +962,7 @@ static int build_impl(const HiraTree* t, const void* keys_in, const void* values
         const float* crad = l == 1 ? nullptr : t->radii[l - 1];
         hipLaunchKernelGGL((k_radii<T>), dim3(t->size[l], NT), dim3(64), 0, s, child,
                            (size_t)t->cap[l - 1], crad, (size_t)t->cap[l - 1], w.order[l - 1],
-                           t->size[l - 1], t->centers[l], (size_t)t->cap[l], t->size[l], bf, D,
+                           t->size[l - 1], t->centers[l], (size_t)t->cap[l], t->size[l], bf, D, lpr,
                            l == 1 ? key_layout_of(t->layout) : center_layout_of(t->layout),
                            center_layout_of(t->layout), t->radii[l], t->counts[l], (size_t)t->cap[l]);
     }
@@ -969,7 +1124,7 @@ extern "C" int hira_nearest(const void* x, int32_t dtype, int32_t num_trees, int
         rc = launch_cent_prep(dim, centers, m, num_trees, b.fill, 1, b.tiles, b.n2, s);
         if (rc == HIRA_OK)
             rc = launch_assign_mfma(dim, x, n, (size_t)n, b.tiles, b.n2, m, num_trees, nullptr,
-                                    nullptr, 0, idx, dist2, s);
+                                    nullptr, 0, idx, dist2, AssignCounting{}, s);
     } else {
         const int epl = dtype == HIRA_F32 ? 4 : 8;
         int lpr = 2;
@@ -977,9 +1132,9 @@ extern "C" int hira_nearest(const void* x, int32_t dtype, int32_t num_trees, int
         const dim3 grid(ceil_div(n, 4 * (64 / lpr) * kPPG), num_trees);
         rc = dtype == HIRA_F32
                  ? launch_assign<float>(lpr, grid, s, x, n, (size_t)n, centers, m, dim, b.fill, 1,
-                                        nullptr, nullptr, 0, idx, dist2)
+                                        nullptr, nullptr, 0, idx, dist2, AssignCounting{})
                  : launch_assign<bf16_t>(lpr, grid, s, x, n, (size_t)n, centers, m, dim, b.fill, 1,
-                                         nullptr, nullptr, 0, idx, dist2);
+                                         nullptr, nullptr, 0, idx, dist2, AssignCounting{});
     }
     if (rc != HIRA_OK) return rc;
     HIRA_CHECK_LAUNCH("nearest-centre kernel");

@@ -136,6 +136,36 @@ def test_lloyd_rounds_tighten_the_balls(gpu_device):
     assert r5 < r0
 
 
+@pytest.mark.parametrize("dtype,d,n,same,bf,nl,niter", [
+    (torch.float32, 64, 3000, 700, 16, 2, 2),      # a bucket of 700: sorting network in LDS
+    (torch.bfloat16, 128, 8192, 3000, 16, 3, 2),   # 3000: packing sorts it in two goes
+    (torch.float32, 32, 8192, 6000, 8, 2, 1),      # 6000: the mean orders it through a bit map
+    (torch.bfloat16, 64, 140000, 5000, 32, 2, 1),  # ... with more item ids than one bit map holds
+])
+def test_buckets_far_larger_than_a_block(dtype, d, n, same, bf, nl, niter, gpu_device):
+    """`same` copies of one key all have the same nearest centroid: one bucket of that many
+    members in every round.  The layout holds, and two builds give the same tree bit for bit
+    although the members of a bucket arrive in a different order in every run."""
+    from hira_amd.indexer.hip import HIPIndexer
+
+    print(f"case {dtype} d={d} n={n} same={same} bf={bf} levels={nl}", flush=True)
+    rnd = bf16_round if dtype == torch.bfloat16 else (lambda x: x)
+    rng = np.random.default_rng(n + same)
+    keys = rnd(normalized_keys(2, n, d, seed=n))
+    where = rng.permutation(n)[:same]
+    keys[0, where] = keys[0, where[0]]
+    keys[1, where] = keys[1, where[0]] * np.float32(0.5)
+    kt = torch.from_numpy(keys)[None].to(dtype)
+    a = HIPIndexer(nl, niter, bf, seed=3).build(kt, kt.clone())
+    b = HIPIndexer(nl, niter, bf, seed=3).build(kt, kt.clone())
+    torch.cuda.synchronize()
+    _check_layout(a, keys, keys, dtype)
+    assert torch.equal(a.perm, b.perm)
+    for l in range(1, nl):
+        assert torch.equal(a.centers[l], b.centers[l]) and torch.equal(a.radii[l], b.radii[l])
+        assert torch.equal(a.counts[l], b.counts[l])
+
+
 def test_tiled_and_row_major_builds_hold_the_same_tree(gpu_device):
     """The tile arrangement only moves 16-byte chunks around: same tree, same answers."""
     from hira_amd.indexer.hip import HIPIndexer, from_tiled, to_tiled
