@@ -67,13 +67,13 @@ __global__ __launch_bounds__(64) void k_cent_prep(const float* cent, int K, cons
     }
 }
 
-template <int KS>
-__global__ __launch_bounds__(kAssignThreads, 2) void k_assign_mfma(
+// The items of one workgroup: RI operand tiles of 16 items a wave.
+template <int KS, int RI>
+__device__ __forceinline__ void assign_items(
     const void* x, int n_c, size_t x_tree_stride, const uint4* tiles, const float* cn2, int Kt,
-    const int32_t* list, const int32_t* list_count, size_t list_stride, int32_t* assign,
-    float* dist, int K, AssignCounting ac) {
+    const int32_t* list, int n_items, size_t list_stride, int32_t* assign, float* dist, int K,
+    const AssignCounting& ac) {
     constexpr int D = 32 * KS;
-    constexpr int RI = kAssignRI;
     constexpr int TILE_CHUNKS = 2 * KS * 64;                 // hi and lo halves of 16 centroids
     constexpr int TPS = assign_stage(KS);
     constexpr int STAGE_CHUNKS = TPS * TILE_CHUNKS;
@@ -87,13 +87,7 @@ __global__ __launch_bounds__(kAssignThreads, 2) void k_assign_mfma(
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n = lane & 15, kb = lane >> 4;  // operand row / centroid column, column block
     const int t = blockIdx.y;
-    const int n_items = list ? list_count[t] : n_c;
     const int first = (blockIdx.x * (kAssignThreads / 64) + wave) * (RI * 16);
-    // (a launch that counts: a workgroup without items still draws its ticket at the end)
-    const bool active = (int)blockIdx.x * (kAssignThreads / 64) * (RI * 16) < n_items;  // uniform
-    if (ac.counts == nullptr && !active) return;
-    if (ac.zero != nullptr && blockIdx.x == 0 && threadIdx.x == 0) ac.zero[t] = 0;
-    if (active) {
 
     // ---- my items: operand tiles in registers, ||x||^2 of row lane % 16 ------------------
     int item[RI];
@@ -198,7 +192,7 @@ __global__ __launch_bounds__(kAssignThreads, 2) void k_assign_mfma(
     // ---- merge the 16 centroid columns of a row group; the wave's 64 results pass through LDS
     // (free behind the loop's last barrier) so that every lane ends up with one item: one store
     // instruction, and one counting instruction, for the whole wave -----------------------------
-    static_assert(RI * 16 == 64, "one result per lane");
+    static_assert(RI == 1 || RI == 4, "a result per lane, or per lane of the first 16");
     int* s_g = reinterpret_cast<int*>(s_dyn) + wave * 128;
     float* s_b = reinterpret_cast<float*>(s_g + 64);
 #pragma unroll
@@ -226,17 +220,53 @@ __global__ __launch_bounds__(kAssignThreads, 2) void k_assign_mfma(
         // lane (kb, n) takes row n of operand tile kb: its item and ||x||^2 are its own
         const int g = s_g[lane];
         const float b = s_b[lane];
-        const int it = kb == 0 ? item[0] : kb == 1 ? item[1] : kb == 2 ? item[2] : item[3];
-        const float xx = kb == 0 ? x2[0] : kb == 1 ? x2[1] : kb == 2 ? x2[2] : x2[3];
-        if (it >= 0) {
+        int it = item[0];
+        float xx = x2[0];
+#pragma unroll
+        for (int ri = 1; ri < RI; ++ri)
+            if (kb == ri) {
+                it = item[ri];
+                xx = x2[ri];
+            }
+        if (kb < RI && it >= 0) {
             assign[(size_t)t * n_c + it] = g;
             dist[(size_t)t * n_c + it] = fmaxf(b + xx, 0.0f);
             if (ac.counts != nullptr && g >= 0)
                 ac.pos[(size_t)t * n_c + it] = atomicAdd(&ac.counts[(size_t)t * K + g], 1);
         }
     }
-    }  // active
-    if (ac.counts != nullptr) finish_counts(ac, t, K, (int)gridDim.x);
+}
+
+// Few items (the later rounds of the packing walk ever shorter lists) are spread over four times
+// as many workgroups, a single operand tile a wave: a workgroup's time is what its walk over all
+// centroid tiles takes, and that walk is four times shorter.  The lists' lengths are known on
+// the device only, so a launch over a list has workgroups for the narrow shape, and each tree
+// picks its shape by the length of its list.
+constexpr int kAssignNarrowItems = 256 * 256;  // (all trees together; measured: beyond this many the
+                                               // wide shape is faster, its tiles read from LDS once for 64 items)
+
+template <int KS, bool LISTED>
+__global__ __launch_bounds__(kAssignThreads, 2) void k_assign_mfma(
+    const void* x, int n_c, size_t x_tree_stride, const uint4* tiles, const float* cn2, int Kt,
+    const int32_t* list, const int32_t* list_count, size_t list_stride, int32_t* assign,
+    float* dist, int K, AssignCounting ac) {
+    const int t = blockIdx.y;
+    const int n_items = LISTED ? list_count[t] : n_c;
+    const bool narrow = LISTED && (long long)n_items * gridDim.y <= kAssignNarrowItems;
+    const int per_block = (kAssignThreads / 64) * 16 * (narrow ? 1 : kAssignRI);
+    // (a launch that counts: the tree's first workgroup draws a ticket also when there is no item)
+    const int nblocks = max((n_items + per_block - 1) / per_block, 1);
+    if ((int)blockIdx.x >= nblocks) return;  // uniform
+    if (ac.zero != nullptr && blockIdx.x == 0 && threadIdx.x == 0) ac.zero[t] = 0;
+    if ((int)blockIdx.x * per_block < n_items) {
+        if (LISTED && narrow)
+            assign_items<KS, 1>(x, n_c, x_tree_stride, tiles, cn2, Kt, list, n_items, list_stride,
+                                assign, dist, K, ac);
+        else
+            assign_items<KS, kAssignRI>(x, n_c, x_tree_stride, tiles, cn2, Kt, list, n_items,
+                                        list_stride, assign, dist, K, ac);
+    }
+    if (ac.counts != nullptr) finish_counts(ac, t, K, nblocks);
 }
 
 // centroid tiles per tree, in whole stages
@@ -266,27 +296,39 @@ int launch_assign_mfma(int dim, const void* x, int n_c, size_t x_tree_stride, co
                        const int32_t* list_count, size_t list_stride, int32_t* assign, float* dist,
                        const AssignCounting& counting, hipStream_t s) {
     const int Kt = assign_tiles(K);
-    const int per_block = (kAssignThreads / 64) * kAssignRI * 16;
+    // (a launch over a list: workgroups for the narrow shape, see kAssignNarrowItems)
+    const int per_block = (kAssignThreads / 64) * (list != nullptr ? 1 : kAssignRI) * 16;
     const int tps = assign_stage(dim / 32);
     const size_t smem = 2 * (size_t)tps * (2 * (dim / 32) * 64) * sizeof(uint4) + 2 * (size_t)tps * 16 * sizeof(float);
     const dim3 grid((n_c + per_block - 1) / per_block, num_trees);
     const uint4* tl = reinterpret_cast<const uint4*>(tiles);
+    constexpr int kMaxDevices = 64;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return fail(HIRA_ELAUNCH, "MFMA assignment: no current device");
     switch (dim) {
-#define HIRA_ASSIGN_MFMA(KS)                                                                        \
+#define HIRA_ASSIGN_MFMA_L(KS, LISTED)                                                              \
     {                                                                                               \
-        /* more than 64 KiB of dynamic LDS has to be asked for */                                   \
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_assign_mfma<KS>),                  \
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) \
-            return fail(HIRA_ELAUNCH, "MFMA assignment: %zu bytes of LDS refused", smem);              \
-        hipLaunchKernelGGL((k_assign_mfma<KS>), grid, dim3(kAssignThreads), smem, s, x, n_c,        \
+        /* more than 64 KiB of dynamic LDS has to be asked for: once per kernel and device */       \
+        static int asked[kMaxDevices];                                                              \
+        if (__atomic_load_n(&asked[dev], __ATOMIC_RELAXED) == 0) {                                  \
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(&k_assign_mfma<KS, LISTED>),      \
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) \
+                return fail(HIRA_ELAUNCH, "MFMA assignment: %zu bytes of LDS refused", smem);          \
+            __atomic_store_n(&asked[dev], 1, __ATOMIC_RELAXED);                                     \
+        }                                                                                           \
+        hipLaunchKernelGGL((k_assign_mfma<KS, LISTED>), grid, dim3(kAssignThreads), smem, s, x, n_c, \
                            x_tree_stride, tl, cn2, Kt, list, list_count, list_stride, assign, dist, \
                            K, counting);                                                            \
-    }                                                                                               \
+    }
+#define HIRA_ASSIGN_MFMA(KS)                                                                        \
+    if (list != nullptr) HIRA_ASSIGN_MFMA_L(KS, true) else HIRA_ASSIGN_MFMA_L(KS, false)            \
     break;
         case 64: HIRA_ASSIGN_MFMA(2)
         case 128: HIRA_ASSIGN_MFMA(4)
         case 256: HIRA_ASSIGN_MFMA(8)
 #undef HIRA_ASSIGN_MFMA
+#undef HIRA_ASSIGN_MFMA_L
         default: return fail(HIRA_EINVAL, "MFMA assignment: dim %d", dim);
     }
     return HIRA_OK;
