@@ -117,22 +117,29 @@ def hira_attention_forward(module, query, key, value, attention_mask=None, dropo
     plan = searcher.decode_plan(indexer, b * h_q, scaling)
     q2 = query.reshape(b * h_q, d).to(device=indexer.device, dtype=indexer.dtype).contiguous()
     out = torch.empty((b * h_q, indexer.vdim), dtype=torch.float32, device=indexer.device)
-    qk, qv = cache.queued_keys, cache.queued_values
-    if qk is not None and qk.shape[-2] > 0:
-        m = qk.shape[-2]
-        qk = qk.to(device=indexer.device, dtype=indexer.dtype).reshape(indexer.num_trees, m, d).contiguous()
-        qv = qv.to(device=indexer.device, dtype=indexer.dtype).reshape(indexer.num_trees, m, -1).contiguous()
-    else:
-        qk = qv = None
+    # the queue: the cache layer's own buffers as they are when they already hold the index's
+    # storage type (rows in use, rows per head), else a converted copy of the rows in use
+    qk = qv = None
+    qlen = int(cache.queued_keys.shape[-2]) if cache.queued_keys is not None else 0
+    if qlen > 0:
+        store = getattr(cache, "queue_store", None)
+        if store is not None and store[0].dtype == indexer.dtype and store[0].device == indexer.device \
+                and store[0].is_contiguous() and store[1].is_contiguous():
+            qk, qv = store
+        else:
+            qk = cache.queued_keys.to(device=indexer.device, dtype=indexer.dtype).reshape(
+                indexer.num_trees, qlen, d).contiguous()
+            qv = cache.queued_values.to(device=indexer.device, dtype=indexer.dtype).reshape(
+                indexer.num_trees, qlen, -1).contiguous()
     if sampled:
         plan.run_sampled(q2, cache.samples, cache.threshold_method, cache.threshold_topk, out,
-                         queue_keys=qk, queue_values=qv)
+                         queue_keys=qk, queue_values=qv, queue_len=qlen)
     else:
         th = torch.as_tensor(hira_threshold, dtype=torch.float32, device=indexer.device)
         if th.ndim == 0:
             th = th.expand(b * h_q)
         th = th.reshape(b * h_q).contiguous()
-        plan.run(q2, th, out, queue_keys=qk, queue_values=qv)
+        plan.run(q2, th, out, queue_keys=qk, queue_values=qv, queue_len=qlen)
     return out.reshape(b, 1, h_q, -1).to(query.dtype), None
 
 

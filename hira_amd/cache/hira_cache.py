@@ -40,6 +40,10 @@ class CacheOutput:
     samples: torch.Tensor | None = None
     threshold_method: str | None = None
     threshold_topk: int = 1
+    # the buffers queued_keys / queued_values are views of: (B, H_kv, cap, D) in the index's
+    # storage type and on its device, the first queued_keys.shape[-2] rows of every head in
+    # use.  The attention function hands them to the library as they are.
+    queue_store: tuple | None = None
 
 
 class HiraCacheLayer(CacheLayerMixin):
@@ -74,22 +78,49 @@ class HiraCacheLayer(CacheLayerMixin):
             raise NotImplementedError(f"Device mode {self.device_mode} not supported yet")
         self.indexed_len = 0
         self.queued_len = 0
+        self._update_takes_sync = None
 
-    def _empty_queue(self):
-        return torch.empty((self.batch, self.H_kv, 0, self.dim), dtype=self.dtype,
-                           device=self.device)
+    def _alloc_queue(self, rows: int):
+        """Room for `rows` queued keys and values per head, allocated once (the reference
+        concatenates per token, cache/hira_cache.py:121-140): in the index's storage type and
+        on its device, so that a decode step passes the buffers on without a copy."""
+        dt = getattr(self.indexer, "dtype", None) or self.dtype
+        dev = getattr(self.indexer, "device", None) or self.device
+        self._queue_k = torch.empty((self.batch, self.H_kv, rows, self.dim), dtype=dt, device=dev)
+        self._queue_v = torch.empty((self.batch, self.H_kv, rows, self.vdim), dtype=dt, device=dev)
+
+    @property
+    def queued_keys(self):
+        return self._queue_k[:, :, : self.queued_len]
+
+    @property
+    def queued_values(self):
+        return self._queue_v[:, :, : self.queued_len]
+
+    def _enqueue(self, key_states, value_states):
+        m = key_states.shape[-2]
+        if self.queued_len + m > self._queue_k.shape[-2]:  # (a step of many tokens)
+            old_k, old_v, n = self._queue_k, self._queue_v, self.queued_len
+            self._alloc_queue(max(2 * old_k.shape[-2], n + m))
+            self._queue_k[:, :, :n] = old_k[:, :, :n]
+            self._queue_v[:, :, :n] = old_v[:, :, :n]
+        self._queue_k[:, :, self.queued_len:self.queued_len + m].copy_(
+            key_states.reshape(self.batch, self.H_kv, m, self.dim))
+        self._queue_v[:, :, self.queued_len:self.queued_len + m].copy_(
+            value_states.reshape(self.batch, self.H_kv, m, self.vdim))
+        self.queued_len += m
 
     def lazy_initialization(self, key_states, value_states):
         self.dim = key_states.shape[-1]
+        self.vdim = value_states.shape[-1]
         self.H_kv = key_states.shape[-3]
         self.batch = key_states.shape[0] if key_states.ndim == 4 else 1
         self.dtype = key_states.dtype
         self.device = key_states.device
         self.indexer = self.indexer_cls(**self.indexer_kwargs)
         self.searcher = self.searcher_cls(**self.searcher_kwargs)
-        self.queued_keys = self._empty_queue()
-        self.queued_values = self._empty_queue()
         self.queued_len = 0
+        self._queue_k = self._queue_v = None  # allocated once the index knows its storage type
         self.keys = None  # the index holds the keys
         self.values = None
         self.is_initialized = True
@@ -99,12 +130,11 @@ class HiraCacheLayer(CacheLayerMixin):
         if not self.is_initialized:
             self.lazy_initialization(key_states, value_states)
             self.indexer.build(key_states, value_states)
+            self._alloc_queue(max(1, min(int(self.update_every), 4096)))
             self.indexed_len = key_states.shape[-2]
             self._take_samples(key_states)
             return self._output(key_states, value_states), None
-        self.queued_keys = torch.cat([self.queued_keys, key_states], dim=-2)
-        self.queued_values = torch.cat([self.queued_values, value_states], dim=-2)
-        self.queued_len += key_states.shape[-2]
+        self._enqueue(key_states, value_states)
         if self.queued_len >= self.update_every:
             self.update_index()
         return self._output(), None
@@ -168,22 +198,23 @@ class HiraCacheLayer(CacheLayerMixin):
             threshold_method=kw.get("method") if self.samples is not None else None,
             threshold_topk=max(1, min(int(kw.get("topk", 1)),
                                       self.samples.shape[1] if self.samples is not None else 1)),
+            queue_store=(self._queue_k, self._queue_v),
         )
 
     def update_index(self):
         # no read-back of the level sizes: the host carries their bounds (HIPIndexer.update,
         # sync=False), so folding the queue into the index does not wait for the GPU; a
         # one-level index has no node counts to bound with and keeps the synchronous form
-        import inspect
+        if self._update_takes_sync is None:
+            import inspect
 
-        if "sync" in inspect.signature(self.indexer.update).parameters:
+            self._update_takes_sync = "sync" in inspect.signature(self.indexer.update).parameters
+        if self._update_takes_sync:
             self.indexer.update(self.queued_keys, self.queued_values,
                                 sync=getattr(self.indexer, "num_levels", 1) < 2)
         else:  # an indexer with the reference's two-argument update
             self.indexer.update(self.queued_keys, self.queued_values)
         self._refresh_samples(self.queued_keys, self.indexed_len)
-        self.queued_keys = self._empty_queue()
-        self.queued_values = self._empty_queue()
         self.indexed_len += self.queued_len
         self.queued_len = 0
 
@@ -207,8 +238,7 @@ class HiraCacheLayer(CacheLayerMixin):
     def reset(self):
         if self.is_initialized:
             self.indexer = self.indexer_cls(**self.indexer_kwargs)
-            self.queued_keys = self._empty_queue()
-            self.queued_values = self._empty_queue()
+            self._queue_k = self._queue_v = None
             self.queued_len = 0
             self.indexed_len = 0
             self.samples = None

@@ -81,7 +81,7 @@ def device_thresholds(samples: torch.Tensor, query: torch.Tensor, method: str, k
     if out is None:
         out = torch.empty((h_q,), dtype=torch.float32, device=samples.device)
     if stream is None:
-        stream = torch.cuda.current_stream(samples.device).cuda_stream
+        stream = _lib.current_stream(samples.device)
     code = {"sample_max": 0, "sample_mean_topk": 1}[method]
     _lib.check(_lib.lib().hira_threshold(
         samples.data_ptr(), _lib.HIRA_BF16 if samples.dtype == torch.bfloat16 else _lib.HIRA_F32,

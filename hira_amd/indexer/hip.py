@@ -356,7 +356,7 @@ class HIPIndexer(BaseIndexer):
             slot_count = self.size[0] - slot_first
         slot_count = -(-slot_count // bf) * bf
         tree = self.tree_struct()
-        stream = torch.cuda.current_stream(self.device).cuda_stream
+        stream = _lib.current_stream(self.device)
         _lib.check(_lib.lib().hira_quantize(C.byref(tree), int(slot_first), int(slot_count),
                                             1 if new_steps else 0, stream))
         return self
@@ -503,7 +503,7 @@ class HIPIndexer(BaseIndexer):
         if need == 0:
             _lib.check(-1)
         ws = torch.empty(need, dtype=torch.uint8, device=self.device)
-        stream = torch.cuda.current_stream(self.device).cuda_stream
+        stream = _lib.current_stream(self.device)
         if key_counts is not None:
             if key_counts.dtype != torch.int32 or tuple(key_counts.shape) != (b * h,) \
                     or key_counts.device.type != self.device.type or not key_counts.is_contiguous():
@@ -817,7 +817,7 @@ class HIPIndexer(BaseIndexer):
             vin = new_values.to(device=self.device, dtype=self.dtype).reshape(
                 t, m, self.vdim).contiguous()
         tree = self.tree_struct()
-        stream = torch.cuda.current_stream(self.device).cuda_stream
+        stream = _lib.current_stream(self.device)
         rc = _lib.lib().hira_update(C.byref(tree), kin.data_ptr(),
                                     None if vin is None else vin.data_ptr(), m,
                                     self._state.data_ptr(), stream)

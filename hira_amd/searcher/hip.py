@@ -178,7 +178,7 @@ class HIPSearcher(BaseSearcher):
                 C.byref(self.launch))
             ws = self._get_workspace(ws_bytes, indexer.device)
             ws_ptr = ws.data_ptr()
-        stream = torch.cuda.current_stream(indexer.device).cuda_stream
+        stream = _lib.current_stream(indexer.device)
         rc = lib.hira_search(C.byref(tree), C.byref(qs), C.byref(queue) if queue else None,
                              C.byref(out), C.byref(self.launch), ws_ptr, ws_bytes, stream)
         _lib.check(rc)
@@ -247,7 +247,7 @@ class HIPSearcher(BaseSearcher):
         if out is None:
             out = torch.empty((h_q, indexer.vdim), dtype=torch.float32, device=dev)
         tree = indexer.tree_struct()
-        stream = torch.cuda.current_stream(dev).cuda_stream
+        stream = _lib.current_stream(dev)
         _lib.check(_lib.lib().hira_sparse_attention(
             C.byref(tree), C.byref(qs), index.data_ptr(), score.data_ptr(), count.data_ptr(),
             int(cap), out.data_ptr(), stream))
@@ -337,9 +337,11 @@ class DecodePlan:
 
     def run(self, query: torch.Tensor, threshold: torch.Tensor, out: torch.Tensor,
             stream: Optional[int] = None, queue_keys: Optional[torch.Tensor] = None,
-            queue_values: Optional[torch.Tensor] = None) -> None:
-        """queue_keys / queue_values: (T, m, D) / (T, m, Dv) contiguous, tree dtype: keys not in
-        the index yet, attended by every head of their tree."""
+            queue_values: Optional[torch.Tensor] = None, queue_len: Optional[int] = None) -> None:
+        """queue_keys / queue_values: (..., cap, D) / (..., cap, Dv) contiguous, tree dtype, the
+        leading dimensions amounting to T trees: keys not in the index yet, attended by every
+        head of their tree; the first `queue_len` rows of every tree are in use (all `cap`
+        when not given)."""
         if self.indexer.tree_struct() is not self.tree:  # the index grew since the plan was made
             self.tree = self.indexer.tree_struct()
             need = self._workspace_need()
@@ -352,12 +354,16 @@ class DecodePlan:
         self.query.tau = threshold.data_ptr()
         self.out.attn_out = out.data_ptr()
         if stream is None:
-            stream = torch.cuda.current_stream(self.indexer.device).cuda_stream
+            stream = _lib.current_stream(self.indexer.device)
         t, q, o, l = self._refs
         qu = None
-        if queue_keys is not None and queue_keys.shape[-2] > 0:
-            m = int(queue_keys.shape[-2])
-            self.queue = _lib.HiraQueue(queue_keys.data_ptr(), queue_values.data_ptr(), m, m)
+        if queue_keys is not None and queue_keys.shape[-2] > 0 and queue_len != 0:
+            cap = int(queue_keys.shape[-2])
+            m = cap if queue_len is None else int(queue_len)
+            if not 0 < m <= cap or queue_values.shape[-2] != cap:
+                raise ValueError(f"queue: {m} rows in use of {cap} "
+                                 f"(values hold {queue_values.shape[-2]})")
+            self.queue = _lib.HiraQueue(queue_keys.data_ptr(), queue_values.data_ptr(), m, cap)
             qu = C.byref(self.queue)
         rc = self.lib.hira_search(t, q, qu, o, l, self.ws.data_ptr(), self.ws_bytes, stream)
         if rc:
@@ -366,7 +372,8 @@ class DecodePlan:
     def run_sampled(self, query: torch.Tensor, samples: torch.Tensor, method: str, k: int,
                     out: torch.Tensor, stream: Optional[int] = None,
                     queue_keys: Optional[torch.Tensor] = None,
-                    queue_values: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    queue_values: Optional[torch.Tensor] = None,
+                    queue_len: Optional[int] = None) -> torch.Tensor:
         """A decode step whose thresholds come from a key sample (T, S, D), tree dtype,
         contiguous: ``hira_threshold`` ("sample_max" or "sample_mean_topk" with k) writes them
         into a buffer of the plan, ``run`` follows on the same stream.  Returns that buffer."""
@@ -379,7 +386,7 @@ class DecodePlan:
             raise ValueError(f"samples {tuple(samples.shape)} {samples.dtype}: expected contiguous "
                              f"({self.tree.num_trees}, S, {self.tree.dim}) {self.indexer.dtype}")
         if stream is None:
-            stream = torch.cuda.current_stream(self.indexer.device).cuda_stream
+            stream = _lib.current_stream(self.indexer.device)
         self.query.q = query.data_ptr()
         rc = self.lib.hira_threshold(
             samples.data_ptr(), self.tree.dtype, self.tree.num_trees, int(samples.shape[1]),
@@ -387,7 +394,7 @@ class DecodePlan:
             self.tau_buf.data_ptr(), stream)
         if rc:
             _lib.check(rc)
-        self.run(query, self.tau_buf, out, stream, queue_keys, queue_values)
+        self.run(query, self.tau_buf, out, stream, queue_keys, queue_values, queue_len)
         return self.tau_buf
 
 

@@ -76,6 +76,32 @@ def test_decode_queues_then_flushes_every_update_every(patched):
     assert l.get_seq_length() == 14 and l.queued_len == 1
 
 
+def test_the_queue_is_one_buffer_allocated_once(patched):
+    """Queued rows land in a buffer of update_every rows that is allocated with the index (the
+    reference concatenates per token, cache/hira_cache.py:121-140); what the layer hands out are
+    views of it, and values may be narrower than keys.  A step of more tokens than fit grows it."""
+    l = _layer(update_every=5)
+    l.update(torch.randn(1, 2, 10, 16), torch.randn(1, 2, 10, 8))
+    store = l._queue_k
+    assert store.shape == (1, 2, 5, 16) and l._queue_v.shape == (1, 2, 5, 8)
+    toks = [(torch.randn(1, 2, 1, 16), torch.randn(1, 2, 1, 8)) for _ in range(4)]
+    for i, t in enumerate(toks):
+        o = l.update(*t)[0]
+        assert l._queue_k is store and o.queue_store[0] is store
+        assert o.queued_keys.shape == (1, 2, i + 1, 16) and o.queued_values.shape == (1, 2, i + 1, 8)
+        assert o.queued_keys.data_ptr() == store.data_ptr()
+    assert torch.equal(o.queued_keys, torch.cat([t[0] for t in toks], dim=-2))
+    assert torch.equal(o.queued_values, torch.cat([t[1] for t in toks], dim=-2))
+    # six tokens at once: more than the buffer holds; they reach update_every and are flushed
+    many = (torch.randn(1, 2, 6, 16), torch.randn(1, 2, 6, 8))
+    o = l.update(*many)[0]
+    assert l.queued_len == 0 and o.queued_keys.shape[-2] == 0 and l.indexed_len == 20
+    fk, fv = l.indexer.updates[0]
+    assert torch.equal(fk, torch.cat([t[0] for t in toks] + [many[0]], dim=-2))
+    assert torch.equal(fv, torch.cat([t[1] for t in toks] + [many[1]], dim=-2))
+    assert l._queue_k.shape[-2] >= 10
+
+
 def test_mask_sizes_lengths_and_reset(patched):
     l = _layer()
     assert l.get_seq_length() == 0 and l.get_max_cache_shape() == -1 and l.get_max_length() == -1
