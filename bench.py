@@ -534,12 +534,14 @@ def main():
     keys_d, values_d = keys.to(dev), values.to(dev)
     niter = w.kmeans_iters if a.kmeans_iters < 0 else a.kmeans_iters
     t0 = time.perf_counter()
-    index = HIPIndexer(w.num_levels, niter, w.bf, device="cuda:0", layout=a.layout).build(keys_d, values_d)
+    index = HIPIndexer(w.num_levels, niter, w.bf, device="cuda:0", layout=a.layout,
+                       heads_per_tree=w.group).build(keys_d, values_d)
     torch.cuda.synchronize()
     build_ms = (time.perf_counter() - t0) * 1e3
     # (the first build of a process also loads the library and its code objects)
     t0 = time.perf_counter()
-    again = HIPIndexer(w.num_levels, niter, w.bf, device="cuda:0", layout=a.layout).build(keys_d, values_d)
+    again = HIPIndexer(w.num_levels, niter, w.bf, device="cuda:0", layout=a.layout,
+                       heads_per_tree=w.group).build(keys_d, values_d)
     torch.cuda.synchronize()
     build_again_ms = (time.perf_counter() - t0) * 1e3
     del again
@@ -677,7 +679,8 @@ def main():
         one_index = 2 * keys_d.numel() * keys_d.element_size()
         a.layers = 8 if one_index <= 256 * 1024 * 1024 else 0
     if a.layers > 1 and not a.profile:
-        copies = [index] + [HIPIndexer(w.num_levels, niter, w.bf, device="cuda:0", layout=a.layout).build(keys_d, values_d)
+        copies = [index] + [HIPIndexer(w.num_levels, niter, w.bf, device="cuda:0", layout=a.layout,
+                       heads_per_tree=w.group).build(keys_d, values_d)
                             for _ in range(a.layers - 1)]
         plans = [plan] + [searcher.plan_attention(c, h_all, scaling=torch.full((h_all,), scale))
                           for c in copies[1:]]
@@ -701,20 +704,24 @@ def main():
                "same_outputs": same}
         del copies, plans, g3
 
-    # ---- the same steps over an index that also keeps an 8-bit shadow of its keys (layout q8):
-    # the scan reads the shadow, the exact test only the rows the shadow cannot rule out
+    # ---- the same steps over an index in the other layout: with an 8-bit shadow of its keys
+    # (layout q8: the scan reads the shadow, the exact test only the rows the shadow cannot rule
+    # out) when the index above has none, without one when it has (layout="auto" adds the shadow
+    # to long trees with many heads)
     q8_leg = None
-    if not index.q8 and not a.profile and w.dtype == torch.bfloat16 and w.d % 64 == 0 \
+    other_layout = "tiled" if index.q8 else "q8"
+    if not a.profile and w.dtype == torch.bfloat16 and w.d in (64, 128) \
             and index.num_levels >= 2 and a.kernel != 1:
         try:
-            qindex = HIPIndexer(w.num_levels, niter, w.bf, device="cuda:0", layout="q8").build(keys_d, values_d)
+            qindex = HIPIndexer(w.num_levels, niter, w.bf, device="cuda:0", layout=other_layout).build(keys_d, values_d)
             qstats = torch.zeros_like(stats)
             qsplan = searcher.plan_attention(qindex, h_all, scaling=torch.full((h_all,), scale), stats=qstats)
             qouts = torch.empty_like(outs)
             for i in range(W, total):
                 qsplan.run(q_d[i], taus[i], qouts[i])
             torch.cuda.synchronize()
-            qb, qb16, qcounts = algorithmic_bytes(qstats.cpu().numpy(), w, qindex.num_levels, K, shadow=True)
+            qb, qb16, qcounts = algorithmic_bytes(qstats.cpu().numpy(), w, qindex.num_levels, K,
+                                                  shadow=qindex.q8)
             qplan = searcher.plan_attention(qindex, h_all, scaling=torch.full((h_all,), scale))
             gq = torch.cuda.CUDAGraph()
             with torch.cuda.stream(stream):
@@ -729,7 +736,7 @@ def main():
                 q1.record(stream)
                 stream.synchronize()
             q_us = q0.elapsed_time(q1) * 1e3 / K
-            q8_leg = {"us_per_step": round(q_us, 3), "algorithmic_bytes_per_step": round(qb),
+            q8_leg = {"layout": qindex.layout_name, "us_per_step": round(q_us, 3), "algorithmic_bytes_per_step": round(qb),
                       "achieved_GBps": round(qb / (q_us * 1e-6) / 1e9, 1),
                       "frac_of_hbm_peak": round(qb / (q_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
                       "exact_rows_per_step": round(qcounts["exact_rows_per_step"], 1),
@@ -739,7 +746,7 @@ def main():
                       "max_abs_diff_of_outputs": float((qouts[W:] - outs[W:]).abs().max())}
             del qindex, qsplan, qplan, gq
         except Exception as ex:  # noqa: BLE001
-            log(f"[bench] q8 leg failed: {ex!r}")
+            log(f"[bench] leg in the {other_layout} layout failed: {ex!r}")
 
     # ---- dense comparators ------------------------------------------------------------
     dense_us = {}
@@ -860,7 +867,7 @@ def main():
                           "p99": round(float(np.percentile(per_step, 99)), 2)},
         "streaming_add_GBps": round(stream_gbs, 1),
         "rotating_indexes": rot,
-        "q8_shadow_layout": q8_leg,
+        ("bf16_scan_layout" if index.q8 else "q8_shadow_layout"): q8_leg,
         "sample_threshold_us": round(thr_us, 2),
         "step_with_sample_threshold_us": round(step_thr_us, 2),
         "dense_attention_us": {k: round(v, 2) for k, v in dense_us.items()},

@@ -115,7 +115,10 @@ def hira_attention_forward(module, query, key, value, attention_mask=None, dropo
         hira_threshold = index_thresholds(indexer, query, hira_topk or max(1, indexer.num_keys // 100))
     # one plan per (index, head count, scale): a decode step is then a single library call
     plan = searcher.decode_plan(indexer, b * h_q, scaling)
-    q2 = query.reshape(b * h_q, d).to(device=indexer.device, dtype=indexer.dtype).contiguous()
+    q2 = query.reshape(b * h_q, d)
+    if q2.dtype != indexer.dtype or q2.device != indexer.device:
+        q2 = q2.to(device=indexer.device, dtype=indexer.dtype)
+    q2 = q2.contiguous()
     out = torch.empty((b * h_q, indexer.vdim), dtype=torch.float32, device=indexer.device)
     # the queue: the cache layer's own buffers as they are when they already hold the index's
     # storage type (rows in use, rows per head), else a converted copy of the rows in use

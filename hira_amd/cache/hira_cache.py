@@ -91,11 +91,11 @@ class HiraCacheLayer(CacheLayerMixin):
 
     @property
     def queued_keys(self):
-        return self._queue_k[:, :, : self.queued_len]
+        return self._queue_k.narrow(2, 0, self.queued_len)
 
     @property
     def queued_values(self):
-        return self._queue_v[:, :, : self.queued_len]
+        return self._queue_v.narrow(2, 0, self.queued_len)
 
     def _enqueue(self, key_states, value_states):
         m = key_states.shape[-2]
@@ -104,10 +104,11 @@ class HiraCacheLayer(CacheLayerMixin):
             self._alloc_queue(max(2 * old_k.shape[-2], n + m))
             self._queue_k[:, :, :n] = old_k[:, :, :n]
             self._queue_v[:, :, :n] = old_v[:, :, :n]
-        self._queue_k[:, :, self.queued_len:self.queued_len + m].copy_(
-            key_states.reshape(self.batch, self.H_kv, m, self.dim))
-        self._queue_v[:, :, self.queued_len:self.queued_len + m].copy_(
-            value_states.reshape(self.batch, self.H_kv, m, self.vdim))
+        if key_states.ndim != 4:
+            key_states = key_states.reshape(self.batch, self.H_kv, m, self.dim)
+            value_states = value_states.reshape(self.batch, self.H_kv, m, self.vdim)
+        self._queue_k.narrow(2, self.queued_len, m).copy_(key_states)
+        self._queue_v.narrow(2, self.queued_len, m).copy_(value_states)
         self.queued_len += m
 
     def lazy_initialization(self, key_states, value_states):
@@ -264,17 +265,39 @@ class HiraCache(Cache):
                 layer_types = ["full_attention" for _ in range(config.num_hidden_layers)]
         if hasattr(config, "num_kv_shared_layers"):
             layer_types = layer_types[: -config.num_kv_shared_layers]
+        # query heads per KV head: the indexer's layout="auto" weighs it (an 8-bit shadow of the
+        # keys pays from 8 heads a tree on)
+        heads, kv_heads = (getattr(config, "num_attention_heads", None),
+                           getattr(config, "num_key_value_heads", None))
+        group = heads // kv_heads if heads and kv_heads and heads % kv_heads == 0 else None
         layers = [
             HiraCacheLayer(
                 device_mode=self.device_mode,
                 update_every=self.update_every,
-                indexer_kwargs=hira_config.get_indexer_kwargs(),
+                indexer_kwargs=self._indexer_kwargs(hira_config, group),
                 searcher_kwargs=hira_config.get_searcher_kwargs(),
                 threshold_kwargs=hira_config.get_threshold_kwargs(),
             )
             for _ in layer_types
         ]
         super().__init__(layers=layers, offloading=False)
+
+    @staticmethod
+    def _indexer_kwargs(hira_config: HiraConfig, group):
+        """The configuration's indexer arguments, plus the heads per tree where the indexer in
+        use takes them (one with the reference's constructor does not)."""
+        import inspect
+
+        import hira_amd.cache.hira_cache as me
+
+        kw = dict(hira_config.get_indexer_kwargs())
+        try:
+            params = inspect.signature(me.CUDAIndexer.__init__).parameters
+        except (TypeError, ValueError):
+            params = {}
+        if group is not None and "heads_per_tree" in params:
+            kw["heads_per_tree"] = group
+        return kw
 
     def update(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int,
                cache_kwargs: dict[str, Any] | None = None, *args, **kwargs):

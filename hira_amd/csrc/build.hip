@@ -986,9 +986,10 @@ static int check_build_args(const HiraTree* t, int n) {
     HIRA_CHECK_ARG(t->layout == HIRA_ROW_MAJOR || t->layout == HIRA_TILE16 ||
                        t->layout == HIRA_TILE16_Q8, "layout %d", t->layout);
     if (t->layout == HIRA_TILE16_Q8)
-        HIRA_CHECK_ARG(t->dim % 64 == 0 && t->num_levels >= 2 && t->keys8 && t->kscale && t->keps,
-                       "the layout with an 8-bit shadow needs rows of a multiple of 64 columns, at "
-                       "least two levels, and the keys8 / kscale / keps arrays");
+        HIRA_CHECK_ARG((t->dim == 64 || t->dim == 128) && t->num_levels >= 2 && t->keys8 &&
+                           t->kscale && t->keps,
+                       "the layout with an 8-bit shadow needs rows of 64 or 128 columns, at least "
+                       "two levels, and the keys8 / kscale / keps arrays");
     if (t->layout != HIRA_ROW_MAJOR) {
         HIRA_CHECK_ARG(t->dtype == HIRA_BF16 && t->dim % 32 == 0,
                        "the tiled layout needs bf16 rows of a multiple of 32 columns");

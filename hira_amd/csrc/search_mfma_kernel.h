@@ -1532,6 +1532,5 @@ void launch_mfma_nt1_d256(const SearchPlan& plan, const SearchParams& p, dim3 gr
 void launch_mfma_nt2_d256(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
 void launch_mfma_q8_d64(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
 void launch_mfma_q8_d128(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
-void launch_mfma_q8_d256(const SearchPlan& plan, const SearchParams& p, dim3 grid, hipStream_t s);
 
 }  // namespace hira

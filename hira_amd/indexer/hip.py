@@ -21,7 +21,7 @@ from __future__ import annotations
 
 import ctypes as C
 from enum import Enum
-from typing import List, Optional
+from typing import List, Optional, Tuple
 
 import torch
 
@@ -70,6 +70,34 @@ def level_sizes(n: int, bf: int, num_levels: int) -> List[int]:
     return sizes
 
 
+# layout="auto" adds the 8-bit shadow of the keys where the search measurably gains from it: long
+# scans shared by many heads (131072 keys a tree and 8 query heads per KV head: a decode step of
+# 64 heads takes 54.8 us against 63.9 us); shorter trees or fewer heads a tree lose to the extra
+# dependent step of the exact test
+Q8_AUTO_MIN_KEYS = 131072
+Q8_AUTO_MIN_HEADS = 8
+
+
+def choose_layout(request: str, dtype: torch.dtype, dim: int, vdim: int, num_levels: int, bf: int,
+                  n: int, heads_per_tree: Optional[int] = None) -> Tuple[bool, bool]:
+    """(tiled, q8) for a layout request: which arrangement an index of `n` keys a tree gets.
+    Raises ValueError for an explicit request the keys cannot have."""
+    tile_ok = dtype == torch.bfloat16 and dim % 32 == 0
+    if request == "tiled" and not tile_ok:
+        raise ValueError("the tiled layout needs bfloat16 keys with dim a multiple of 32")
+    q8_ok = tile_ok and dim in (64, 128) and num_levels >= 2
+    if request == "q8" and not q8_ok:
+        raise ValueError("the q8 layout needs bfloat16 keys with dim 64 or 128 and at least two "
+                         "levels")
+    auto_tiled = (request == "auto" and tile_ok and num_levels >= 2 and bf % 16 == 0
+                  and dim in (64, 128, 256) and vdim in (0, dim))
+    q8 = request == "q8" or (
+        auto_tiled and q8_ok and vdim == dim and heads_per_tree is not None
+        and heads_per_tree >= Q8_AUTO_MIN_HEADS and n >= Q8_AUTO_MIN_KEYS)
+    tiled = tile_ok and (request in ("tiled", "q8") or auto_tiled)
+    return tiled, q8
+
+
 class HIPIndexer(BaseIndexer):
     class DEPTH(Enum):
         TWO_LEVELS = 2
@@ -89,6 +117,7 @@ class HIPIndexer(BaseIndexer):
         layout: str = "auto",
         device: str = "cuda",
         graft_min: Optional[int] = None,
+        heads_per_tree: Optional[int] = None,
     ):
         if isinstance(num_levels, HIPIndexer.DEPTH):
             num_levels = num_levels.value
@@ -107,6 +136,9 @@ class HIPIndexer(BaseIndexer):
         if layout not in ("auto", "row_major", "tiled", "q8"):
             raise ValueError("layout must be 'auto', 'row_major', 'tiled' or 'q8'")
         self.layout_request = layout
+        # query heads per KV head the searches will come with, when the caller knows (the cache
+        # layer does): layout="auto" takes it into account, see choose_layout
+        self.heads_per_tree = None if heads_per_tree is None else int(heads_per_tree)
         self.tiled = False  # centers (and, unless q8, keys) stored in the MFMA tile arrangement
         # q8: tiled centers, row-major keys and beside them an 8-bit shadow copy of the keys
         # (keys8, one step per tree and channel in kscale, error bounds per level-1 node in
@@ -244,18 +276,8 @@ class HIPIndexer(BaseIndexer):
         self.size = level_sizes(n, bf, nl)
         want = max(n, int(self.capacity or 0))
         self.cap = level_sizes(want, bf, nl) if want > n else list(self.size)
-        tile_ok = (dtype == torch.bfloat16 and dim % 32 == 0)
-        if self.layout_request == "tiled" and not tile_ok:
-            raise ValueError("the tiled layout needs bfloat16 keys with dim a multiple of 32")
-        q8_ok = tile_ok and dim % 64 == 0 and dim <= 256 and nl >= 2
-        if self.layout_request == "q8" and not q8_ok:
-            raise ValueError("the q8 layout needs bfloat16 keys with dim 64, 128, 192 or 256 and at "
-                             "least two levels")
-        self.q8 = self.layout_request == "q8"
-        self.tiled = tile_ok and (
-            self.layout_request in ("tiled", "q8")
-            or (self.layout_request == "auto" and nl >= 2 and bf % 16 == 0
-                and dim in (64, 128, 256) and vdim in (0, dim)))
+        self.tiled, self.q8 = choose_layout(self.layout_request, dtype, dim, vdim, nl, bf, n,
+                                            self.heads_per_tree)
         if self.tiled:
             self.cap = [-(-c // 16) * 16 for c in self.cap]
         dev, t = self.device, self.num_trees
@@ -419,7 +441,8 @@ class HIPIndexer(BaseIndexer):
             tensors = {k: f.get_tensor(k) for k in f.keys()}
         self = cls(meta["num_levels"], meta["max_iterations"], meta["branching_factor"],
                    pad_value=meta["pad_value"], seed=meta["seed"], pack_rounds=meta["pack_rounds"],
-                   layout=meta["layout_request"], capacity=capacity, device=device)
+                   layout="q8" if meta.get("q8") else ("tiled" if meta["tiled"] else "row_major"),
+                   capacity=capacity, device=device)
         dtype = torch.bfloat16 if meta["dtype"] == "bfloat16" else torch.float32
         size, rows = list(meta["size"]), list(meta["rows"])
         # room for what the file holds (and for `capacity`), then the saved sizes

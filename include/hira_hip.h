@@ -44,7 +44,7 @@ enum { HIRA_F32 = 0, HIRA_BF16 = 1 };
  * i.e. one wave-wide 128-bit load fetches a complete 16x32 MFMA operand tile from 1 KiB of
  * contiguous memory.  Values, radii, counts and perm are never tiled. */
 enum { HIRA_ROW_MAJOR = 0, HIRA_TILE16 = 1, HIRA_TILE16_Q8 = 2 };
-/* HIRA_TILE16_Q8 (bf16 only, D a multiple of 64, every cap a multiple of 16): the centers of
+/* HIRA_TILE16_Q8 (bf16 only, D = 64 or 128, every cap a multiple of 16): the centers of
  * every level are tiled as in HIRA_TILE16, the keys are ROW-MAJOR, and beside them sits an
  * 8-bit shadow copy `keys8` that the search scans first: k8 = round(k / kscale[channel]),
  * clipped to [-127, 127], with one step `kscale` per tree and channel, in tiles of 16 rows x

@@ -322,3 +322,35 @@ def test_storage_dtype_policy():
     with pytest.warns(UserWarning, match="bfloat16"):
         assert HIPIndexer.storage_dtype(torch.float16) == torch.bfloat16
     assert HIPIndexer.storage_dtype(torch.float64) == torch.float32
+
+
+def test_layout_rule_adds_the_shadow_only_for_long_trees_with_many_heads():
+    """layout="auto": tiled where the MFMA kernel can scan, with the 8-bit shadow only from
+    131072 keys a tree and 8 query heads per KV head on (where it measurably wins); explicit
+    requests are honoured or refused."""
+    import torch
+    from hira_amd.indexer.hip import Q8_AUTO_MIN_HEADS, Q8_AUTO_MIN_KEYS, choose_layout
+
+    bf16, f32 = torch.bfloat16, torch.float32
+    assert (Q8_AUTO_MIN_KEYS, Q8_AUTO_MIN_HEADS) == (131072, 8)
+    # (request, dtype, dim, vdim, levels, bf, n, heads per tree) -> (tiled, q8)
+    assert choose_layout("auto", bf16, 128, 128, 4, 32, 131072, 8) == (True, True)
+    assert choose_layout("auto", bf16, 128, 128, 4, 32, 131071, 8) == (True, False)
+    assert choose_layout("auto", bf16, 128, 128, 4, 32, 1 << 20, 7) == (True, False)
+    assert choose_layout("auto", bf16, 128, 128, 4, 32, 1 << 20, None) == (True, False)
+    assert choose_layout("auto", bf16, 64, 64, 3, 16, 1 << 18, 16) == (True, True)
+    assert choose_layout("auto", bf16, 256, 256, 3, 32, 1 << 18, 16) == (True, False)  # no shadow kernels
+    assert choose_layout("auto", bf16, 128, 0, 3, 32, 1 << 18, 16) == (True, False)    # no values: scores only
+    assert choose_layout("auto", bf16, 128, 128, 1, 32, 1 << 18, 16) == (False, False)
+    assert choose_layout("auto", bf16, 128, 128, 3, 8, 1 << 18, 16) == (False, False)  # fan-out not in tiles
+    assert choose_layout("auto", f32, 128, 128, 3, 32, 1 << 18, 16) == (False, False)
+    assert choose_layout("q8", bf16, 128, 128, 2, 32, 100, None) == (True, True)
+    assert choose_layout("tiled", bf16, 96, 96, 2, 8, 100, 16) == (True, False)
+    assert choose_layout("row_major", bf16, 128, 128, 4, 32, 1 << 20, 16) == (False, False)
+    import pytest
+    with pytest.raises(ValueError):
+        choose_layout("q8", bf16, 256, 256, 3, 32, 1000, 8)
+    with pytest.raises(ValueError):
+        choose_layout("q8", f32, 128, 128, 3, 32, 1000, 8)
+    with pytest.raises(ValueError):
+        choose_layout("tiled", f32, 128, 128, 3, 32, 1000, 8)

@@ -45,11 +45,11 @@ Q8_CASES = [
     (2, 16, 1024, 128, 32, 3, 30),      # 8 heads per tree
     (1, 16, 1100, 64, 16, 3, 33),       # 16 heads per tree, d = 64, fan-out 16
     (1, 20, 900, 64, 16, 2, 27),        # 20 heads per tree: two passes of the head loop
-    (1, 4, 3000, 256, 48, 2, 60),       # d = 256, fan-out 48 (3 tiles per block)
+    (1, 4, 3000, 128, 48, 2, 60),       # fan-out 48 (3 tiles per block)
     (1, 4, 5000, 128, 64, 3, 50),       # fan-out 64
     (2, 8, 40000, 128, 32, 4, 400),     # four levels
-    (1, 8, 3000, 256, 64, 2, 40),       # d = 256, fan-out 64, 8 heads: nodes scanned as two halves
-    (1, 16, 2600, 256, 64, 3, 30),      # the same with 16 heads
+    (1, 8, 3000, 128, 64, 2, 40),       # fan-out 64, 8 heads
+    (1, 16, 2600, 64, 64, 3, 30),       # d = 64, fan-out 64, 16 heads
 ]
 
 
