@@ -451,6 +451,85 @@ def timeline_report(a, w, index, searcher, q_d, taus, outs, W, total, scale):
                   f"mean {we[sel].mean():6.2f}  max {we[sel].max():6.2f}")
 
 
+# Search alone at the shapes the reference publishes (single head, d = 128, fp32, one unit-norm random
+# query, a threshold that keeps 10 keys; its figures are from an unnamed NVIDIA GPU on real Llama-3
+# keys that are not shipped): (N, fan-out, levels, published us, where)
+PUBLISHED_SEARCH = [
+    (10000, 4, 3, 8.16, "benchmark_area/cuda_bench/reports/three_level_filter_real.csv:2"),
+    (40000, 4, 3, 11.11, "benchmark_area/cuda_bench/reports/three_level_filter_real.csv:4"),
+    (90000, 4, 3, 14.43, "benchmark_area/cuda_bench/reports/three_level_filter_real.csv:7"),
+    (40000, 8, 2, 13.54, "benchmark_area/cuda_bench/reports/three_level_filter_real.csv:4"),
+    (90000, 8, 2, 20.65, "benchmark_area/cuda_bench/reports/three_level_filter_real.csv:7"),
+    (40000, 16, 3, 20.43, "benchmark_area/cuda_bench/reports/triton_benchmarking.csv:4"),
+    (40000, 32, 3, 34.74, "benchmark_area/cuda_bench/reports/triton_benchmarking.csv:4"),
+    (40000, 64, 3, 626.2, "benchmark_area/cuda_bench/reports/triton_benchmarking.csv:4"),
+    (90000, 32, 3, 45.97, "benchmark_area/cuda_bench/reports/triton_benchmarking.csv:7"),
+]
+
+
+def published_shapes(spreads=(0.5, 0.15)):
+    """`HIPSearcher.search` (dense output, as the reference's searcher returns it) at the shapes of
+    PUBLISHED_SEARCH, on synthetic keys: 256 Gaussian clusters of a given spread around unit-scale
+    centres, normalised.  The published figures are on real keys, whose balls prune (the
+    reference's own study counts 2512 leaf products for 10 000 keys at fan-out 4,
+    benchmark_area/pruning/notebooks/ball_pruning_power_results.csv:2); a spread of 0.5 gives keys
+    whose balls prune almost nothing, 0.15 keys that prune about as the real ones do, and the share
+    of the keys a query's walk reads is reported with every figure.  One JSON line."""
+    import torch
+
+    from hira_amd import _lib
+    from hira_amd.cache.threshold_finder import exact_topk
+    from hira_amd.indexer import HIPIndexer
+    from hira_amd.searcher import HIPSearcher
+
+    def replayed_us(f, n=100):
+        for _ in range(5):
+            f()
+        torch.cuda.synchronize()
+        st = torch.cuda.Stream()
+        st.wait_stream(torch.cuda.current_stream())
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(st):
+            with torch.cuda.graph(g, stream=st):
+                for _ in range(n):
+                    f()
+            g.replay()
+            st.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(st)
+            g.replay()
+            e1.record(st)
+            st.synchronize()
+        return e0.elapsed_time(e1) / n * 1e3
+
+    rows = []
+    for spread in spreads:
+        gen = torch.Generator().manual_seed(0)
+        for n, bf, levels, pub, where in PUBLISHED_SEARCH:
+            c = torch.randn(256, 128, generator=gen)
+            keys = torch.nn.functional.normalize(
+                c[torch.randint(0, 256, (n,), generator=gen)] + spread * torch.randn(n, 128, generator=gen), dim=-1)
+            q = torch.nn.functional.normalize(torch.randn(1, 128, generator=gen), dim=-1).cuda()
+            kd = keys[None, None].cuda()
+            idx = HIPIndexer(levels, 1, bf).build(kd)
+            th = exact_topk(kd[0], q, 10)
+            se = HIPSearcher()
+            stats = torch.zeros(1, _lib.HIRA_STATS_COLS, dtype=torch.int64, device="cuda")
+            out = se.search(q, th, idx, stats=stats)
+            assert int((out != 0).sum()) == 10
+            us = replayed_us(lambda: se.search(q, th, idx))
+            kq = kd[0, 0].float()
+            qt = q.float().T.contiguous()
+            dense = replayed_us(lambda: kq @ qt)
+            rows.append({"n": n, "fanout": bf, "levels": levels, "cluster_spread": spread,
+                         "us": round(us, 2), "published_us": pub, "published_at": where,
+                         "keys_read_share": round(float(stats[0, 0]) / n, 3), "torch_k_at_q_us": round(dense, 2)})
+            log(f"[bench] published shape N={n} fan-out {bf} levels {levels} spread {spread}: "
+                f"{us:.2f} us (published {pub}), keys read {rows[-1]['keys_read_share']:.2f} of N")
+            del idx, kd
+    print(json.dumps({"mode": "published_shapes", "dtype": "f32", "data": "synthetic", "rows": rows}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -478,6 +557,8 @@ def main():
                     help="also time the steps over this many copies of the index in turn "
                          "(each with its own memory, like the layers of a model); default: 8 "
                          "where one index fits the Infinity Cache, else none")
+    ap.add_argument("--published", action="store_true",
+                    help="search alone at the single-head shapes the reference publishes figures for")
     ap.add_argument("--context", type=int, default=0,
                     help="keys per KV head instead of the configuration's (a sweep point, not a "
                          "benchmark configuration)")
@@ -514,6 +595,11 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     dev = torch.device("cuda:0")
+    if a.published:
+        if a.lib:
+            _lib.use_library(a.lib)
+        published_shapes()
+        return
     if a.timeline:
         _lib.use_library(_lib.CSRC / "libhira_hip_timeline.so")
     elif a.lib:

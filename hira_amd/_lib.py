@@ -17,7 +17,7 @@ HIRA_MAX_LEVELS = 8
 HIRA_STATS_COLS = HIRA_MAX_LEVELS + 3  # counters per tree a search can fill in
 HIRA_F32, HIRA_BF16 = 0, 1
 HIRA_ROW_MAJOR, HIRA_TILE16, HIRA_TILE16_Q8 = 0, 1, 2
-HIRA_ABI_VERSION = 5
+HIRA_ABI_VERSION = 6
 
 _vp = C.c_void_p
 
@@ -68,10 +68,12 @@ class HiraSearchOut(C.Structure):
         ("dense", _vp),
         ("dense_stride", C.c_int64),
         ("dense_by_position", C.c_int32),
+        ("dense_fill", C.c_int32),
         ("sel_index", _vp),
         ("sel_score", _vp),
         ("sel_count", _vp),
         ("sel_cap", C.c_int32),
+        ("dense_fill_value", C.c_float),
         ("attn_out", _vp),
         ("stats", _vp),
     ]

@@ -46,6 +46,8 @@ struct SearchParams {
     float* dense;
     int64_t dense_stride;
     int32_t dense_by_position;
+    int32_t dense_fill;       // the kernels write dense_fill_value wherever no score goes
+    float dense_fill_value;
     int32_t* sel_index;
     float* sel_score;
     int32_t* sel_count;

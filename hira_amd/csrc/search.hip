@@ -258,6 +258,8 @@ static int search_impl(const HiraTree* tree, const HiraQuery* query, const HiraQ
     if (out->dense && !out->dense_by_position)
         HIRA_CHECK_ARG(out->dense_stride >= tree->size[0], "dense_stride %lld < %d slots",
                        (long long)out->dense_stride, tree->size[0]);
+    HIRA_CHECK_ARG(!(out->dense && out->dense_fill && out->dense_by_position),
+                   "dense_fill goes with key slots, not with positions");
     if (out->dense_by_position && (out->dense || out->sel_count))
         HIRA_CHECK_ARG(tree->perm != nullptr, "perm missing");
     if (out->sel_count)
@@ -311,6 +313,8 @@ static int search_impl(const HiraTree* tree, const HiraQuery* query, const HiraQ
     p.dense = out->dense;
     p.dense_stride = out->dense_stride;
     p.dense_by_position = out->dense_by_position;
+    p.dense_fill = out->dense != nullptr ? out->dense_fill : 0;
+    p.dense_fill_value = out->dense_fill_value;
     p.sel_index = out->sel_index;
     p.sel_score = out->sel_score;
     p.sel_count = out->sel_count;

@@ -559,6 +559,19 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
         // ---- gate: one tile per wave at a time ------------------------------------------------
         while (tl_mine < ntile) {  // uniform in the wave
             const int t1 = tile_of(tl_mine);
+            if constexpr (OUT) {
+                // the dense output's stretch under this tile starts out as the fill value (the
+                // barrier behind the gates has every wave wait for these stores, so the scores
+                // that any wave writes later come after them)
+                if (p.dense_fill) {
+                    const int r0 = t1 * 16 * bf, r1 = min(r0 + 16 * bf, p.size[0]);
+                    for (int g = 0; g < G; ++g) {
+                        const int head = p.group_size > 0 ? hoff + g : p.tree_q_heads[hoff + g];
+                        for (int i = r0 + lane; i < r1; i += 64)
+                            p.dense[(int64_t)head * p.dense_stride + i] = p.dense_fill_value;
+                    }
+                }
+            }
             const bool count_nodes = stats != nullptr && lane == 0;
             size_t span = 1;  // level-1 nodes under one node of the current level
             for (int l = 2; l < L; ++l) span *= (size_t)bf;

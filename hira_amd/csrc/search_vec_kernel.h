@@ -154,6 +154,17 @@ __global__ __launch_bounds__(256) void search_kernel(const SearchParams p) {
     const int block_rows = real_nodes ? p.bf : kPseudoBlock;
     const int klayout = is_queue ? HIRA_ROW_MAJOR : p.key_layout;
 
+    // The dense output's stretch under this wave's nodes starts out as the fill value; the
+    // scores of selected keys follow from the same wave, behind these stores.
+    if (p.dense_fill && !is_queue && node_first < node_last) {
+        const int r0 = node_first * block_rows, r1 = min(node_last * block_rows, n_rows);
+#pragma unroll
+        for (int g = 0; g < GMAX; ++g)
+            if (g < G)
+                for (int i = r0 + lane; i < r1; i += kWave)
+                    p.dense[(int64_t)qh[g] * p.dense_stride + i] = p.dense_fill_value;
+    }
+
     if constexpr (NGX == 1) {
         for (int n0 = node_first; n0 < node_last; n0 += RPW) {
             // -------- gates: lane group rg owns node n0 + rg -----------------------------

@@ -158,13 +158,13 @@ class HIPSearcher(BaseSearcher):
             self._workspace = torch.zeros(max(nbytes, 1), dtype=torch.uint8, device=device)
         return self._workspace
 
-    def _prepare_output_buffer(self, h_q: int, n: int, device) -> torch.Tensor:
-        """searcher/cuda.py:35-54."""
+    def _prepare_output_buffer(self, h_q: int, n: int, device, fill: bool = True) -> torch.Tensor:
+        """searcher/cuda.py:35-54.  fill=False: the search writes the fill value itself."""
         if self._tmp_out is None or not _on(self._tmp_out, device) or \
                 tuple(self._tmp_out.shape) != (h_q, n):
             self._tmp_out = torch.full((h_q, n), self.output_fill_value, device=device,
                                        dtype=torch.float32)
-        else:
+        elif fill:
             self._tmp_out.fill_(self.output_fill_value)
         return self._tmp_out
 
@@ -192,11 +192,15 @@ class HIPSearcher(BaseSearcher):
         space = index_space or self.index_space
         qs, keep = self._query_struct(query, threshold, indexer, q_head_to_kv, scaling)
         n = indexer.size[0] if space == "slot" else indexer.num_keys
-        dense = self._prepare_output_buffer(qs.num_q_heads, n, indexer.device)
+        # in slot space the search fills what it does not select itself: one launch per call
+        fused_fill = space == "slot"
+        dense = self._prepare_output_buffer(qs.num_q_heads, n, indexer.device, fill=not fused_fill)
         out = _lib.HiraSearchOut()
         out.dense = dense.data_ptr()
         out.dense_stride = dense.stride(0)
         out.dense_by_position = 1 if space == "position" else 0
+        out.dense_fill = 1 if fused_fill else 0
+        out.dense_fill_value = self.output_fill_value
         out.stats = None if stats is None else stats.data_ptr()
         self._run(indexer, qs, out, None)
         del keep

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define HIRA_ABI_VERSION 5
+#define HIRA_ABI_VERSION 6
 #define HIRA_MAX_LEVELS 8
 #define HIRA_STATS_COLS (HIRA_MAX_LEVELS + 3) /* counters per tree a search can fill in */
 
@@ -119,10 +119,14 @@ typedef struct HiraSearchOut {
      *     searcher/cuda.py:56-143): dense[h*dense_stride + i] = (q_h.k_i)*scaling[h] for
      *     every selected key, untouched elsewhere (caller pre-fills).  dense_by_position
      *     != 0: i = position of the key in insertion order (CPU searcher's index space);
-     *     0: i = key slot (GPU searcher's index space). */
+     *     0: i = key slot (GPU searcher's index space).  dense_fill != 0 (slots only): the
+     *     search writes dense_fill_value to every other element dense[h*dense_stride + i],
+     *     i < size[0], itself -- no pre-fill, one launch less (the reference fills its output
+     *     buffer before every search, searcher/cuda.py:35-54). */
     float* dense;
     int64_t dense_stride;
     int32_t dense_by_position;
+    int32_t dense_fill;
     /* (2) compact lists: for head h, sel_count[h] entries (unordered) of
      *     sel_index[h*sel_cap + j] (slot or position, as above) and sel_score (raw q.k).
      *     sel_count must be zeroed by the caller; entries beyond sel_cap are counted but
@@ -131,6 +135,7 @@ typedef struct HiraSearchOut {
     float* sel_score;
     int32_t* sel_count;
     int32_t sel_cap;
+    float dense_fill_value;
     /* (3) attention over the selected keys (+ the queue): out (H_q, Dv) fp32.
      *     Heads with an empty selection get zeros. */
     float* attn_out;

@@ -59,6 +59,10 @@ def test_struct_layout_matches_header():
     assert ctypes.sizeof(_lib.HiraLaunch) == 16
     assert _lib.HiraQuery.max_group.offset == 48 and _lib.HiraQuery.group_size.offset == 52
     assert _lib.HiraSearchOut.attn_out.offset == 56
+    # (the two fields of the fused fill sit in what used to be padding: older callers' structs,
+    # zero there, keep their meaning)
+    assert _lib.HiraSearchOut.dense_fill.offset == 20 and _lib.HiraSearchOut.dense_fill_value.offset == 52
+    assert ctypes.sizeof(_lib.HiraSearchOut) == 72
 
 
 def test_new_entry_points_validate_without_a_gpu():

@@ -155,6 +155,44 @@ def test_mfma_kernel_matches_oracle_and_vector_kernel(case, gpu_device):
     assert rel_err(full, ref_full) <= 2e-3
 
 
+@pytest.mark.parametrize("case", [
+    # h_kv, h_q, n, d, bf, levels, dtype, keep, kernel
+    (2, 6, 192, 128, 8, 3, torch.float32, 48, 1),
+    (3, 3, 203, 32, 4, 4, torch.float32, 25, 1),       # pad slots, batched gates
+    (2, 2, 300, 64, 8, 1, torch.float32, 30, 1),       # one level: flat scan
+    (2, 8, 2048, 128, 32, 3, torch.bfloat16, 41, 2),
+    (1, 12, 600, 64, 16, 3, torch.bfloat16, 30, 2),    # 12 heads a tree: two passes; a partial tile
+    (2, 8, 2048, 128, 32, 3, torch.bfloat16, 41, 1),
+], ids=lambda c: f"hkv{c[0]}_hq{c[1]}_n{c[2]}_d{c[3]}_bf{c[4]}_L{c[5]}_k{c[8]}")
+def test_search_fills_what_it_does_not_select(case, gpu_device):
+    """In slot space the search writes the fill value itself (HiraSearchOut.dense_fill; the
+    reference fills its buffer before every search, searcher/cuda.py:35-54): a buffer that
+    holds anything else beforehand comes back with the scores of the selected keys and the fill
+    value everywhere else, pad slots included; in position space the wrapper still pre-fills."""
+    from hira_amd.searcher.hip import HIPSearcher
+
+    h_kv, h_q, n, d, bf, nl, dtype, keep, kernel = case
+    print(f"case {case}", flush=True)
+    su = _setup(h_kv, h_q, n, d, bf, nl, dtype, seed=77 + n, keep=keep)
+    q, th = torch.from_numpy(su["q"]), torch.from_numpy(su["th"])
+    for fill in (0.0, -5.0):
+        se = HIPSearcher(kernel=kernel, output_fill_value=fill)
+        first = se.search(q, th, su["idx"]).clone()
+        se._tmp_out.fill_(7.0)                          # whatever an earlier call left behind
+        again = se.search(q, th, su["idx"])
+        assert torch.equal(first, again)
+        out = again.cpu().numpy()
+        want = np.where(su["valid"] & (su["s"] >= su["th"][:, None]), su["s"], np.float32(fill))
+        band = np.abs(su["s"] - su["th"][:, None]) <= 1e-5 * np.abs(su["th"][:, None])
+        ok = band | np.isclose(out, want, rtol=2e-5, atol=1e-6)
+        assert ok.all(), int((~ok).sum())
+        assert (out[~su["valid"]] == np.float32(fill)).all()
+        se._tmp_out.fill_(7.0)
+        pos = se.search(q, th, su["idx"], index_space="position").cpu().numpy()
+        assert not (pos == 7.0).any()
+        assert (pos != np.float32(fill)).sum() == (out != np.float32(fill)).sum()
+
+
 def test_mfma_kernel_is_refused_where_it_does_not_apply(gpu_device):
     from hira_amd.searcher.hip import HIPSearcher
 
