@@ -85,6 +85,7 @@ __global__ __launch_bounds__(256) void search_kernel(const SearchParams p) {
 
     extern __shared__ float smem[];
 
+    touch_kernel_arguments();
     const int lane = lane_id();
     const int wave = threadIdx.x >> 6;
     const int nwaves = blockDim.x >> 6;
