@@ -22,6 +22,16 @@ struct AssignCounting {
     int32_t* zero;
 };
 
+// The centroids that still take items, put side by side (packing rounds from the second on: most
+// blocks are full by then, and a round multiplies every unplaced item with every centroid it is
+// given).  ids (T, K): the centroids with room, in increasing order; count (T): how many; the
+// assignment then walks tiles and norms holding only those (same arrays' shapes as the full ones)
+// and translates the column it finds back through ids.  Both NULL: all centroids, as they lie.
+struct AssignOpen {
+    const int32_t* count;
+    const int32_t* ids;
+};
+
 // Exclusive prefix sums of n numbers by a workgroup of 256 threads, 1024 numbers a step; every
 // thread returns the total.
 template <typename Load, typename Store>
@@ -130,6 +140,9 @@ int launch_cent_prep(int dim, const float* cent, int K, int num_trees, const int
 int launch_assign_mfma(int dim, const void* x, int n_c, size_t x_tree_stride, const void* tiles,
                        const float* cn2, int K, int num_trees, const int32_t* list,
                        const int32_t* list_count, size_t list_stride, int32_t* assign, float* dist,
-                       const AssignCounting& counting, hipStream_t s);
+                       const AssignCounting& counting, const AssignOpen& open, hipStream_t s);
+int launch_open_centroids(int dim, const void* tiles, const float* cn2, const int32_t* fill, int bf,
+                          int K, int num_trees, int32_t* open_ids, int32_t* open_count,
+                          void* open_tiles, float* open_cn2, hipStream_t s);
 
 }  // namespace hira

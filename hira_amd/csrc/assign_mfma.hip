@@ -72,7 +72,7 @@ template <int KS, int RI>
 __device__ __forceinline__ void assign_items(
     const void* x, int n_c, size_t x_tree_stride, const uint4* tiles, const float* cn2, int Kt,
     const int32_t* list, int n_items, size_t list_stride, int32_t* assign, float* dist, int K,
-    const AssignCounting& ac) {
+    const AssignCounting& ac, const AssignOpen& open) {
     constexpr int D = 32 * KS;
     constexpr int TILE_CHUNKS = 2 * KS * 64;                 // hi and lo halves of 16 centroids
     constexpr int TPS = assign_stage(KS);
@@ -127,9 +127,11 @@ __device__ __forceinline__ void assign_items(
 
     // ---- all centroid tiles, staged through LDS TPS at a time (the last stage may hold fewer;
     // the arrays are padded to whole stages, their norms with +inf) ---------------------------
-    const int Ks = (Kt + TPS - 1) / TPS;  // stages
-    const uint4* tt = tiles + (size_t)t * Ks * STAGE_CHUNKS;
-    const float* n2t = cn2 + (size_t)t * Ks * (TPS * 16);
+    const int Ks_all = (Kt + TPS - 1) / TPS;  // stages a tree's arrays hold
+    // (centroids with room side by side: only the stages that hold any)
+    const int Ks = open.count ? min(((open.count[t] + 15) / 16 + TPS - 1) / TPS, Ks_all) : Ks_all;
+    const uint4* tt = tiles + (size_t)t * Ks_all * STAGE_CHUNKS;
+    const float* n2t = cn2 + (size_t)t * Ks_all * (TPS * 16);
     uint4 stage[CPT];
     float stage_n2 = 0.0f;
 #pragma unroll
@@ -142,7 +144,7 @@ __device__ __forceinline__ void assign_items(
         const float* n2buf = s_n2 + (st & 1) * (TPS * 16);
         // the next stage is on its way while this one is used (after the last stage: the last
         // one again, unused; straight-line code keeps `stage` in registers)
-        const int nst = min(st + 1, Ks - 1);
+        const int nst = min(st + 1, Ks - 1);  // (Ks >= 1 inside the loop)
 #pragma unroll
         for (int c = 0; c < CPT; ++c)
             stage[c] = tt[(size_t)nst * STAGE_CHUNKS + threadIdx.x + c * kAssignThreads];
@@ -218,7 +220,7 @@ __device__ __forceinline__ void assign_items(
     __builtin_amdgcn_wave_barrier();
     {
         // lane (kb, n) takes row n of operand tile kb: its item and ||x||^2 are its own
-        const int g = s_g[lane];
+        int g = s_g[lane];  // (meaningless in the lanes that hold no result: kb >= RI)
         const float b = s_b[lane];
         int it = item[0];
         float xx = x2[0];
@@ -229,6 +231,7 @@ __device__ __forceinline__ void assign_items(
                 xx = x2[ri];
             }
         if (kb < RI && it >= 0) {
+            if (open.ids != nullptr && g >= 0) g = open.ids[(size_t)t * K + g];  // column -> centroid
             assign[(size_t)t * n_c + it] = g;
             dist[(size_t)t * n_c + it] = fmaxf(b + xx, 0.0f);
             if (ac.counts != nullptr && g >= 0)
@@ -249,7 +252,7 @@ template <int KS, bool LISTED>
 __global__ __launch_bounds__(kAssignThreads, 2) void k_assign_mfma(
     const void* x, int n_c, size_t x_tree_stride, const uint4* tiles, const float* cn2, int Kt,
     const int32_t* list, const int32_t* list_count, size_t list_stride, int32_t* assign,
-    float* dist, int K, AssignCounting ac) {
+    float* dist, int K, AssignCounting ac, AssignOpen open) {
     const int t = blockIdx.y;
     const int n_items = LISTED ? list_count[t] : n_c;
     const bool narrow = LISTED && (long long)n_items * gridDim.y <= kAssignNarrowItems;
@@ -261,12 +264,71 @@ __global__ __launch_bounds__(kAssignThreads, 2) void k_assign_mfma(
     if ((int)blockIdx.x * per_block < n_items) {
         if (LISTED && narrow)
             assign_items<KS, 1>(x, n_c, x_tree_stride, tiles, cn2, Kt, list, n_items, list_stride,
-                                assign, dist, K, ac);
+                                assign, dist, K, ac, open);
         else
             assign_items<KS, kAssignRI>(x, n_c, x_tree_stride, tiles, cn2, Kt, list, n_items,
-                                        list_stride, assign, dist, K, ac);
+                                        list_stride, assign, dist, K, ac, open);
     }
     if (ac.counts != nullptr) finish_counts(ac, t, K, nblocks);
+}
+
+// ---- the centroids with room, side by side ---------------------------------------------------
+// one workgroup per tree: which centroids are not full, in order
+__global__ __launch_bounds__(256) void k_open_scan(const int32_t* fill, int K, int bf, int32_t* ids,
+                                                   int32_t* count) {
+    const int t = blockIdx.x;
+    const int32_t* ft = fill + (size_t)t * K;
+    int32_t* it = ids + (size_t)t * K;
+    const int total = block_exclusive_scan(
+        K, [&](int k) { return ft[k] < bf ? 1 : 0; },
+        [&](int k, int v) {
+            if (ft[k] < bf) it[v] = k;
+        });
+    if (threadIdx.x == 0) count[t] = total;
+}
+
+// one wave per tile of the side-by-side arrays: column i of tile c is centroid ids[16 c + i]; the
+// columns behind the last one, up to the end of the stage, are zeros with norm +inf
+template <int KS>
+__global__ __launch_bounds__(64) void k_open_gather(const uint4* tiles, const float* cn2,
+                                                    const int32_t* ids, const int32_t* count, int K,
+                                                    int Kt, uint4* otiles, float* ocn2) {
+    constexpr int TILE_CHUNKS = 2 * KS * 64;
+    constexpr int TPS = assign_stage(KS);
+    const int tile = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
+    const int no = count[t];
+    const int need = min((((no + 15) / 16 + TPS - 1) / TPS) * TPS, Kt);  // tiles the assignment will walk
+    if (tile >= need) return;
+    const uint4* src = tiles + (size_t)t * Kt * TILE_CHUNKS;
+    uint4* dst = otiles + ((size_t)t * Kt + tile) * TILE_CHUNKS;
+    const int i = lane & 15;
+    const int col = tile * 16 + i;
+    const int k = col < no ? ids[(size_t)t * K + col] : -1;
+#pragma unroll
+    for (int c0 = 0; c0 < TILE_CHUNKS; c0 += 64) {
+        const int ci = c0 + lane;  // (ci % 16 == i: a lane always moves chunks of its own column)
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (k >= 0) v = src[(size_t)(k >> 4) * TILE_CHUNKS + (ci - i) + (k & 15)];
+        dst[ci] = v;
+    }
+    if (lane < 16) ocn2[((size_t)t * Kt + tile) * 16 + i] = k >= 0 ? cn2[(size_t)t * Kt * 16 + k] : INFINITY;
+}
+
+int launch_open_centroids(int dim, const void* tiles, const float* cn2, const int32_t* fill, int bf,
+                          int K, int num_trees, int32_t* open_ids, int32_t* open_count,
+                          void* open_tiles, float* open_cn2, hipStream_t s) {
+    const int Kt = assign_tiles(K);
+    hipLaunchKernelGGL(k_open_scan, dim3(num_trees), dim3(256), 0, s, fill, K, bf, open_ids, open_count);
+    const dim3 grid(Kt, num_trees);
+    const uint4* tl = reinterpret_cast<const uint4*>(tiles);
+    uint4* ot = reinterpret_cast<uint4*>(open_tiles);
+    switch (dim) {
+        case 64: hipLaunchKernelGGL((k_open_gather<2>), grid, dim3(64), 0, s, tl, cn2, open_ids, open_count, K, Kt, ot, open_cn2); break;
+        case 128: hipLaunchKernelGGL((k_open_gather<4>), grid, dim3(64), 0, s, tl, cn2, open_ids, open_count, K, Kt, ot, open_cn2); break;
+        case 256: hipLaunchKernelGGL((k_open_gather<8>), grid, dim3(64), 0, s, tl, cn2, open_ids, open_count, K, Kt, ot, open_cn2); break;
+        default: return fail(HIRA_EINVAL, "MFMA assignment: dim %d", dim);
+    }
+    return HIRA_OK;
 }
 
 // centroid tiles per tree, in whole stages
@@ -294,7 +356,7 @@ int launch_cent_prep(int dim, const float* cent, int K, int num_trees, const int
 int launch_assign_mfma(int dim, const void* x, int n_c, size_t x_tree_stride, const void* tiles,
                        const float* cn2, int K, int num_trees, const int32_t* list,
                        const int32_t* list_count, size_t list_stride, int32_t* assign, float* dist,
-                       const AssignCounting& counting, hipStream_t s) {
+                       const AssignCounting& counting, const AssignOpen& open, hipStream_t s) {
     const int Kt = assign_tiles(K);
     // (a launch over a list: workgroups for the narrow shape, see kAssignNarrowItems)
     const int per_block = (kAssignThreads / 64) * (list != nullptr ? 1 : kAssignRI) * 16;
@@ -319,7 +381,7 @@ int launch_assign_mfma(int dim, const void* x, int n_c, size_t x_tree_stride, co
         }                                                                                           \
         hipLaunchKernelGGL((k_assign_mfma<KS, LISTED>), grid, dim3(kAssignThreads), smem, s, x, n_c, \
                            x_tree_stride, tl, cn2, Kt, list, list_count, list_stride, assign, dist, \
-                           K, counting);                                                            \
+                           K, counting, open);                                                      \
     }
 #define HIRA_ASSIGN_MFMA(KS)                                                                        \
     if (list != nullptr) HIRA_ASSIGN_MFMA_L(KS, true) else HIRA_ASSIGN_MFMA_L(KS, false)            \

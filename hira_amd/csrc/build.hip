@@ -730,6 +730,9 @@ struct BuildWs {
     float* cent_f32;
     void* cent_tiles;  // centroids as bf16 operand tiles (matrix-core assignment), or NULL
     float* cent_n2;
+    void* open_tiles;  // the same for the centroids with room, side by side (later packing rounds)
+    float* open_n2;
+    int32_t *open_ids, *open_count;
     int32_t *assign, *pos, *placed, *members, *ordered;
     int32_t* list[2];     // the items of a packing round, and those of the round after it
     int32_t* list_count;  // (2, T)
@@ -764,10 +767,17 @@ static void carve(const HiraTree* t, int n, void* ws, BuildWs* b) {
     b->cent_f32 = c.take<float>((size_t)T * k1 * D);
     b->cent_tiles = nullptr;
     b->cent_n2 = nullptr;
+    b->open_tiles = nullptr;
+    b->open_n2 = nullptr;
+    b->open_ids = b->open_count = nullptr;
     if (assign_on_mfma(t)) {
         const size_t kpad = (size_t)assign_tiles((int)k1) * 16;
         b->cent_tiles = c.take<char>((size_t)T * kpad * D * 4);  // hi and lo halves, 2 bytes each
         b->cent_n2 = c.take<float>((size_t)T * kpad);
+        b->open_tiles = c.take<char>((size_t)T * kpad * D * 4);
+        b->open_n2 = c.take<float>((size_t)T * kpad);
+        b->open_ids = c.take<int32_t>((size_t)T * k1);
+        b->open_count = c.take<int32_t>((size_t)T);
     }
     b->assign = c.take<int32_t>((size_t)T * n);
     b->pos = c.take<int32_t>((size_t)T * n);
@@ -872,12 +882,19 @@ static int build_impl(const HiraTree* t, const void* keys_in, const void* values
         // a round: the assignment (which also counts the items of every centroid and turns the
         // counts into offsets), the buckets, and what the round does with every bucket
         auto assign_round = [&](const int32_t* list, const int32_t* lcnt, const int32_t* fill,
-                                int32_t* zero) -> int {
+                                int32_t* zero, bool only_open) -> int {
             const AssignCounting ac{w.counts, w.pos, w.done, w.offsets, zero};
             int rc;
-            if (on_mfma)
+            if (on_mfma && only_open) {
+                rc = launch_open_centroids(D, w.cent_tiles, w.cent_n2, w.fill, bf, Kl, NT, w.open_ids,
+                                           w.open_count, w.open_tiles, w.open_n2, s);
+                if (rc == HIRA_OK)
+                    rc = launch_assign_mfma(D, x, n_c, xs, w.open_tiles, w.open_n2, Kl, NT, list, lcnt,
+                                            (size_t)n_c, w.assign, w.dist, ac,
+                                            AssignOpen{w.open_count, w.open_ids}, s);
+            } else if (on_mfma)
                 rc = launch_assign_mfma(D, x, n_c, xs, w.cent_tiles, w.cent_n2, Kl, NT, list, lcnt,
-                                        (size_t)n_c, w.assign, w.dist, ac, s);
+                                        (size_t)n_c, w.assign, w.dist, ac, AssignOpen{nullptr, nullptr}, s);
             else
                 rc = launch_assign<T>(lpr, g_assign, s, x, n_c, xs, w.cent_f32, Kl, D, fill, bf, list,
                                       lcnt, (size_t)n_c, w.assign, w.dist, ac);
@@ -887,7 +904,7 @@ static int build_impl(const HiraTree* t, const void* keys_in, const void* values
             return HIRA_OK;
         };
         for (int it = 0; it < niter; ++it) {
-            const int rc = assign_round(live, live_cnt, ragged ? w.fill : nullptr, nullptr);
+            const int rc = assign_round(live, live_cnt, ragged ? w.fill : nullptr, nullptr, false);
             if (rc != HIRA_OK) return rc;
             hipLaunchKernelGGL((k_bucket_mean<T>), g_cent, dim3(kBucketThreads), 0, s, x, xs, n_c,
                                Kl, D, w.offsets, w.members, w.ordered, ragged ? w.fill : nullptr, bf,
@@ -899,7 +916,9 @@ static int build_impl(const HiraTree* t, const void* keys_in, const void* values
             const int32_t* list = r == 0 ? live : w.list[r & 1];
             const int32_t* lcnt = r == 0 ? live_cnt : w.list_count + (size_t)(r & 1) * NT;
             int32_t* next_cnt = w.list_count + (size_t)((r + 1) & 1) * NT;
-            const int rc = assign_round(list, lcnt, w.fill, next_cnt);
+            // (from the second round on most blocks are full: the assignment then sees only the
+            // centroids with room, side by side; worth its two small launches from 32 tiles on)
+            const int rc = assign_round(list, lcnt, w.fill, next_cnt, r >= 1 && Kl >= 512);
             if (rc != HIRA_OK) return rc;
             hipLaunchKernelGGL(k_bucket_accept, g_cent, dim3(kBucketThreads), 0, s, w.members,
                                w.offsets, w.dist, n_c, Kl, bf, w.fill, w.slots[l], w.placed,
@@ -1125,7 +1144,7 @@ extern "C" int hira_nearest(const void* x, int32_t dtype, int32_t num_trees, int
         rc = launch_cent_prep(dim, centers, m, num_trees, b.fill, 1, b.tiles, b.n2, s);
         if (rc == HIRA_OK)
             rc = launch_assign_mfma(dim, x, n, (size_t)n, b.tiles, b.n2, m, num_trees, nullptr,
-                                    nullptr, 0, idx, dist2, AssignCounting{}, s);
+                                    nullptr, 0, idx, dist2, AssignCounting{}, AssignOpen{nullptr, nullptr}, s);
     } else {
         const int epl = dtype == HIRA_F32 ? 4 : 8;
         int lpr = 2;
