@@ -333,8 +333,9 @@ __global__ __launch_bounds__(64 * kMfmaWaves, 2) void search_mfma_kernel(const S
     // rows, and lane (row group rg, chunk cc) sums columns 8 cc .. 8 cc + 7 of the rows of its
     // group in acc8; the row groups' sums meet before the merge.  (A quarter of the load
     // instructions and half the instructions per row of the gather below, which holds a row in
-    // 4 bytes a lane and has the registers that the tiles in flight of several rounds leave.)
-    constexpr bool WIDE = ONE && !Q8 && GS <= 8 && KS == 4;
+    // 4 bytes a lane.  A launch of several rounds keeps the next round's tiles in flight during
+    // the gather: its registers take the eight columns of up to four heads, 233 in all.)
+    constexpr bool WIDE = (ONE ? GS <= 8 : GS <= 4) && !Q8 && KS == 4;
     constexpr int LR = D / 8;     // lanes per value row
     constexpr int RPI = 64 / LR;  // rows per load instruction
     const int rg = lane / LR, cc = lane % LR;
