@@ -716,7 +716,10 @@ def main():
         ev0.record(stream)
         graph.replay()
         ev1.record(stream)
-        stream.synchronize()
+        # (the host polls for the end instead of sleeping until it is woken: a blocking wait's
+        # wake-up is tens of microseconds, which a run of few steps would carry in its figure)
+        while not ev1.query():
+            pass
         torch.cuda.synchronize()
         wall_ms = (time.perf_counter() - t0) * 1e3
         graph_ms = ev0.elapsed_time(ev1)
