@@ -12,12 +12,18 @@
 // k_cent_prep   centroids (T, K, D) fp32 -> tiles of 16 centroids, hi and lo halves, in the
 //               operand layout (chunk (s, kb, i) of 16 bytes at s*64 + kb*16 + i), plus
 //               ||hi + lo||^2; a centroid that is full (fill[k] >= bf) or past K gets +inf.
+//               (hira_nearest; the build's kernels write the tile of a centroid where they make
+//               the centroid, assign.h.)
 // k_assign_mfma a workgroup of 4 waves owns 256 items (64 a wave: 4 operand tiles kept in
 //               registers) and walks all centroid tiles; four tiles at a time are staged once
 //               per workgroup in LDS (double buffered, one barrier a stage).  Lane (n, kb) of a wave sees
 //               the products of its centroid column n with rows 4*kb + j, keeps the best
 //               (value, index) per row, and the 16 columns are merged at the end
-//               (lowest index on ties).
+//               (lowest index on ties).  For the build it also counts the items of every
+//               centroid and, in a tree's last workgroup, turns the counts into offsets
+//               (AssignCounting); over a short list of items it spreads them 64 a workgroup; and
+//               it can walk the centroids with room only, put side by side by k_open_scan /
+//               k_open_gather (AssignOpen).
 #include "assign.h"
 
 namespace hira {
