@@ -467,6 +467,14 @@ PUBLISHED_SEARCH = [
 ]
 
 
+# (window, published ms per call with two / three levels: the "v2" columns, its current code)
+PUBLISHED_UPDATE = [
+    (64, 1.02, 2.25, "benchmark_area/updating_index/cuda/cuda_updating_results.csv:2"),
+    (1024, 1.45, 3.58, "benchmark_area/updating_index/cuda/cuda_updating_results.csv:22"),
+    (4096, 2.59, 6.73, "benchmark_area/updating_index/cuda/cuda_updating_results.csv:32"),
+]
+
+
 def published_shapes(spreads=(0.5, 0.15)):
     """`HIPSearcher.search` (dense output, as the reference's searcher returns it) at the shapes of
     PUBLISHED_SEARCH, on synthetic keys: 256 Gaussian clusters of a given spread around unit-scale
@@ -527,7 +535,35 @@ def published_shapes(spreads=(0.5, 0.15)):
             log(f"[bench] published shape N={n} fan-out {bf} levels {levels} spread {spread}: "
                 f"{us:.2f} us (published {pub}), keys read {rows[-1]['keys_read_share']:.2f} of N")
             del idx, kd
-    print(json.dumps({"mode": "published_shapes", "dtype": "f32", "data": "synthetic", "rows": rows}), flush=True)
+    # ---- the reference's update benchmark (benchmark_area/updating_index/cuda/cuda_updating_bench.ipynb:
+    # one head, d = 128, fp32, fan-out 8, an index of 10 000 keys grown to 90 000 in windows; mean
+    # time per update call, host clock, synchronised before AND after the call here)
+    upd = []
+    gen = torch.Generator().manual_seed(42)
+    c = torch.randn(256, 128, generator=gen)
+    allk = torch.nn.functional.normalize(
+        c[torch.randint(0, 256, (90000,), generator=gen)] + 0.15 * torch.randn(90000, 128, generator=gen),
+        dim=-1)[None, None].cuda()
+    for window, pub2, pub3, where in PUBLISHED_UPDATE:
+        for levels, pub in ((2, pub2), (3, pub3)):
+            idx = HIPIndexer(levels, 1, 8).build(allk[:, :, :10000])
+            torch.cuda.synchronize()
+            times = []
+            for at in range(10000, 90000 - window + 1, window):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                idx.update(allk[:, :, at:at + window])
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t0)
+            assert idx.num_keys == 10000 + len(times) * window
+            times = times[2:]  # (the first calls load code objects)
+            upd.append({"window": window, "levels": levels, "ms_per_call": round(1e3 * sum(times) / len(times), 4),
+                        "calls": len(times), "published_ms": pub, "published_at": where})
+            log(f"[bench] published update: window {window}, {levels} levels: "
+                f"{upd[-1]['ms_per_call']:.3f} ms per call (published {pub})")
+            del idx
+    print(json.dumps({"mode": "published_shapes", "dtype": "f32", "data": "synthetic", "rows": rows,
+                      "updates": upd}), flush=True)
 
 
 def main():
