@@ -17,7 +17,7 @@ HIRA_MAX_LEVELS = 8
 HIRA_STATS_COLS = HIRA_MAX_LEVELS + 3  # counters per tree a search can fill in
 HIRA_F32, HIRA_BF16 = 0, 1
 HIRA_ROW_MAJOR, HIRA_TILE16, HIRA_TILE16_Q8 = 0, 1, 2
-HIRA_ABI_VERSION = 6
+HIRA_ABI_VERSION = 7
 
 _vp = C.c_void_p
 
@@ -128,6 +128,11 @@ SYMBOLS = {
     "hira_sparse_attention": (
         C.c_int,
         [C.POINTER(HiraTree), C.POINTER(HiraQuery), _vp, _vp, _vp, C.c_int32, _vp, _vp],
+    ),
+    "hira_update_threshold": (
+        C.c_int,
+        [C.POINTER(HiraTree), _vp, _vp, C.c_int32, _vp, _vp, C.c_int32, C.POINTER(HiraQuery),
+         C.c_int32, C.c_int32, _vp, _vp],
     ),
     "hira_threshold": (
         C.c_int,

@@ -25,6 +25,7 @@
 // bound that the search for a node with room starts from and raises as it learns more (0 is
 // always valid; whoever lowers a count of a level-1 node from outside must lower it too).
 #include "rows.h"
+#include "threshold_kernel.h"
 
 namespace hira {
 
@@ -326,6 +327,30 @@ __global__ __launch_bounds__(kUpdThreads) void k_update(const UpdateParams p) {
         update_one_key<T>(p, (int)blockIdx.x, i, sm, red_f, red_i, s_dist, s_rad);
 }
 
+// An append of a few keys per tree and the thresholds of a decode step in one launch: the first
+// `trees` workgroups append (their first kUpdThreads threads; the others leave at once, and a
+// barrier counts only the waves still there), the ones behind them take a head each.  The two
+// halves share nothing: the sample is not touched by the append.
+template <typename T, int E>
+__global__ __launch_bounds__(kTauThreads) void k_update_threshold(
+    const UpdateParams p, const int trees, const T* __restrict__ samples, const int S,
+    const T* __restrict__ q, const int32_t* __restrict__ tree_q_off,
+    const int32_t* __restrict__ tree_q_heads, const int group_size, const int method, const int k,
+    float* __restrict__ tau) {
+    extern __shared__ float sm[];
+    __shared__ float red_f[4];
+    __shared__ int red_i[4];
+    __shared__ float s_dist[HIRA_MAX_LEVELS], s_rad[HIRA_MAX_LEVELS];
+    if ((int)blockIdx.x < trees) {  // uniform in the workgroup
+        if (threadIdx.x >= kUpdThreads) return;
+        for (int i = 0; i < p.m; ++i)
+            update_one_key<T>(p, (int)blockIdx.x, i, sm, red_f, red_i, s_dist, s_rad);
+        return;
+    }
+    threshold_block<T, E>(samples, S, p.dim, q, tree_q_off, tree_q_heads, group_size, trees, method, k,
+                          tau, (int)blockIdx.x - trees);
+}
+
 // The general way as a call (the kernel below needs it now and then: its loop stays small, and the
 // compiler keeps the loop's values in registers instead of asking for them again every key).
 template <typename T>
@@ -618,9 +643,10 @@ __global__ __launch_bounds__(kUpdThreads) void k_update_window(const UpdateParam
 
 using namespace hira;
 
-/* see include/hira_hip.h */
-extern "C" int hira_update(const HiraTree* tree, const void* new_keys, const void* new_values,
-                           int32_t m, int32_t* state, void* stream) {
+// hira_update's checks and the kernels' arguments; *window: the launch takes the window kernel
+static int update_arguments(const HiraTree* tree, const void* new_keys, const void* new_values,
+                            int32_t m, int32_t* state, UpdateParams* out, bool* window,
+                            size_t* smem, size_t* smem_w) {
     HIRA_CHECK_ARG(tree != nullptr && new_keys != nullptr && state != nullptr,
                    "tree / new_keys / state missing");
     HIRA_CHECK_ARG(tree->dtype == HIRA_F32 || tree->dtype == HIRA_BF16, "dtype %d", tree->dtype);
@@ -631,9 +657,11 @@ extern "C" int hira_update(const HiraTree* tree, const void* new_keys, const voi
     HIRA_CHECK_ARG(tree->keys && tree->perm, "keys / perm missing");
     HIRA_CHECK_ARG((new_values == nullptr) || tree->values != nullptr,
                    "values given but the index holds none");
-    if (m == 0) return HIRA_OK;
-    UpdateParams p;
+    UpdateParams& p = *out;
     memset(&p, 0, sizeof(p));
+    *window = false;
+    *smem = *smem_w = 0;
+    if (m == 0) return HIRA_OK;  // nothing to append: the callers launch nothing for it
     p.keys = tree->keys;
     p.values = tree->values;
     p.perm = tree->perm;
@@ -662,17 +690,29 @@ extern "C" int hira_update(const HiraTree* tree, const void* new_keys, const voi
     p.new_values = new_values;
     p.m = m;
     p.state = state;
-    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    const size_t smem = 2 * (size_t)tree->dim * sizeof(float);
+    *smem = 2 * (size_t)tree->dim * sizeof(float);
     // windows of a few keys and more: the nodes with room are read into LDS once (where they fit:
     // 48 centres of up to 256 columns beside the rest)
-    const size_t cand_bytes = smem + (size_t)kCandMax * tree->dim * sizeof(float);
+    const size_t cand_bytes = *smem + (size_t)kCandMax * tree->dim * sizeof(float);
     const size_t row_bytes = (size_t)(tree->dim + tree->vdim) * sizeof(float);
     int chunk = cand_bytes + row_bytes <= 60 * 1024 ? (int)((60 * 1024 - cand_bytes) / row_bytes) : 0;
     chunk = chunk > 16 ? 16 : chunk;
-    const bool window = m >= 4 && tree->num_levels >= 2 && chunk >= 1;
-    const size_t smem_w = cand_bytes + (size_t)chunk * row_bytes;
+    *window = m >= 4 && tree->num_levels >= 2 && chunk >= 1;
+    *smem_w = cand_bytes + (size_t)chunk * row_bytes;
     p.chunk = chunk;
+    return HIRA_OK;
+}
+
+/* see include/hira_hip.h */
+extern "C" int hira_update(const HiraTree* tree, const void* new_keys, const void* new_values,
+                           int32_t m, int32_t* state, void* stream) {
+    UpdateParams p;
+    bool window;
+    size_t smem, smem_w;
+    if (const int rc = update_arguments(tree, new_keys, new_values, m, state, &p, &window, &smem, &smem_w))
+        return rc;
+    if (m == 0) return HIRA_OK;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     if (window) {
         if (tree->dtype == HIRA_F32)
             hipLaunchKernelGGL(k_update_window<float>, dim3(tree->num_trees), dim3(kUpdThreads), smem_w, s, p);
@@ -684,5 +724,53 @@ extern "C" int hira_update(const HiraTree* tree, const void* new_keys, const voi
         hipLaunchKernelGGL(k_update<bf16_t>, dim3(tree->num_trees), dim3(kUpdThreads), smem, s, p);
     }
     HIRA_CHECK_LAUNCH("update kernel");
+    return HIRA_OK;
+}
+
+namespace hira {
+template <typename T>
+static void launch_update_threshold(int e, const UpdateParams& p, const HiraTree* tree, size_t smem,
+                                    hipStream_t s, const void* samples, int S, const HiraQuery* qu,
+                                    int method, int k, float* tau) {
+    const T* x = static_cast<const T*>(samples);
+    const T* q = static_cast<const T*>(qu->q);
+    const dim3 grid(tree->num_trees + qu->num_q_heads), block(kTauThreads);
+#define HIRA_UT_LAUNCH(E)                                                                         \
+    hipLaunchKernelGGL((k_update_threshold<T, E>), grid, block, smem, s, p, tree->num_trees, x, S, \
+                       q, qu->tree_q_off, qu->tree_q_heads, qu->group_size, method, k, tau)
+    if (e == 1) HIRA_UT_LAUNCH(1);
+    else if (e == 2) HIRA_UT_LAUNCH(2);
+    else HIRA_UT_LAUNCH(4);
+#undef HIRA_UT_LAUNCH
+}
+}  // namespace hira
+
+/* see include/hira_hip.h */
+extern "C" int hira_update_threshold(const HiraTree* tree, const void* new_keys,
+                                     const void* new_values, int32_t m, int32_t* state,
+                                     const void* samples, int32_t num_samples,
+                                     const HiraQuery* query, int32_t method, int32_t k,
+                                     float* tau_out, void* stream) {
+    UpdateParams p;
+    bool window;
+    size_t smem, smem_w;
+    if (const int rc = update_arguments(tree, new_keys, new_values, m, state, &p, &window, &smem, &smem_w))
+        return rc;
+    if (const int rc = check_threshold_arguments(samples, tree->dtype, tree->num_trees, num_samples,
+                                                 tree->dim, query, method, k, tau_out))
+        return rc;
+    if (m == 0 || window) {
+        // nothing to append, or a window that takes the window kernel: the two launches
+        if (const int rc = hira_update(tree, new_keys, new_values, m, state, stream)) return rc;
+        return hira_threshold(samples, tree->dtype, tree->num_trees, num_samples, tree->dim, query,
+                              method, k, tau_out, stream);
+    }
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const int e = threshold_sort_registers(num_samples);
+    if (tree->dtype == HIRA_F32)
+        launch_update_threshold<float>(e, p, tree, smem, s, samples, num_samples, query, method, k, tau_out);
+    else
+        launch_update_threshold<bf16_t>(e, p, tree, smem, s, samples, num_samples, query, method, k, tau_out);
+    HIRA_CHECK_LAUNCH("update + threshold kernel");
     return HIRA_OK;
 }

@@ -339,13 +339,7 @@ class DecodePlan:
         return self.lib.hira_search_workspace_bytes(
             C.byref(self.tree), C.byref(fake_q), C.byref(self.queue), C.byref(self.launch))
 
-    def run(self, query: torch.Tensor, threshold: torch.Tensor, out: torch.Tensor,
-            stream: Optional[int] = None, queue_keys: Optional[torch.Tensor] = None,
-            queue_values: Optional[torch.Tensor] = None, queue_len: Optional[int] = None) -> None:
-        """queue_keys / queue_values: (..., cap, D) / (..., cap, Dv) contiguous, tree dtype, the
-        leading dimensions amounting to T trees: keys not in the index yet, attended by every
-        head of their tree; the first `queue_len` rows of every tree are in use (all `cap`
-        when not given)."""
+    def _follow_index(self) -> None:
         if self.indexer.tree_struct() is not self.tree:  # the index grew since the plan was made
             self.tree = self.indexer.tree_struct()
             need = self._workspace_need()
@@ -354,6 +348,15 @@ class DecodePlan:
             self.ws_bytes = need
             self._refs = (C.byref(self.tree), C.byref(self.query), C.byref(self.out),
                           C.byref(self.launch))
+
+    def run(self, query: torch.Tensor, threshold: torch.Tensor, out: torch.Tensor,
+            stream: Optional[int] = None, queue_keys: Optional[torch.Tensor] = None,
+            queue_values: Optional[torch.Tensor] = None, queue_len: Optional[int] = None) -> None:
+        """queue_keys / queue_values: (..., cap, D) / (..., cap, Dv) contiguous, tree dtype, the
+        leading dimensions amounting to T trees: keys not in the index yet, attended by every
+        head of their tree; the first `queue_len` rows of every tree are in use (all `cap`
+        when not given)."""
+        self._follow_index()
         self.query.q = query.data_ptr()
         self.query.tau = threshold.data_ptr()
         self.out.attn_out = out.data_ptr()
@@ -377,10 +380,13 @@ class DecodePlan:
                     out: torch.Tensor, stream: Optional[int] = None,
                     queue_keys: Optional[torch.Tensor] = None,
                     queue_values: Optional[torch.Tensor] = None,
-                    queue_len: Optional[int] = None) -> torch.Tensor:
+                    queue_len: Optional[int] = None, append=None) -> torch.Tensor:
         """A decode step whose thresholds come from a key sample (T, S, D), tree dtype,
         contiguous: ``hira_threshold`` ("sample_max" or "sample_mean_topk" with k) writes them
-        into a buffer of the plan, ``run`` follows on the same stream.  Returns that buffer."""
+        into a buffer of the plan, ``run`` follows on the same stream.  Returns that buffer.
+        ``append`` = (new_keys (T, m, D), new_values (T, m, Dv) or None, state): the step first
+        appends these rows to the index (``hira_update``'s arguments), in the launch that takes
+        the thresholds (``hira_update_threshold``)."""
         if self.tau_buf is None:
             self.tau_buf = torch.empty((self.query.num_q_heads,), dtype=torch.float32,
                                        device=self.indexer.device)
@@ -391,11 +397,20 @@ class DecodePlan:
                              f"({self.tree.num_trees}, S, {self.tree.dim}) {self.indexer.dtype}")
         if stream is None:
             stream = _lib.current_stream(self.indexer.device)
+        self._follow_index()
         self.query.q = query.data_ptr()
-        rc = self.lib.hira_threshold(
-            samples.data_ptr(), self.tree.dtype, self.tree.num_trees, int(samples.shape[1]),
-            self.tree.dim, self._refs[1], 0 if method == "sample_max" else 1, int(k),
-            self.tau_buf.data_ptr(), stream)
+        rule = 0 if method == "sample_max" else 1
+        if append is not None:
+            new_keys, new_values, state = append
+            rc = self.lib.hira_update_threshold(
+                self._refs[0], new_keys.data_ptr(),
+                new_values.data_ptr() if new_values is not None else None,
+                int(new_keys.shape[-2]), state.data_ptr(), samples.data_ptr(),
+                int(samples.shape[1]), self._refs[1], rule, int(k), self.tau_buf.data_ptr(), stream)
+        else:
+            rc = self.lib.hira_threshold(
+                samples.data_ptr(), self.tree.dtype, self.tree.num_trees, int(samples.shape[1]),
+                self.tree.dim, self._refs[1], rule, int(k), self.tau_buf.data_ptr(), stream)
         if rc:
             _lib.check(rc)
         self.run(query, self.tau_buf, out, stream, queue_keys, queue_values, queue_len)
@@ -404,9 +419,9 @@ class DecodePlan:
 
 class StreamingStep:
     """One decode step over a growing index as ONE captured HIP graph: append a key/value per
-    tree (``hira_update``), thresholds from a key sample (``hira_threshold``; optional),
-    search + sparse attention (``hira_search``) -- no host work between the launches and no
-    read-back.  The graph works on fixed device buffers that ``step`` fills:
+    tree (``hira_update``), thresholds from a key sample (optional; then ``hira_update_threshold``
+    does both in one launch), search + sparse attention (``hira_search``) -- no host work between
+    the launches and no read-back.  The graph works on fixed device buffers that ``step`` fills:
     ``new_keys`` (T, 1, D), ``new_values`` (T, 1, Dv), ``query`` (H_q, D), ``threshold`` (H_q)
     and writes ``out`` (H_q, Dv).  It is good for ``horizon`` steps (the index reserves room for
     that many appends and searches with level sizes fixed at their bound); ``refresh`` reads
@@ -443,14 +458,16 @@ class StreamingStep:
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.stream(stream):
             with torch.cuda.graph(self.graph, stream=stream):
-                _lib.check(lib.hira_update(C.byref(tree), self.new_keys.data_ptr(),
-                                           self.new_values.data_ptr(), 1, idx._state.data_ptr(),
-                                           stream.cuda_stream))
                 if self.samples is not None:
+                    # the append and the thresholds share a launch
                     self.plan.tau_buf = self.threshold
                     self.plan.run_sampled(self.query, self.samples, self.method, self.k, self.out,
-                                          stream=stream.cuda_stream)
+                                          stream=stream.cuda_stream,
+                                          append=(self.new_keys, self.new_values, idx._state))
                 else:
+                    _lib.check(lib.hira_update(C.byref(tree), self.new_keys.data_ptr(),
+                                               self.new_values.data_ptr(), 1, idx._state.data_ptr(),
+                                               stream.cuda_stream))
                     self.plan.run(self.query, self.threshold, self.out, stream=stream.cuda_stream)
         torch.cuda.current_stream(idx.device).wait_stream(stream)
         self.left = self.horizon

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define HIRA_ABI_VERSION 6
+#define HIRA_ABI_VERSION 7
 #define HIRA_MAX_LEVELS 8
 #define HIRA_STATS_COLS (HIRA_MAX_LEVELS + 3) /* counters per tree a search can fill in */
 
@@ -311,6 +311,20 @@ enum { HIRA_TAU_SAMPLE_MAX = 0, HIRA_TAU_SAMPLE_MEAN_TOPK = 1 };
 int hira_threshold(const void* samples, int32_t dtype, int32_t num_trees, int32_t num_samples,
                    int32_t dim, const HiraQuery* query, int32_t method, int32_t k,
                    float* tau_out, void* stream);
+
+/*
+ * hira_update and hira_threshold of one decode step as ONE launch, for a step that appends a key
+ * per tree and takes its thresholds from a key sample: the reference does the two from Python
+ * one after the other (cache/hira_cache.py:121-153 appends, cache/threshold_finder.py:1-14 names
+ * the rules), and the two share no data, so one launch's workgroups can do both (a launch less
+ * per token: some 6 us).  Arguments and results are those of the two calls, bit for bit; the
+ * samples have the tree's dtype, dim and tree count.  A window that hira_update places with its
+ * window kernel (m >= 4 on two or more levels) and m = 0 are served by the two launches.
+ */
+int hira_update_threshold(const HiraTree* tree, const void* new_keys, const void* new_values,
+                          int32_t m, int32_t* state, const void* samples, int32_t num_samples,
+                          const HiraQuery* query, int32_t method, int32_t k, float* tau_out,
+                          void* stream);
 
 /*
  * Softmax attention over given lists of selected keys, for callers that edit the selection

@@ -455,3 +455,74 @@ def test_a_window_placed_at_once_equals_key_by_key(t, n0, m, d, bf, nl, dtype, l
     if layout == "q8":
         assert torch.equal(a.keys8, b.keys8) and torch.equal(a.keps[:, :a.size[1]], b.keps[:, :b.size[1]])
     _check_tree(a, keys[:, :n0 + m + 7], keys[:, :n0 + m + 7])
+
+
+@pytest.mark.parametrize("dtype,d,m,s,method,k", [
+    (torch.bfloat16, 128, 1, 400, 1, 6),     # a key per tree, few of up to 1024 samples
+    (torch.bfloat16, 128, 3, 1500, 1, 40),   # three keys, the sort with two registers a thread
+    (torch.bfloat16, 64, 2, 3000, 0, 1),     # the maximum of 3000 samples
+    (torch.float32, 128, 1, 700, 1, 20),
+    (torch.float32, 32, 3, 2500, 1, 300),    # four registers a thread
+    (torch.bfloat16, 128, 6, 400, 1, 6),     # a window: served by the two launches
+    (torch.bfloat16, 128, 0, 400, 1, 6),     # nothing to append
+])
+def test_append_and_thresholds_in_one_launch_equal_the_two_calls(dtype, d, m, s, method, k, gpu_device):
+    """hira_update_threshold == hira_update followed by hira_threshold, bit for bit: the
+    thresholds, the update state and every array of the tree, over several calls in a row."""
+    import ctypes as C
+
+    from hira_amd import _lib
+    from hira_amd.indexer.hip import HIPIndexer
+    from hira_amd.searcher.hip import HIPSearcher
+
+    t, h_q, bf, n0, calls = 3, 12, 8, 3200, 40
+    rnd = bf16_round if dtype == torch.bfloat16 else (lambda x: x)
+    keys = rnd(clustered_keys(t, n0 + calls * max(m, 1), d, seed=77, clusters=30))
+    K = torch.from_numpy(keys)[None].to(dtype).cuda()
+    a = HIPIndexer(3, 1, bf).build(K[:, :, :n0], K[:, :, :n0])
+    b = HIPIndexer(3, 1, bf).build(K[:, :, :n0], K[:, :, :n0])
+    se = HIPSearcher()
+    plans = [se.plan_attention(i, h_q, scaling=torch.full((h_q,), d ** -0.5)) for i in (a, b)]
+    for i in (a, b):
+        i.begin_unsynced(calls * max(m, 1))
+    samples = K[0][:, torch.randperm(n0, generator=torch.Generator().manual_seed(5))[:s].sort().values]
+    samples = samples.contiguous()
+    assert samples.shape == (t, s, d)
+    lib = _lib.lib()
+    stream = _lib.current_stream(a.device)
+    tau_a = torch.zeros(h_q, dtype=torch.float32, device="cuda")
+    tau_b = torch.zeros_like(tau_a)
+    for c in range(calls):
+        # (m = 0: a buffer that is not read, since the calls refuse a null pointer)
+        nk = K[0][:, n0 + c * m:n0 + (c + 1) * m].contiguous() if m else K[0][:, :1].contiguous()
+        q = torch.from_numpy(rnd(random_query(h_q, d, seed=900 + c))).to(dtype).cuda()
+        for p in plans:
+            p.query.q = q.data_ptr()
+        ta, tb = a.tree_struct(), b.tree_struct()
+        _lib.check(lib.hira_update(C.byref(ta), nk.data_ptr(), nk.data_ptr(), m, a._state.data_ptr(), stream))
+        _lib.check(lib.hira_threshold(samples.data_ptr(), ta.dtype, t, s, d, C.byref(plans[0].query),
+                                      method, k, tau_a.data_ptr(), stream))
+        _lib.check(lib.hira_update_threshold(C.byref(tb), nk.data_ptr(), nk.data_ptr(), m,
+                                             b._state.data_ptr(), samples.data_ptr(), s,
+                                             C.byref(plans[1].query), method, k, tau_b.data_ptr(), stream))
+        a.note_unsynced(m)
+        b.note_unsynced(m)
+        assert torch.equal(tau_a, tau_b), c
+        assert torch.equal(a._state, b._state), c
+    a.sync_sizes()
+    b.sync_sizes()
+    assert a.size == b.size and a.num_keys == b.num_keys == n0 + calls * m
+    s0 = a.size[0]
+    assert torch.equal(a.perm[:, :s0], b.perm[:, :s0])
+    held = a.perm[:, :s0] >= 0
+    assert torch.equal(a.keys_rowmajor()[held], b.keys_rowmajor()[held])
+    assert torch.equal(a.values_buf[:, :s0][held], b.values_buf[:, :s0][held])
+    for l in (1, 2):
+        assert torch.equal(a.counts[l][:, : a.size[l]], b.counts[l][:, : a.size[l]])
+        assert torch.equal(a.radii[l][:, : a.size[l]], b.radii[l][:, : a.size[l]])
+    _check_tree(b, keys[:, :b.num_keys], keys[:, :b.num_keys])
+    # the thresholds themselves: the two rules on the same sample, in fp64
+    sc = np.einsum("hd,hsd->hs", q.float().cpu().numpy().astype(np.float64),
+                   samples.float().cpu().numpy().astype(np.float64)[ho.default_q2kv(h_q, t)])
+    want = sc.max(1) if method == 0 else np.sort(sc, 1)[:, ::-1][:, :k].mean(1)
+    np.testing.assert_allclose(tau_b.cpu().numpy(), want, rtol=2e-5, atol=1e-5)
