@@ -131,6 +131,10 @@ class HiraCacheLayer(CacheLayerMixin):
         if not self.is_initialized:
             self.lazy_initialization(key_states, value_states)
             self.indexer.build(key_states, value_states)
+            # what the first append and the first subtree rebuild of a process load on first use
+            # is loaded now, beside the prefill, not in the middle of the decode
+            if hasattr(self.indexer, "warm_up"):
+                self.indexer.warm_up()
             self._alloc_queue(max(1, min(int(self.update_every), 4096)))
             self.indexed_len = key_states.shape[-2]
             self._take_samples(key_states)

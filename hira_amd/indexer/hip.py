@@ -862,6 +862,57 @@ class HIPIndexer(BaseIndexer):
             self._tree_struct = None
         return self
 
+    _warmed: set = set()
+
+    @torch.no_grad()
+    def warm_up(self) -> None:
+        """The first append, window append and subtree rebuild of a process pay for code that is
+        loaded on first use (this library's kernels, torch's sort / gather / reduction kernels,
+        the allocator's first blocks): some 60 ms for the first append and 0.4-0.6 s for the first
+        rebuild, in the middle of a decode.  This runs them once on a throw-away index of this
+        one's kind (levels, fan-out, row widths, storage type, layout) with a few hundred keys,
+        so that a serving process pays at set-up; once per kind and process.  The index itself
+        is not touched."""
+        if self.keys_buf is None:
+            raise ValueError("Indexer is not built: call build() first.")
+        kind = (self.num_levels, self.branching_factor, self.dim, self.vdim, self.dtype,
+                self.layout_name, str(self.device), self.values_buf is not None)
+        if kind in HIPIndexer._warmed:
+            return
+        HIPIndexer._warmed.add(kind)
+        bf = self.branching_factor
+        n = 2 * bf ** min(self.num_levels - 1, 2) + 3
+        # the smallest window that update() builds as a subtree of its own and grafts in (its
+        # own rule, below), where that is small enough for a toy
+        big = 0
+        if self.num_levels >= 2 and (not self.tiled or bf % 16 == 0):
+            big = self.graft_min if self.graft_min is not None else \
+                max(256, bf ** max(self.num_levels - 2, 1) // 2)
+            big = big if big <= 1024 else 0
+        g = torch.Generator().manual_seed(7)
+        k = torch.randn((1, 2, n + 9 + big, self.dim), generator=g).to(self.dtype).to(self.device)
+        v = None
+        if self.values_buf is not None:
+            v = torch.randn((1, 2, n + 9 + big, self.vdim), generator=g).to(self.dtype).to(self.device)
+        toy = HIPIndexer(self.num_levels, self.max_iterations, bf, seed=self.seed,
+                         pack_rounds=self.pack_rounds, layout=self.layout_name,
+                         device=str(self.device), graft_min=self.graft_min)
+        toy.build(k[:, :, :n], None if v is None else v[:, :, :n])
+        if toy.layout_name != self.layout_name:
+            return  # (a layout that a toy of this size cannot take: nothing more to run)
+
+        def rows(x, a, b):
+            return None if x is None else x[:, :, a:b]
+
+        toy.update(k[:, :, n:n + 1], rows(v, n, n + 1))               # a key
+        if self.num_levels >= 2:
+            toy.update(k[:, :, n + 1:n + 9], rows(v, n + 1, n + 9), sync=False)  # a window
+            if big:
+                toy.update(k[:, :, n + 9:n + 9 + big], rows(v, n + 9, n + 9 + big))  # a grafted one
+        if self.num_levels >= 3 and not (self.tiled and bf % 16):
+            toy.rebuild_subtree(0)
+        torch.cuda.synchronize(self.device)
+
     @torch.no_grad()
     def rebuild_subtree(self, node: int) -> "HIPIndexer":
         """Re-cluster everything under node `node` of level 2 (its bf level-1 nodes and their

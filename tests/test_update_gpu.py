@@ -526,3 +526,38 @@ def test_append_and_thresholds_in_one_launch_equal_the_two_calls(dtype, d, m, s,
                    samples.float().cpu().numpy().astype(np.float64)[ho.default_q2kv(h_q, t)])
     want = sc.max(1) if method == 0 else np.sort(sc, 1)[:, ::-1][:, :k].mean(1)
     np.testing.assert_allclose(tau_b.cpu().numpy(), want, rtol=2e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype,d,bf,nl,layout", [
+    (torch.float32, 32, 8, 2, "auto"),
+    (torch.bfloat16, 128, 16, 3, "auto"),
+    (torch.bfloat16, 64, 16, 4, "q8"),
+    (torch.float32, 16, 5, 3, "auto"),
+])
+def test_warm_up_runs_the_first_use_paths_and_leaves_the_index_alone(dtype, d, bf, nl, layout, gpu_device):
+    """warm_up runs an append, a window, a grafted window and a subtree rebuild on a throw-away
+    index of the same kind; the index it was called on keeps every array, and appends to it
+    afterwards behave as without the call."""
+    from hira_amd.indexer.hip import HIPIndexer
+
+    t, n = 2, 700
+    rnd = bf16_round if dtype == torch.bfloat16 else (lambda x: x)
+    keys = rnd(clustered_keys(t, n + 40, d, seed=3, clusters=12))
+    K = torch.from_numpy(keys)[None].to(dtype).cuda()
+    a = HIPIndexer(nl, 1, bf, layout=layout).build(K[:, :, :n], K[:, :, :n])
+    b = HIPIndexer(nl, 1, bf, layout=layout).build(K[:, :, :n], K[:, :, :n])
+    before = [x.clone() for x in (a.keys_buf, a.values_buf, a.perm)]
+    HIPIndexer._warmed.clear()
+    a.warm_up()
+    assert len(HIPIndexer._warmed) == 1
+    a.warm_up()  # a second call does nothing
+    assert len(HIPIndexer._warmed) == 1
+    for x, y in zip(before, (a.keys_buf, a.values_buf, a.perm)):
+        assert torch.equal(x, y)
+    for i in (a, b):
+        i.update(K[:, :, n:n + 40], K[:, :, n:n + 40])
+    assert a.size == b.size and a.num_keys == b.num_keys == n + 40
+    assert torch.equal(a.perm[:, :a.size[0]], b.perm[:, :b.size[0]])
+    for l in range(1, nl):
+        assert torch.equal(a.radii[l][:, : a.size[l]], b.radii[l][:, : a.size[l]])
+    _check_tree(a, keys, keys)
