@@ -341,6 +341,26 @@ def streaming(a, w, index, plan, q_d, taus, out, dev):
         step.replay()
     torch.cuda.synchronize()
     res["graph_step"]["us_per_step_replay_only"] = round((time.perf_counter() - h0) * 1e6 / max(n2, 1), 2)
+    # the same with the thresholds taken from a key sample inside the step (512 keys a tree, mean
+    # of the 8 best): the append and the thresholds share a launch (hira_update_threshold)
+    index.sync_sizes()
+    rows = index.keys_rowmajor()
+    pick = torch.linspace(0, w.n - 1, 512, device=rows.device).long()
+    live = index.perm[:, : index.size[0]] >= 0
+    samples = torch.stack([rows[t][live[t]][pick] for t in range(index.num_trees)]).contiguous()
+    step2 = StreamingStep(plan.searcher, index, q_d.shape[1], plan.scaling, horizon=512, samples=samples,
+                          method="sample_mean_topk", k=8)
+    step2.step(sk2[:, :, 0], sv2[:, :, 0], q_d[0])
+    for _ in range(8):
+        step2.replay()
+    torch.cuda.synchronize()
+    h0 = time.perf_counter()
+    for _ in range(n2):
+        step2.replay()
+    torch.cuda.synchronize()
+    res["graph_step_sampled_thresholds"] = {
+        "samples_per_tree": 512, "rule": "mean of the 8 best",
+        "us_per_step_replay_only": round((time.perf_counter() - h0) * 1e6 / n2, 2)}
     log(f"[bench] streaming: {res}")
     return res
 
