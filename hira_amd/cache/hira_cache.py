@@ -134,7 +134,12 @@ class HiraCacheLayer(CacheLayerMixin):
             # what the first append and the first subtree rebuild of a process load on first use
             # is loaded now, beside the prefill, not in the middle of the decode
             if hasattr(self.indexer, "warm_up"):
-                self.indexer.warm_up()
+                try:
+                    self.indexer.warm_up()
+                except Exception as ex:  # (a courtesy, not a step of the prefill)
+                    import warnings
+
+                    warnings.warn(f"index warm-up skipped: {ex}")
             self._alloc_queue(max(1, min(int(self.update_every), 4096)))
             self.indexed_len = key_states.shape[-2]
             self._take_samples(key_states)
